@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X FP8 linear hot path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+    python bench.py --table          # every BASELINE shape -> gpurun_out/bench_table.json
+
+A "step" is one pass of the hot path over one batch of synthetic input already resident
+in HBM: dynamic activation quantisation (bf16 -> e4m3fn + f32 scales) followed by the
+scaled FP8 matmul (bf16 out), or the grouped matmul for the MoE workload.  Inputs rotate
+through enough copies to exceed twice the 256 MB Infinity Cache, so no step finds its
+operands cached.  Prints ONE JSON line with the whole-step throughput, the roofline of
+the dominant kernel (timed with events on the launch stream inside the timed region) and
+the CPU oracle timed on this host's cores on a bounded slice of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "FP8 GEMM TFLOPS & % of MI355X FP8 peak; decode-M HBM GB/s & % of peak"
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense FP8 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+CACHE_BUST_BYTES = 2 * 256 * 2 ** 20
+
+# name -> (kind, M, K, N, model label)
+WORKLOADS = {
+    # configs[1]: Llama-3.1-8B-shaped blockwise FP8 linears (default: the largest, gate_up at M=2048)
+    "llama8b_gate_up_m2048": ("block", 2048, 4096, 28672),
+    "llama8b_qkv_m2048": ("block", 2048, 4096, 6144),
+    "llama8b_down_m2048": ("block", 2048, 14336, 4096),
+    "llama8b_o_proj_m2048": ("block", 2048, 4096, 4096),
+    "llama8b_gate_up_m128": ("block", 128, 4096, 28672),
+    "llama8b_gate_up_m16": ("block", 16, 4096, 28672),
+    "llama8b_gate_up_m1": ("block", 1, 4096, 28672),
+    # configs[0]
+    "single_linear_m64": ("block", 64, 4096, 4096),
+    # configs[2]: DeepSeek-V3 attention projections
+    "dsv3_q_a_m4096": ("block", 4096, 7168, 1536),
+    "dsv3_q_b_m4096": ("block", 4096, 1536, 24576),
+    "dsv3_kv_a_m4096": ("block", 4096, 7168, 576),
+    "dsv3_kv_b_m4096": ("block", 4096, 512, 32768),
+    "dsv3_o_proj_m4096": ("block", 4096, 16384, 7168),
+    "dsv3_o_proj_m1024": ("block", 1024, 16384, 7168),
+    "dsv3_o_proj_m256": ("block", 256, 16384, 7168),
+    # configs[3]: Llama-3.1-70B decode, per-token x per-channel scales
+    "decode70b_qkv_m1": ("row", 1, 8192, 10240),
+    "decode70b_qkv_m8": ("row", 8, 8192, 10240),
+    "decode70b_gate_up_m1": ("row", 1, 8192, 57344),
+    "decode70b_gate_up_m8": ("row", 8, 8192, 57344),
+    "decode70b_down_m1": ("row", 1, 28672, 8192),
+    "decode70b_down_m8": ("row", 8, 28672, 8192),
+    # configs[4]: DeepSeek-V3 MoE grouped GEMM, 256 experts, 32768 routed rows
+    "moe_gate_up": ("grouped", 32768, 7168, 4096),
+    "moe_down": ("grouped", 32768, 2048, 7168),
+}
+DEFAULT = "llama8b_gate_up_m2048"
+
+
+def algorithmic(kind, M, K, N):
+    """(flops, HBM bytes) of one step's matmul, and bytes of the quantisation."""
+    flops = 2.0 * M * N * K
+    if kind == "row":
+        mm_bytes = N * K + 4 * N + M * K + 4 * M + 2 * M * N
+        q_bytes = 3 * M * K + 4 * M
+    else:
+        mm_bytes = N * K + 4 * math.ceil(N / 128) * (K // 128) + M * K + 4 * M * (K // 128) + 2 * M * N
+        q_bytes = 3 * M * K + 4 * M * (K // 128)
+    return flops, mm_bytes, q_bytes
+
+
+class Workload:
+    def __init__(self, name, dev):
+        import torch
+        import modular_amd as mx
+        from modular_amd import synth
+
+        self.name = name
+        self.kind, self.M, self.K, self.N = WORKLOADS[name]
+        self.dev = dev
+        self.mx = mx
+        kind, M, K, N = self.kind, self.M, self.K, self.N
+        self.cfg = mx.rowwise_fp8_config() if kind == "row" else mx.blockwise_fp8_config()
+        E = 256 if kind == "grouped" else 1
+        w_bytes = E * N * K
+        per_copy = w_bytes + 2 * M * K + 2 * M * N
+        self.copies = max(2, min(8, math.ceil(CACHE_BUST_BYTES / per_copy) + 1))
+        if kind == "grouped":
+            self.copies = 2 if w_bytes > 2 ** 32 else 3
+        self.x, self.w, self.ws = [], [], []
+        for c in range(self.copies):
+            self.x.append(synth.activations(M, K, seed=c, outlier_frac=0.0 if kind == "row" else 0.01, device=dev))
+            if kind == "row":
+                wq, ws = synth.quantize_weight_rowwise(synth.weights_f32(N, K, seed=100 + c, device=dev))
+            elif kind == "block":
+                wq, ws = synth.quantize_weight_block(synth.weights_f32(N, K, seed=100 + c, device=dev))
+            else:
+                wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device=dev)
+                ws = torch.empty((E, math.ceil(N / 128), K // 128), dtype=torch.float32, device=dev)
+                for e0 in range(0, E, 16):
+                    q16, s16 = synth.quantize_weight_block(
+                        synth.weights_f32(16 * N, K, seed=1000 * c + e0, device=dev).reshape(16, N, K))
+                    wq[e0:e0 + 16], ws[e0:e0 + 16] = q16, s16
+            self.w.append(wq)
+            self.ws.append(ws)
+        if kind == "grouped":
+            self.off, self.ids, self.counts, self.stats = synth.moe_routing(4096, 256, 8, seed=0, device=dev)
+            assert int(self.counts.sum()) == M
+        torch.cuda.synchronize()
+
+    def step(self, i, ev=None):
+        """quantise + matmul on copy i; ev = (start, end) events recorded around the matmul."""
+        mx, cfg = self.mx, self.cfg
+        import torch
+        c = i % self.copies
+        q, sa = mx.quantize_dynamic_scaled_float8(self.x[c], cfg.input_scale, cfg.weight_scale,
+                                                  scales_type=torch.float32)
+        if ev:
+            ev[0].record()
+        if self.kind == "grouped":
+            out = mx.grouped_dynamic_scaled_fp8_matmul(q, self.w[c], sa, self.ws[c], self.off, self.ids, self.stats,
+                                                       cfg.input_scale, cfg.weight_scale)
+        else:
+            out = mx.dynamic_scaled_matmul(q, self.w[c], sa, self.ws[c], cfg.input_scale, cfg.weight_scale)
+        if ev:
+            ev[1].record()
+        return out
+
+
+def run_gpu(name, steps, warmup):
+    import torch
+
+    dev = torch.device("cuda:0")
+    wl = Workload(name, dev)
+    for i in range(warmup):
+        wl.step(i)
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        wl.step(warmup + i, events[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_step = (t1 - t0) * 1e3 / steps
+    mm_ms = sorted(e[0].elapsed_time(e[1]) for e in events)
+    mm_avg = sum(mm_ms) / len(mm_ms)
+    return wl, ms_step, mm_avg, mm_ms[len(mm_ms) // 2], mm_ms[0]
+
+
+def cpu_baseline(wl, budget_s=15.0):
+    """The oracle (a port of the reference's host loops) on this host's cores, on a bounded
+    slice of the same workload; throughput in the metric's unit."""
+    import numpy as np
+    import oracle
+
+    threads = oracle.default_threads()
+    kind, M, K, N = wl.kind, wl.M, wl.K, wl.N
+    x = wl.x[0].cpu()
+    w = wl.w[0] if kind != "grouped" else wl.w[0][0]
+    ws = wl.ws[0] if kind != "grouped" else wl.ws[0][0]
+    wb = w.cpu().view(__import__("torch").uint8).numpy()
+    wsn = ws.cpu().numpy()
+    G = K if kind == "row" else 128
+
+    def run(rows):
+        xb = x[:rows].contiguous().view(__import__("torch").int16).numpy().view(np.uint16)
+        t0 = time.perf_counter()
+        q, sa = oracle.quantize_dynamic_scaled_fp8(xb, G, threads=threads)
+        if kind == "row":
+            oracle.matmul_rowwise(q, wb, sa, wsn, c_dtype=oracle.BF16, threads=threads)
+        else:
+            oracle.matmul_blockwise(q, wb, sa, wsn, c_dtype=oracle.BF16, mode=1, threads=threads)
+        return time.perf_counter() - t0
+
+    rows = min(M, max(1, threads))
+    t = run(rows)
+    per_row = t / rows
+    rows2 = int(min(M, max(rows, budget_s / max(per_row, 1e-9))))
+    if rows2 > rows:
+        t, rows = run(rows2), rows2
+    flops = 2.0 * rows * N * K
+    if kind == "row":
+        value, unit = (N * K + rows * K + 2 * rows * N) / t / 1e9, "GB/s"
+    else:
+        value, unit = flops / t / 1e12, "TFLOP/s"
+    sample = (f"oracle quantise + matmul (per-128-slab order) on rows 0..{rows - 1} of M={M}"
+              + (" against expert 0's weights" if kind == "grouped" else "")
+              + f", N={N}, K={K}: {t:.2f} s")
+    return {"value": value, "unit": unit, "cores": threads, "kind": "port", "sample": sample}
+
+
+def result_line(name, steps, warmup, with_cpu=True):
+    wl, ms_step, mm_avg, mm_med, mm_min = run_gpu(name, steps, warmup)
+    kind, M, K, N = wl.kind, wl.M, wl.K, wl.N
+    flops, mm_bytes, q_bytes = algorithmic(kind, M, K, N)
+    if kind == "grouped":
+        mm_bytes += 255 * N * K  # every expert's weights are streamed once
+    hbm_bound = kind == "row" or M <= 16
+    if hbm_bound:
+        value, unit = (mm_bytes + q_bytes) / (ms_step * 1e-3) / 1e9, "GB/s"
+        roof = {"bound": "hbm", "achieved": mm_bytes / (mm_avg * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s"}
+    else:
+        value, unit = flops / (ms_step * 1e-3) / 1e12, "TFLOP/s"
+        roof = {"bound": "mfma", "achieved": flops / (mm_avg * 1e-3) / 1e12, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["kernel"] = {"grouped": "gemm_tiled_kernel<grouped>", "row": "gemm_skinny_kernel"}.get(
+        kind, "gemm_skinny_kernel" if M <= 64 else "gemm_tiled_kernel")
+    roof["kernel_ms_avg"], roof["kernel_ms_median"], roof["kernel_ms_min"] = mm_avg, mm_med, mm_min
+    out = {
+        "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3fn (f32 accumulate, bf16 out)", "data": "synthetic",
+        "config": {"workload": name, "M": M, "K": K, "N": N,
+                   "scaling": "per-token x per-channel" if kind == "row" else "1x128 activations, 128x128 weights",
+                   "step": "dynamic quantise + " + ("grouped " if kind == "grouped" else "") + "scaled matmul",
+                   "input_copies": wl.copies},
+        "roofline": roof,
+    }
+    if with_cpu:
+        out["cpu_baseline"] = cpu_baseline(wl)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--table", action="store_true", help="run every workload, write gpurun_out/bench_table.json")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no collective); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP kernels are the only compute path", file=sys.stderr)
+        sys.exit(1)
+    if args.table:
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        rows = []
+        for name in WORKLOADS:
+            print(f"[bench] {name}", file=sys.stderr, flush=True)
+            r = result_line(name, args.steps, args.warmup, with_cpu=False)
+            rows.append(r)
+            print(json.dumps({"workload": name, "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+                              "kernel_ms": r["roofline"]["kernel_ms_avg"], "frac": r["roofline"]["frac"]}),
+                  file=sys.stderr, flush=True)
+            with open(os.path.join(ROOT, "gpurun_out", "bench_table.json"), "w") as f:
+                json.dump(rows, f, indent=1)
+            torch.cuda.empty_cache()
+        return
+    print(json.dumps(result_line(args.workload, args.steps, args.warmup, with_cpu=not args.no_cpu)))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,172 @@
+/*
+ * maxfp8.h -- C ABI of the MI355X (gfx950) FP8 linear hot path.
+ *
+ * Three operators, named after the MAX custom ops they stand in for:
+ *
+ *   mo.quantize_dynamic_scaled_float8      -> maxfp8_quantize_dynamic_scaled_fp8
+ *   mo.matmul_dynamic_scaled_fp8           -> maxfp8_matmul_dynamic_scaled_fp8
+ *   mo.grouped.matmul.dynamic.scaled.fp8   -> maxfp8_grouped_matmul_dynamic_scaled_fp8
+ *
+ * Conventions (the same as the reference's destination-passing custom-op ABI,
+ * max/kernels/src/graph_compiler/extensibility/decorators.mojo:46-131):
+ *   - every pointer is a DEVICE pointer owned by the caller; outputs are
+ *     pre-allocated; the library never allocates or frees caller memory;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *     null stream) and the call returns without synchronising;
+ *   - zero-sized work is a silent no-op returning MAXFP8_OK;
+ *   - the return value is MAXFP8_OK (0) or a negative maxfp8_status; the text of
+ *     the last error on the calling thread is returned by maxfp8_last_error().
+ */
+#ifndef MAXFP8_H
+#define MAXFP8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum maxfp8_status {
+  MAXFP8_OK = 0,
+  MAXFP8_ERR_DTYPE = -1,       /* unsupported element / scale dtype            */
+  MAXFP8_ERR_SHAPE = -2,       /* inconsistent sizes, strides or group size    */
+  MAXFP8_ERR_ALIGN = -3,       /* pointer or stride alignment not supported    */
+  MAXFP8_ERR_GRANULARITY = -4, /* unsupported scaling granularity combination  */
+  MAXFP8_ERR_LAUNCH = -5,      /* HIP reported an error at launch              */
+  MAXFP8_ERR_NULL = -6,        /* required pointer was NULL                    */
+  MAXFP8_ERR_WORKSPACE = -7    /* workspace missing or too small               */
+} maxfp8_status;
+
+typedef enum maxfp8_dtype {
+  MAXFP8_BF16 = 0,
+  MAXFP8_F16 = 1,
+  MAXFP8_F32 = 2,
+  MAXFP8_E4M3FN = 3
+} maxfp8_dtype;
+
+/* Scaling granularity names, verbatim from
+ * max/python/max/nn/quant_config.py:26-46 (ScaleGranularity). */
+typedef enum maxfp8_granularity {
+  MAXFP8_GRAN_TENSOR = 0,
+  MAXFP8_GRAN_ROWWISE = 1,
+  MAXFP8_GRAN_COLWISE = 2,
+  MAXFP8_GRAN_BLOCK = 3
+} maxfp8_granularity;
+
+/* Kernel selection for the dense matmul.  AUTO picks by shape. */
+typedef enum maxfp8_algo {
+  MAXFP8_ALGO_AUTO = 0,
+  MAXFP8_ALGO_NAIVE = 1,  /* one thread per output, reference summation order */
+  MAXFP8_ALGO_TILED = 2,  /* LDS-staged MFMA tiles                            */
+  MAXFP8_ALGO_SKINNY = 3  /* weight-streaming kernel for M <= 16              */
+} maxfp8_algo;
+
+const char* maxfp8_last_error(void);
+const char* maxfp8_version(void);
+
+/*
+ * Dynamic activation quantisation.
+ * Replaces QuantizeDynamicScaledFloat8.execute
+ *   (max/kernels/src/graph_compiler/builtin_kernels/quantization.mojo:1363-1406)
+ * -> quantize_dynamic_scaled_fp8 (max/kernels/src/linalg/fp8_quantization.mojo:369-463).
+ *
+ *   in          [M, K] row-major with row stride `in_row_stride` elements,
+ *               dtype `in_dtype` (MAXFP8_BF16, MAXFP8_F16 or MAXFP8_F32)
+ *   out_fp8     [M, K] e4m3fn bytes, row stride `out_row_stride` bytes
+ *   out_scales  [K / group_size, scales_ld] of `scales_dtype` (MAXFP8_F32 or
+ *               MAXFP8_BF16); element (g, r) = scale of row r, group g
+ *               (TRANSPOSED, fp8_quantization.mojo:564-565); columns
+ *               M..scales_ld-1 are never written
+ *   group_size  128 for blockwise, K for per-token; must divide K and be a
+ *               multiple of 4
+ *   scale_ub    upper clamp on the group amax (1200.0 in every reference call,
+ *               max/python/max/nn/kernels.py:6880)
+ */
+int maxfp8_quantize_dynamic_scaled_fp8(
+    void* out_fp8, void* out_scales, const void* in,
+    int64_t M, int64_t K, int64_t in_row_stride, int64_t out_row_stride,
+    int64_t group_size, int64_t scales_ld,
+    int in_dtype, int scales_dtype, float scale_ub, void* stream);
+
+/*
+ * Scaled FP8 matmul, C = A . B^T with B stored [N, K] ("transpose_b").
+ * Replaces MatmulDynamicScaledFloat8.execute
+ *   (max/kernels/src/graph_compiler/builtin_kernels/linalg.mojo:1677-1720)
+ * -> matmul_dynamic_scaled_fp8 (max/kernels/src/linalg/fp8_quantization.mojo:963-1334).
+ *
+ *   a  [M, K] e4m3fn, row stride lda bytes     b  [N, K] e4m3fn, row stride ldb bytes
+ *   c  [M, N] of c_dtype (MAXFP8_BF16 or MAXFP8_F32), row stride ldc elements
+ *
+ *   input/weight granularity BLOCK/BLOCK with (gm, gn, gk) = (1, 128, 128):
+ *       a_scales [ceil(K/128), a_scales_ld] f32, element (k/128, m)
+ *       b_scales [ceil(N/128), b_scales_ld] f32, element (n/128, k/128)
+ *       C[m,n] = sum_k A[m,k] B[n,k] a_scales[k/128,m] b_scales[n/128,k/128]
+ *   input COLWISE, weight ROWWISE (per-token / per-output-channel):
+ *       a_scales [1, M], b_scales [N, 1] (b_scales_ld = element stride between
+ *       rows of b_scales, normally 1)
+ *       C[m,n] = (sum_k A[m,k] B[n,k]) * a_scales[m] * b_scales[n]
+ *   input TENSOR, weight TENSOR: a_scales[0], b_scales[0].
+ *
+ *   scales_dtype MAXFP8_F32 (block requires it) or MAXFP8_BF16 (rowwise/tensor).
+ *   algo        a maxfp8_algo value.
+ *   workspace   optional device scratch for split-K (may be NULL: then kernels
+ *               that need none are used).
+ */
+int maxfp8_matmul_dynamic_scaled_fp8(
+    void* c, const void* a, const void* b,
+    const void* a_scales, const void* b_scales,
+    int64_t M, int64_t N, int64_t K,
+    int64_t lda, int64_t ldb, int64_t ldc,
+    int input_granularity, int weight_granularity,
+    int64_t gm, int64_t gn, int64_t gk,
+    int64_t a_scales_ld, int64_t b_scales_ld,
+    int c_dtype, int scales_dtype, int algo,
+    void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of workspace that lets AUTO use every kernel for this shape. */
+size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Grouped (MoE) blockwise-scaled FP8 matmul over token rows sorted by expert.
+ * Replaces Struct_grouped_matmul_dynamic_scaled_fp8.execute
+ *   (max/kernels/src/graph_compiler/builtin_kernels/linalg.mojo:702-757)
+ * -> grouped_matmul_dynamic_scaled_fp8
+ *   (max/kernels/src/linalg/grouped_matmul_sm100_blockwise_fp8.mojo:2938-3105).
+ *
+ *   a  [T, K] e4m3fn (row stride K)            b  [E, N, K] e4m3fn (contiguous)
+ *   c  [T, N] c_dtype (row stride N)
+ *   a_scales [ceil(K/128), a_scales_ld] f32    b_scales [E, ceil(N/128), ceil(K/128)] f32
+ *   expert_start_indices  uint32[num_active_experts + 1], device
+ *   expert_ids            int32[num_active_experts], device; -1 => the slot's
+ *                         rows of C are written with zeros
+ *   max_num_tokens_per_expert, num_active_experts: host scalars; either == 0
+ *                         => no-op.  max_num_tokens_per_expert is an upper bound
+ *                         used only to bound the launch.
+ */
+int maxfp8_grouped_matmul_dynamic_scaled_fp8(
+    void* c, const void* a, const void* b,
+    const void* a_scales, const void* b_scales,
+    const uint32_t* expert_start_indices, const int32_t* expert_ids,
+    int64_t T, int64_t N, int64_t K, int64_t num_experts,
+    int64_t max_num_tokens_per_expert, int64_t num_active_experts,
+    int64_t a_scales_ld, int c_dtype, int scales_dtype, int algo, void* stream);
+
+/*
+ * Elementwise f32 -> e4m3fn (clamp to +-448, round to nearest even), the cast
+ * inside fp8_quantize (max/kernels/src/internal_utils/fp8_utils.mojo:96-143).
+ * Exposed so the hardware convert can be checked exhaustively.
+ */
+int maxfp8_cast_f32_to_e4m3fn(void* out_fp8, const float* in, int64_t n, void* stream);
+
+/* Elementwise e4m3fn -> f32 (mojo/stdlib/std/builtin/simd.mojo:3690-3749). */
+int maxfp8_cast_e4m3fn_to_f32(float* out, const void* in_fp8, int64_t n, void* stream);
+
+/* Plain device copy kernel of n bytes (n % 16 == 0); the calibration unit for
+ * hardware byte counters. */
+int maxfp8_copy_bytes(void* dst, const void* src, int64_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAXFP8_H */

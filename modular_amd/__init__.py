@@ -1,0 +1,19 @@
+"""MI355X-native FP8 linear path: dynamic activation quantisation, scaled FP8
+matmul and its grouped (MoE) variant, behind the op names of the reference.
+
+All compute runs in hand-written gfx950 HIP kernels (modular_amd/csrc) loaded
+through the C ABI of include/maxfp8.h; there is no CPU or PyTorch fallback.
+"""
+from .quant_config import (InputScaleSpec, QuantConfig, QuantFormat, ScaleGranularity, ScaleOrigin,
+                           WeightScaleSpec, blockwise_fp8_config, rowwise_fp8_config)
+from .kernels import (dynamic_scaled_matmul, grouped_dynamic_scaled_fp8_matmul,
+                      quantize_dynamic_scaled_float8)
+from .quant_ops import matmul_float8, quantized_matmul
+from .linear import Linear
+
+__all__ = [
+    "InputScaleSpec", "QuantConfig", "QuantFormat", "ScaleGranularity", "ScaleOrigin", "WeightScaleSpec",
+    "blockwise_fp8_config", "rowwise_fp8_config", "dynamic_scaled_matmul",
+    "grouped_dynamic_scaled_fp8_matmul", "quantize_dynamic_scaled_float8", "matmul_float8",
+    "quantized_matmul", "Linear",
+]

@@ -1,0 +1,226 @@
+// C ABI of the library (include/maxfp8.h): argument checks, kernel selection, error text.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+#include "gemm_args.h"
+
+namespace maxfp8 {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int launch_status(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+  return MAXFP8_OK;
+}
+
+// kernels (defined in the other translation units)
+int quantize_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, int,
+                      float, hipStream_t);
+int cast_f32_to_e4m3fn_dispatch(void*, const float*, int64_t, hipStream_t);
+int cast_e4m3fn_to_f32_dispatch(float*, const void*, int64_t, hipStream_t);
+int copy_bytes_dispatch(void*, const void*, int64_t, hipStream_t);
+int naive_blockwise_dispatch(void*, const void*, const void*, const void*, const void*, int64_t, int64_t, int64_t,
+                             int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int,
+                             hipStream_t);
+int naive_rowwise_dispatch(void*, const void*, const void*, const void*, const void*, int64_t, int64_t, int64_t,
+                           int64_t, int64_t, int64_t, int64_t, int64_t, int, int, hipStream_t);
+int naive_grouped_dispatch(void*, const void*, const void*, const void*, const void*, const uint32_t*,
+                           const int32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int, hipStream_t);
+int gemm_tiled_dispatch(const GemmArgs&, bool, hipStream_t);
+int gemm_grouped_dispatch(const GemmArgs&, int64_t, hipStream_t);
+int gemm_skinny_dispatch(const GemmArgs&, bool, hipStream_t);
+int gemm_skinny_max_m();
+
+static bool is_aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+}  // namespace maxfp8
+
+using namespace maxfp8;
+
+extern "C" {
+
+const char* maxfp8_last_error(void) { return g_error; }
+const char* maxfp8_version(void) { return "maxfp8 0.1 (gfx950)"; }
+
+int maxfp8_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, int64_t M, int64_t K,
+                                       int64_t in_row_stride, int64_t out_row_stride, int64_t group_size,
+                                       int64_t scales_ld, int in_dtype, int scales_dtype, float scale_ub,
+                                       void* stream) {
+  if (in_dtype != MAXFP8_BF16 && in_dtype != MAXFP8_F16 && in_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize: input dtype %d is not bf16, f16 or f32", in_dtype);
+  if (scales_dtype != MAXFP8_F32 && scales_dtype != MAXFP8_BF16)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize: scales dtype should be bfloat16 or float32 (got %d)", scales_dtype);
+  if (M < 0 || K < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: negative size M=%lld K=%lld", (long long)M, (long long)K);
+  if (M == 0 || K == 0) return MAXFP8_OK;  // fp8_quantization.mojo:428-429
+  if (group_size == -1) group_size = K;
+  if (group_size <= 0 || K % group_size != 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: group size %lld must divide K = %lld", (long long)group_size, (long long)K);
+  if (group_size % 4 != 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: group size must be multiple of simd size (4), got %lld", (long long)group_size);
+  if (in_row_stride < K || out_row_stride < K || scales_ld < M)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: strides (in %lld, out %lld, scales %lld) smaller than the extents",
+                (long long)in_row_stride, (long long)out_row_stride, (long long)scales_ld);
+  if (!out_fp8 || !out_scales || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize: null pointer");
+  return quantize_dispatch(out_fp8, out_scales, in, M, K, in_row_stride, out_row_stride, group_size, scales_ld,
+                           in_dtype, scales_dtype, scale_ub, (hipStream_t)stream);
+}
+
+size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  (void)M; (void)N; (void)K;
+  return 0;  // no kernel of this version needs scratch memory
+}
+
+int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
+                                     const void* b_scales, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                     int64_t ldb, int64_t ldc, int input_granularity, int weight_granularity,
+                                     int64_t gm, int64_t gn, int64_t gk, int64_t a_scales_ld, int64_t b_scales_ld,
+                                     int c_dtype, int scales_dtype, int algo, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+  (void)workspace; (void)workspace_bytes;
+  if (c_dtype != MAXFP8_BF16 && c_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "matmul: output dtype %d is not bf16 or f32", c_dtype);
+  if (M < 0 || N < 0 || K < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: negative size");
+  if (M == 0 || N == 0) return MAXFP8_OK;  // fp8_quantization.mojo:1103-1104
+  if (M >= ((int64_t)1 << 31) || N >= ((int64_t)1 << 31) || K >= ((int64_t)1 << 31))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: sizes must fit 31 bits");
+  if (lda < K || ldb < K || ldc < N) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: leading dimension smaller than the row length");
+  if (!c || !a || !b || !a_scales || !b_scales) MAXFP8_FAIL(MAXFP8_ERR_NULL, "matmul: null pointer");
+
+  const bool block = input_granularity == MAXFP8_GRAN_BLOCK && weight_granularity == MAXFP8_GRAN_BLOCK;
+  const bool row = input_granularity == MAXFP8_GRAN_COLWISE && weight_granularity == MAXFP8_GRAN_ROWWISE;
+  const bool tensor = input_granularity == MAXFP8_GRAN_TENSOR && weight_granularity == MAXFP8_GRAN_TENSOR;
+  if (!block && !row && !tensor) MAXFP8_FAIL(MAXFP8_ERR_GRANULARITY, "unsupported FP8 scaling granularity");
+  hipStream_t st = (hipStream_t)stream;
+
+  if (block) {
+    if (scales_dtype != MAXFP8_F32) MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "a_scales and b_scales dtypes must be float32");
+    if (gm <= 0 || gn <= 0 || gk <= 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: block granularities must be positive");
+    if (a_scales_ld < ceil_div(M, gm) || b_scales_ld < ceil_div(K, gk))
+      MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: scale leading dimensions too small");
+  } else if (scales_dtype != MAXFP8_F32 && scales_dtype != MAXFP8_BF16) {
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "matmul: scales dtype %d is not f32 or bf16", scales_dtype);
+  }
+
+  // Fast kernels: f32 scales, 16-byte aligned rows, K a multiple of 16, and for
+  // block scaling the (1, 128, 128) granularity.
+  const bool fast_layout = is_aligned(a, 16) && is_aligned(b, 16) && lda % 16 == 0 && ldb % 16 == 0 && K % 16 == 0 &&
+                           K > 0 && scales_dtype == MAXFP8_F32 && (!block || (gm == 1 && gn == 128 && gk == 128));
+  if (algo == MAXFP8_ALGO_AUTO) {
+    if (!fast_layout) algo = MAXFP8_ALGO_NAIVE;
+    else if (M <= gemm_skinny_max_m()) algo = MAXFP8_ALGO_SKINNY;
+    else algo = MAXFP8_ALGO_TILED;
+  }
+  if (algo == MAXFP8_ALGO_NAIVE) {
+    if (block)
+      return naive_blockwise_dispatch(c, a, b, a_scales, b_scales, M, N, K, lda, ldb, ldc, gm, gn, gk, a_scales_ld,
+                                      b_scales_ld, c_dtype, st);
+    return naive_rowwise_dispatch(c, a, b, a_scales, b_scales, M, N, K, lda, ldb, ldc, tensor ? 0 : 1,
+                                  tensor ? 0 : b_scales_ld, c_dtype, scales_dtype, st);
+  }
+  if (algo != MAXFP8_ALGO_TILED && algo != MAXFP8_ALGO_SKINNY) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: unknown algo %d", algo);
+  if (!fast_layout)
+    MAXFP8_FAIL(MAXFP8_ERR_ALIGN,
+                "matmul: the MFMA kernels need 16-byte aligned rows, K %% 16 == 0, f32 scales and (1,128,128) blocks");
+
+  GemmArgs p;
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t*)a;
+  p.b = (const uint8_t*)b;
+  p.c = c;
+  p.a_scales = (const float*)a_scales;
+  p.b_scales = (const float*)b_scales;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.a_scales_ld = a_scales_ld;
+  p.b_scales_ld = b_scales_ld;
+  p.a_scale_stride = tensor ? 0 : 1;
+  p.b_scale_stride = tensor ? 0 : b_scales_ld;
+  p.c_dtype = c_dtype;
+  p.c_vec_ok = (ldc % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
+  if (algo == MAXFP8_ALGO_SKINNY) return gemm_skinny_dispatch(p, block, st);
+  return gemm_tiled_dispatch(p, block, st);
+}
+
+int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
+                                             const void* b_scales, const uint32_t* expert_start_indices,
+                                             const int32_t* expert_ids, int64_t T, int64_t N, int64_t K,
+                                             int64_t num_experts, int64_t max_num_tokens_per_expert,
+                                             int64_t num_active_experts, int64_t a_scales_ld, int c_dtype,
+                                             int scales_dtype, int algo, void* stream) {
+  if (c_dtype != MAXFP8_BF16 && c_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "grouped matmul: output dtype %d is not bf16 or f32", c_dtype);
+  if (scales_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "grouped matmul: scales must be float32");
+  if (T < 0 || N < 0 || K < 0 || num_experts < 0 || max_num_tokens_per_expert < 0 || num_active_experts < 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: negative size");
+  // grouped_matmul_sm100_blockwise_fp8.mojo:3016-3017
+  if (max_num_tokens_per_expert == 0 || num_active_experts == 0 || T == 0 || N == 0) return MAXFP8_OK;
+  if (num_active_experts > num_experts)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: %lld active slots but expert_ids holds %lld", (long long)num_active_experts,
+                (long long)num_experts);
+  if (T >= ((int64_t)1 << 31) || N >= ((int64_t)1 << 31) || K >= ((int64_t)1 << 31))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: sizes must fit 31 bits");
+  if (a_scales_ld < T) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: a_scales leading dimension %lld < T = %lld",
+                                   (long long)a_scales_ld, (long long)T);
+  if (!c || !a || !b || !a_scales || !b_scales || !expert_start_indices || !expert_ids)
+    MAXFP8_FAIL(MAXFP8_ERR_NULL, "grouped matmul: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const bool fast_layout = is_aligned(a, 16) && is_aligned(b, 16) && K % 16 == 0 && K > 0;
+  if (algo == MAXFP8_ALGO_AUTO) algo = fast_layout ? MAXFP8_ALGO_TILED : MAXFP8_ALGO_NAIVE;
+  if (algo == MAXFP8_ALGO_NAIVE)
+    return naive_grouped_dispatch(c, a, b, a_scales, b_scales, expert_start_indices, expert_ids, N, K,
+                                  max_num_tokens_per_expert, num_active_experts, a_scales_ld, c_dtype, st);
+  if (algo != MAXFP8_ALGO_TILED) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: unknown algo %d", algo);
+  if (!fast_layout) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "grouped matmul: the MFMA kernel needs 16-byte aligned rows and K %% 16 == 0");
+
+  GemmArgs p;
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t*)a;
+  p.b = (const uint8_t*)b;
+  p.c = c;
+  p.a_scales = (const float*)a_scales;
+  p.b_scales = (const float*)b_scales;
+  p.M = (int)T; p.N = (int)N; p.K = (int)K;
+  p.lda = K; p.ldb = K; p.ldc = N;
+  p.a_scales_ld = a_scales_ld;
+  p.b_scales_ld = ceil_div(K, 128);
+  p.c_dtype = c_dtype;
+  p.c_vec_ok = (N % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
+  p.offsets = expert_start_indices;
+  p.expert_ids = expert_ids;
+  p.num_active = (int)num_active_experts;
+  p.b_expert_stride = N * K;
+  p.bs_expert_stride = ceil_div(N, 128) * ceil_div(K, 128);
+  return gemm_grouped_dispatch(p, T, st);
+}
+
+int maxfp8_cast_f32_to_e4m3fn(void* out_fp8, const float* in, int64_t n, void* stream) {
+  if (n <= 0) return MAXFP8_OK;
+  if (!out_fp8 || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "cast: null pointer");
+  return cast_f32_to_e4m3fn_dispatch(out_fp8, in, n, (hipStream_t)stream);
+}
+
+int maxfp8_cast_e4m3fn_to_f32(float* out, const void* in_fp8, int64_t n, void* stream) {
+  if (n <= 0) return MAXFP8_OK;
+  if (!out || !in_fp8) MAXFP8_FAIL(MAXFP8_ERR_NULL, "cast: null pointer");
+  return cast_e4m3fn_to_f32_dispatch(out, in_fp8, n, (hipStream_t)stream);
+}
+
+int maxfp8_copy_bytes(void* dst, const void* src, int64_t n, void* stream) {
+  if (n <= 0) return MAXFP8_OK;
+  if (!dst || !src) MAXFP8_FAIL(MAXFP8_ERR_NULL, "copy: null pointer");
+  if (n % 16 != 0 || !is_aligned(dst, 16) || !is_aligned(src, 16))
+    MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "copy: size and pointers must be multiples of 16 bytes");
+  return copy_bytes_dispatch(dst, src, n, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,30 @@
+// Argument block shared by the tiled, skinny and grouped matmul kernels.
+#pragma once
+#include <stdint.h>
+
+namespace maxfp8 {
+
+struct GemmArgs {
+  const uint8_t* a;        // [M, K] e4m3fn, row stride lda bytes
+  const uint8_t* b;        // [N, K] e4m3fn (per expert when grouped), row stride ldb bytes
+  void* c;                 // [M, N] bf16 or f32, row stride ldc elements
+  const float* a_scales;   // block: [ceil(K/128), a_scales_ld]; row/tensor: element m * a_scale_stride
+  const float* b_scales;   // block: [ceil(N/128), b_scales_ld]; row/tensor: element n * b_scale_stride
+  int M, N, K;
+  int64_t lda, ldb, ldc;
+  int64_t a_scales_ld, b_scales_ld;
+  int64_t a_scale_stride, b_scale_stride;
+  int c_dtype;
+  int c_vec_ok;            // C base and ldc allow 4-element vector stores
+  // grouped only
+  const uint32_t* offsets;
+  const int32_t* expert_ids;
+  int num_active;
+  int64_t b_expert_stride;   // bytes between experts in b
+  int64_t bs_expert_stride;  // elements between experts in b_scales
+  // split-K / skinny only
+  float* workspace;
+  int splits;
+};
+
+}  // namespace maxfp8

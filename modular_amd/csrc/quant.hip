@@ -1,0 +1,271 @@
+// Dynamic activation quantisation for gfx950: bf16/f16/f32 [M, K] -> e4m3fn [M, K]
+// plus one scale per (row, group), stored transposed as scales[group, row].
+//
+// Arithmetic (max/kernels/src/linalg/fp8_quantization.mojo:509-583,
+// max/kernels/src/internal_utils/fp8_utils.mojo:24-143):
+//   amax  = max |x| over the group (f32)
+//   scale = min(amax, scale_ub) / 448          (correctly rounded division)
+//   recip = scale == 0 ? 0 : 1 / scale         (0 when that is inf or nan)
+//   q     = e4m3fn(clamp(x * recip, -448, 448)) (round to nearest even)
+//
+// Kernels:
+//   quant_g128_bf16   group 128, bf16 in, f32 scales.  One pass: 16 lanes own one
+//                     group (16-byte loads), amax by DPP inside the 16-lane row,
+//                     8-byte packed fp8 stores.  A block covers 16 rows x (4*U)
+//                     groups so the transposed scale stores of one group are 64
+//                     contiguous bytes.
+//   quant_row_bf16    per-token (group == K), bf16 in, f32 scales.  One block per
+//                     row, the row is kept in registers between the amax and the
+//                     convert pass.
+//   quant_generic     every other dtype / group size / alignment: one block per
+//                     (row, group), two passes over the group.
+#include "common.h"
+
+namespace maxfp8 {
+
+// ---------------------------------------------------------------------------
+template <int U>
+__global__ __launch_bounds__(256) void quant_g128_bf16_kernel(
+    uint8_t* __restrict__ out, float* __restrict__ scales, const uint16_t* __restrict__ in,
+    int M, int ngroups, int nxb, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
+    float scale_ub) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int seg = lane >> 4, sl = lane & 15;
+  const int rb = blockIdx.x / nxb, xb = blockIdx.x - rb * nxb;
+  const int row = rb * 16 + wave * 4 + seg;
+  // Each wave owns 4 rows (one per 16-lane segment) and the block's U consecutive groups.
+  const int gbase = xb * U;
+  const bool row_ok = row < M;
+
+  uint4 v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int g = gbase + u;
+    if (row_ok && g < ngroups)
+      v[u] = *reinterpret_cast<const uint4*>(in + (int64_t)row * in_stride + (int64_t)g * 128 + sl * 8);
+    else
+      v[u] = make_uint4(0, 0, 0, 0);
+  }
+
+  float my_scale = 0.0f;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(f[i]));
+    amax = row16_max(amax);
+    float scale, recip;
+    dynamic_scale_f32(amax, scale_ub, scale, recip);
+    if (sl == u) my_scale = scale;
+    int lo = 0, hi = 0;
+    lo = cvt_pk_e4m3fn(clamp448(f[0] * recip), clamp448(f[1] * recip), lo, false);
+    lo = cvt_pk_e4m3fn(clamp448(f[2] * recip), clamp448(f[3] * recip), lo, true);
+    hi = cvt_pk_e4m3fn(clamp448(f[4] * recip), clamp448(f[5] * recip), hi, false);
+    hi = cvt_pk_e4m3fn(clamp448(f[6] * recip), clamp448(f[7] * recip), hi, true);
+    const int g = gbase + u;
+    if (row_ok && g < ngroups)
+      *reinterpret_cast<uint2*>(out + (int64_t)row * out_stride + (int64_t)g * 128 + sl * 8) =
+          make_uint2((uint32_t)lo, (uint32_t)hi);
+  }
+  if (row_ok && sl < U && gbase + sl < ngroups) scales[(int64_t)(gbase + sl) * scales_ld + row] = my_scale;
+}
+
+// ---------------------------------------------------------------------------
+// One block (256 threads) per row, group == K.  NV 16-byte vectors per thread are
+// held in registers; K <= 256 * 8 * NV.
+template <int NV>
+__global__ __launch_bounds__(256) void quant_row_bf16_kernel(
+    uint8_t* __restrict__ out, float* __restrict__ scales, const uint16_t* __restrict__ in,
+    int K, int64_t in_stride, int64_t out_stride, float scale_ub) {
+  __shared__ float red[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const uint16_t* src = in + (int64_t)row * in_stride;
+  const int nvec = K >> 3;
+  uint4 v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * 256;
+    v[i] = idx < nvec ? reinterpret_cast<const uint4*>(src)[idx] : make_uint4(0, 0, 0, 0);
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      amax = fmaxf(amax, fabsf(__uint_as_float(w[j] << 16)));
+      amax = fmaxf(amax, fabsf(__uint_as_float(w[j] & 0xffff0000u)));
+    }
+  }
+  amax = wave_max(amax);
+  if ((tid & 63) == 0) red[tid >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float scale, recip;
+  dynamic_scale_f32(amax, scale_ub, scale, recip);
+  if (tid == 0) scales[row] = scale;
+  uint8_t* dst = out + (int64_t)row * out_stride;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * 256;
+    if (idx < nvec) {
+      const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+      float f[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        f[2 * j] = __uint_as_float(w[j] << 16);
+        f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+      int lo = 0, hi = 0;
+      lo = cvt_pk_e4m3fn(clamp448(f[0] * recip), clamp448(f[1] * recip), lo, false);
+      lo = cvt_pk_e4m3fn(clamp448(f[2] * recip), clamp448(f[3] * recip), lo, true);
+      hi = cvt_pk_e4m3fn(clamp448(f[4] * recip), clamp448(f[5] * recip), hi, false);
+      hi = cvt_pk_e4m3fn(clamp448(f[6] * recip), clamp448(f[7] * recip), hi, true);
+      reinterpret_cast<uint2*>(dst)[idx] = make_uint2((uint32_t)lo, (uint32_t)hi);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float load_elem(const void* p, int dtype, int64_t i) {
+  if (dtype == MAXFP8_BF16) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+  if (dtype == MAXFP8_F16) return (float)reinterpret_cast<const _Float16*>(p)[i];
+  return reinterpret_cast<const float*>(p)[i];
+}
+
+__device__ __forceinline__ uint8_t encode_one(float v) {
+  return (uint8_t)(cvt_pk_e4m3fn(v, 0.0f, 0, false) & 0xff);
+}
+
+// One block per (row, group); any group size, dtype and alignment.
+__global__ __launch_bounds__(256) void quant_generic_kernel(
+    uint8_t* __restrict__ out, void* __restrict__ scales, const void* __restrict__ in,
+    int ngroups, int G, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
+    int in_dtype, int scales_dtype, float scale_ub) {
+  __shared__ float red[4];
+  const int row = blockIdx.x / ngroups, g = blockIdx.x - row * ngroups;
+  const int tid = threadIdx.x;
+  const int64_t base = (int64_t)row * in_stride + (int64_t)g * G;
+  float amax = 0.0f;
+  for (int i = tid; i < G; i += 256) amax = fmaxf(amax, fabsf(load_elem(in, in_dtype, base + i)));
+  amax = wave_max(amax);
+  if ((tid & 63) == 0) red[tid >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float scale, recip;
+  if (scales_dtype == MAXFP8_BF16) {
+    // scale is formed in f32 from bf16-rounded operands and rounded to bf16 once more
+    const float a = bf16_bits_to_f32(f32_to_bf16_bits(amax));
+    const float ub = bf16_bits_to_f32(f32_to_bf16_bits(scale_ub));
+    const uint32_t sb = f32_to_bf16_bits(fminf(a, ub) / 448.0f);
+    scale = bf16_bits_to_f32(sb);
+    float r = 0.0f;
+    if (scale != 0.0f) {
+      r = 1.0f / scale;
+      if (isinf(r) || isnan(r)) r = 0.0f;
+    }
+    recip = r;
+    if (tid == 0) reinterpret_cast<uint16_t*>(scales)[(int64_t)g * scales_ld + row] = (uint16_t)sb;
+  } else {
+    dynamic_scale_f32(amax, scale_ub, scale, recip);
+    if (tid == 0) reinterpret_cast<float*>(scales)[(int64_t)g * scales_ld + row] = scale;
+  }
+  uint8_t* dst = out + (int64_t)row * out_stride + (int64_t)g * G;
+  for (int i = tid; i < G; i += 256) dst[i] = encode_one(clamp448(load_elem(in, in_dtype, base + i) * recip));
+}
+
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void cast_f32_to_e4m3fn_kernel(uint8_t* out, const float* in, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i < n; i += stride) out[i] = encode_one(clamp448(in[i]));
+}
+
+__global__ __launch_bounds__(256) void cast_e4m3fn_to_f32_kernel(float* out, const uint8_t* in, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i < n; i += stride) {
+    v2f f = __builtin_amdgcn_cvt_pk_f32_fp8((int)in[i], false);
+    out[i] = f.x;
+  }
+}
+
+__global__ __launch_bounds__(256) void copy_bytes_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, int64_t nvec) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i < nvec; i += stride) dst[i] = src[i];
+}
+
+// ---------------------------------------------------------------------------
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M, int64_t K,
+                      int64_t in_row_stride, int64_t out_row_stride, int64_t G, int64_t scales_ld,
+                      int in_dtype, int scales_dtype, float scale_ub, hipStream_t stream) {
+  const int64_t ngroups = K / G;
+  const bool fast_types = in_dtype == MAXFP8_BF16 && scales_dtype == MAXFP8_F32;
+  const bool vec_ok = aligned16(in) && (in_row_stride % 8 == 0) && (reinterpret_cast<uintptr_t>(out_fp8) % 8 == 0) &&
+                      (out_row_stride % 8 == 0);
+  if (fast_types && vec_ok && G == 128) {
+    constexpr int U = 4;
+    const int64_t nxb = ceil_div(ngroups, U);
+    const int64_t blocks = ceil_div(M, 16) * nxb;
+    if (blocks < (int64_t)1 << 31) {
+      hipLaunchKernelGGL(quant_g128_bf16_kernel<U>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                         (uint8_t*)out_fp8, (float*)out_scales, (const uint16_t*)in, (int)M, (int)ngroups,
+                         (int)nxb, in_row_stride, out_row_stride, scales_ld, scale_ub);
+      return launch_status("quant_g128_bf16");
+    }
+  }
+  if (fast_types && vec_ok && G == K && K % 8 == 0 && K <= 256 * 8 * 16 && M < ((int64_t)1 << 31)) {
+    const int nvec = (int)(K / 8);
+    const int nv = (nvec + 255) / 256;
+    uint8_t* o = (uint8_t*)out_fp8;
+    float* s = (float*)out_scales;
+    const uint16_t* x = (const uint16_t*)in;
+#define LAUNCH_ROW(NV)                                                                            \
+  hipLaunchKernelGGL(quant_row_bf16_kernel<NV>, dim3((unsigned)M), dim3(256), 0, stream, o, s, x, \
+                     (int)K, in_row_stride, out_row_stride, scale_ub)
+    if (nv <= 1) LAUNCH_ROW(1);
+    else if (nv <= 2) LAUNCH_ROW(2);
+    else if (nv <= 4) LAUNCH_ROW(4);
+    else if (nv <= 8) LAUNCH_ROW(8);
+    else LAUNCH_ROW(16);
+#undef LAUNCH_ROW
+    return launch_status("quant_row_bf16");
+  }
+  const int64_t blocks = M * ngroups;
+  if (blocks >= (int64_t)1 << 31) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: M * K/group_size = %lld exceeds the grid limit", (long long)blocks);
+  hipLaunchKernelGGL(quant_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint8_t*)out_fp8,
+                     out_scales, in, (int)ngroups, (int)G, in_row_stride, out_row_stride, scales_ld, in_dtype,
+                     scales_dtype, scale_ub);
+  return launch_status("quant_generic");
+}
+
+int cast_f32_to_e4m3fn_dispatch(void* out, const float* in, int64_t n, hipStream_t stream) {
+  const unsigned blocks = (unsigned)(ceil_div(n, 256) < 65536 ? ceil_div(n, 256) : 65536);
+  hipLaunchKernelGGL(cast_f32_to_e4m3fn_kernel, dim3(blocks), dim3(256), 0, stream, (uint8_t*)out, in, n);
+  return launch_status("cast_f32_to_e4m3fn");
+}
+
+int cast_e4m3fn_to_f32_dispatch(float* out, const void* in, int64_t n, hipStream_t stream) {
+  const unsigned blocks = (unsigned)(ceil_div(n, 256) < 65536 ? ceil_div(n, 256) : 65536);
+  hipLaunchKernelGGL(cast_e4m3fn_to_f32_kernel, dim3(blocks), dim3(256), 0, stream, out, (const uint8_t*)in, n);
+  return launch_status("cast_e4m3fn_to_f32");
+}
+
+int copy_bytes_dispatch(void* dst, const void* src, int64_t n, hipStream_t stream) {
+  const int64_t nvec = n / 16;
+  const unsigned blocks = (unsigned)(ceil_div(nvec, 256) < 16384 ? ceil_div(nvec, 256) : 16384);
+  hipLaunchKernelGGL(copy_bytes_kernel, dim3(blocks), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src, nvec);
+  return launch_status("copy_bytes");
+}
+
+}  // namespace maxfp8

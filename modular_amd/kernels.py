@@ -1,0 +1,299 @@
+"""Eager op wrappers with the names, argument order, shape rules and exceptions
+of the reference's graph-op wrappers:
+
+  quantize_dynamic_scaled_float8      max/python/max/nn/kernels.py:6876-6957
+  dynamic_scaled_matmul               max/python/max/nn/kernels.py:6960-7078
+  grouped_dynamic_scaled_fp8_matmul   max/python/max/nn/kernels.py:6327-6487
+
+They take torch tensors that live on the MI355X and call the HIP kernels through
+the C ABI on torch's current stream.  Nothing here computes on the CPU.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .quant_config import InputScaleSpec, WeightScaleSpec
+
+_FP8 = torch.float8_e4m3fn
+_DT = {torch.bfloat16: _lib.BF16, torch.float16: _lib.F16, torch.float32: _lib.F32, _FP8: _lib.E4M3FN}
+_ALGOS = {"auto": _lib.ALGO_AUTO, "naive": _lib.ALGO_NAIVE, "tiled": _lib.ALGO_TILED, "skinny": _lib.ALGO_SKINNY}
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("maxfp8 kernels run on the GPU only: got a tensor on " + str(t.device))
+
+
+def quantize_output_geometry(M: int, K: int, input_scale_spec: InputScaleSpec,
+                             weight_scale_spec: WeightScaleSpec, group_size_or_per_token: int,
+                             scales_type: torch.dtype) -> tuple[int, int]:
+    """(group size, padded column count of the scales tensor), the rules of
+    max/python/max/nn/kernels.py:6910-6931: the group is block_size[1] for block
+    specs and K otherwise; block specs pad the token axis of the scales to 16 bytes."""
+    if group_size_or_per_token == -1:
+        if input_scale_spec.is_block or weight_scale_spec.is_block:
+            assert input_scale_spec.block_size is not None
+            group_size = input_scale_spec.block_size[1]
+        else:
+            group_size = int(K)
+    else:
+        group_size = group_size_or_per_token
+    a_scales_dim1 = M
+    if input_scale_spec.is_block or weight_scale_spec.is_block:
+        if not (input_scale_spec.is_block and weight_scale_spec.is_block):
+            raise ValueError("both input and weight must be blockwise scaled for blockwise scaling")
+        padding_size = 16 // torch.empty((), dtype=scales_type).element_size()
+        a_scales_dim1 = ((M + padding_size - 1) // padding_size) * padding_size
+    return group_size, a_scales_dim1
+
+
+def quantize_dynamic_scaled_float8(
+    input: torch.Tensor,
+    input_scale_spec: InputScaleSpec,
+    weight_scale_spec: WeightScaleSpec,
+    scale_ub: float = 1200.0,
+    group_size_or_per_token: int = -1,
+    out_type: torch.dtype = _FP8,
+    scales_type: torch.dtype = torch.bfloat16,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Dynamically quantize `input` [M, K] to fp8.
+
+    Returns (quantized [M, K] e4m3fn, scales [K / group, M_pad]) where, for block
+    specs, M_pad rounds M up to a multiple of 16 bytes / sizeof(scale); the padding
+    columns are allocated but never written.
+    """
+    if input.dim() != 2:
+        raise ValueError("input must be rank 2 tensor")
+    if out_type != _FP8:
+        # e4m3fnuz is only ever requested on gfx94x (kernels.py:8408-8417)
+        raise ValueError("out_type must be float8_e4m3fn or float8_e4m3fnuz")
+    M, K = input.shape
+
+    group_size, a_scales_dim1 = quantize_output_geometry(
+        M, K, input_scale_spec, weight_scale_spec, group_size_or_per_token, scales_type)
+
+    if scales_type not in (torch.float32, torch.bfloat16):
+        raise TypeError("scales dtype should be bfloat16 or float32")
+    if input.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError(f"input dtype {input.dtype} is not bfloat16, float16 or float32")
+    if group_size <= 0 or K % group_size != 0:
+        raise ValueError(f"group size {group_size} must divide K = {K}")
+
+    _require_gpu(input)
+    if input.stride(1) != 1:
+        input = input.contiguous()
+    out = torch.empty((M, K), dtype=_FP8, device=input.device)
+    scales = torch.empty((K // group_size, a_scales_dim1), dtype=scales_type, device=input.device)
+    st = _lib.lib().maxfp8_quantize_dynamic_scaled_fp8(
+        out.data_ptr(), scales.data_ptr(), input.data_ptr(), M, K, input.stride(0) if M > 1 else K, K,
+        group_size, a_scales_dim1, _DT[input.dtype], _DT[scales_type], float(scale_ub), _stream(input))
+    _lib.check(st)
+    return out, scales
+
+
+def dynamic_scaled_matmul(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    input_scale_spec: InputScaleSpec,
+    weight_scale_spec: WeightScaleSpec,
+    out_type: torch.dtype = torch.bfloat16,
+    *,
+    algo: str = "auto",
+) -> torch.Tensor:
+    """C = A . B^T with scaling factors; `b` is [N, K] (already "transposed")."""
+    if a.dim() != 2 or b.dim() != 2 or a_scales.dim() != 2 or b_scales.dim() != 2:
+        raise ValueError("All arguments must be rank 2 tensors")
+    if a.shape[1] != b.shape[1]:
+        raise ValueError("The second dimension of b must match the second dimension of a")
+
+    gm = gn = gk = -1
+    if input_scale_spec.is_tensor and weight_scale_spec.is_tensor:
+        if input_scale_spec.origin.is_dynamic:
+            if not (b_scales.shape[0] == b_scales.shape[1] == 1):
+                raise ValueError("scaler weight tensors must be of shape [1, 1] for dynamic tensor scaling")
+        else:
+            if not (a_scales.shape[0] == a_scales.shape[1] == b_scales.shape[0] == b_scales.shape[1] == 1):
+                raise ValueError("scaler tensors must be of shape [1, 1] for tensor scaling")
+        gin, gw = _lib.GRAN_TENSOR, _lib.GRAN_TENSOR
+    elif input_scale_spec.is_colwise and weight_scale_spec.is_rowwise:
+        if a_scales.shape[0] != 1:
+            raise ValueError("only per-token scaling is supported for a")
+        if b_scales.shape[1] != 1:
+            raise ValueError("only channel-wise scaling is supported for b")
+        gin, gw = _lib.GRAN_COLWISE, _lib.GRAN_ROWWISE
+    elif input_scale_spec.is_block or weight_scale_spec.is_block:
+        if input_scale_spec.block_size is None or weight_scale_spec.block_size is None:
+            raise ValueError("both input and weight block size must be set for blockwise scaling")
+        if not (input_scale_spec.is_block and weight_scale_spec.is_block):
+            raise ValueError("both input and weight must be blockwise scaled for blockwise scaling")
+        if a_scales.dtype != b_scales.dtype or a_scales.dtype != torch.float32:
+            raise TypeError(
+                f"a_scales and b_scales dtypes must be float32, but got {a_scales.dtype}, {b_scales.dtype}")
+        if a_scales.shape[0] != b_scales.shape[1]:
+            raise ValueError(
+                "both a_scales and b_scales must have the same shape on the K dimension. got "
+                f"a_scales.shape={tuple(a_scales.shape)} and b_scales.shape={tuple(b_scales.shape)}")
+        gin, gw = _lib.GRAN_BLOCK, _lib.GRAN_BLOCK
+        gm = input_scale_spec.block_size[0]
+        gn, gk = weight_scale_spec.block_size
+    else:
+        raise ValueError("unsupported FP8 scaling granularity")
+
+    if (a.dtype != b.dtype) or (a_scales.dtype != b_scales.dtype):
+        raise TypeError(
+            f"a and b dtypes {a.dtype}, {b.dtype} must match, as do a and b scales dtypes "
+            f"{a_scales.dtype}, {b_scales.dtype}")
+    if a.dtype != _FP8:
+        raise TypeError(f"a and b must be float8_e4m3fn, got {a.dtype}")
+    if a_scales.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"scales dtype {a_scales.dtype} is not float32 or bfloat16")
+    if out_type not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"out_type {out_type} is not bfloat16 or float32")
+    if gin == _lib.GRAN_COLWISE and a_scales.shape[1] < a.shape[0]:
+        raise ValueError("a_scales must hold one scale per row of a")
+    if gin == _lib.GRAN_COLWISE and b_scales.shape[0] != b.shape[0]:
+        raise ValueError("b_scales must hold one scale per row of b")
+    if gin == _lib.GRAN_BLOCK:
+        if a_scales.shape[0] != -(-a.shape[1] // gk) or a_scales.shape[1] < -(-a.shape[0] // gm):
+            raise ValueError(f"a_scales shape {tuple(a_scales.shape)} does not cover a {tuple(a.shape)}")
+        if b_scales.shape[0] != -(-b.shape[0] // gn):
+            raise ValueError(f"b_scales shape {tuple(b_scales.shape)} does not cover b {tuple(b.shape)}")
+
+    _require_gpu(a, b, a_scales, b_scales)
+    if a.stride(1) != 1:
+        a = a.contiguous()
+    if b.stride(1) != 1:
+        b = b.contiguous()
+    if a_scales.stride(1) != 1:
+        a_scales = a_scales.contiguous()
+    if b_scales.dim() == 2 and b_scales.shape[1] > 1 and b_scales.stride(1) != 1:
+        b_scales = b_scales.contiguous()
+    M, K = a.shape
+    N = b.shape[0]
+    c = torch.empty((M, N), dtype=out_type, device=a.device)
+    lda = a.stride(0) if M > 1 else K
+    ldb = b.stride(0) if N > 1 else K
+    a_ld = a_scales.stride(0) if a_scales.shape[0] > 1 else a_scales.shape[1]
+    b_ld = b_scales.stride(0) if b_scales.shape[0] > 1 else b_scales.shape[1]
+    st = _lib.lib().maxfp8_matmul_dynamic_scaled_fp8(
+        c.data_ptr(), a.data_ptr(), b.data_ptr(), a_scales.data_ptr(), b_scales.data_ptr(), M, N, K,
+        lda, ldb, N, gin, gw, gm, gn, gk, a_ld, b_ld, _DT[out_type], _DT[a_scales.dtype], _ALGOS[algo],
+        None, 0, _stream(a))
+    _lib.check(st)
+    return c
+
+
+def grouped_dynamic_scaled_fp8_matmul(
+    hidden_states: torch.Tensor,
+    weight: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    expert_start_indices: torch.Tensor,
+    expert_ids: torch.Tensor,
+    expert_usage_stats_host: torch.Tensor,
+    input_scale_spec: InputScaleSpec,
+    weight_scale_spec: WeightScaleSpec,
+    out_type: torch.dtype = torch.bfloat16,
+    *,
+    algo: str = "auto",
+) -> torch.Tensor:
+    """Grouped blockwise scaled matmul of the MoE layer: rows of `hidden_states`
+    are sorted by expert, `expert_start_indices` delimits the groups,
+    `expert_usage_stats_host` = [max tokens of any expert, number of active experts]
+    on the CPU."""
+    if weight.dim() != 3:
+        raise ValueError(f"expected weight of rank 3 but got {weight.dim()}")
+    if hidden_states.dim() != 2:
+        raise ValueError(f"expected hidden_states of rank 2 but got {hidden_states.dim()}")
+    if weight.shape[2] != hidden_states.shape[1] or weight.shape[0] != expert_ids.shape[0]:
+        raise ValueError(
+            f"expected weight is of shape [num_experts, *, {hidden_states.shape[1]}] but got {tuple(weight.shape)}")
+    if (hidden_states.dtype != weight.dtype) or (hidden_states.dtype != _FP8):
+        raise TypeError(
+            f"hidden_states and weight dtypes must be float8_e4m3fn, but got {hidden_states.dtype}, {weight.dtype}")
+    if (a_scales.dtype != b_scales.dtype) or (a_scales.dtype not in (torch.float32, torch.bfloat16)):
+        raise TypeError(
+            f"a_scales and b_scales dtypes must be float32 or bfloat16 and match, but got {a_scales.dtype}, {b_scales.dtype}")
+    if expert_ids.dtype != torch.int32:
+        raise TypeError(f"expert_ids dtype must be int32, but got {expert_ids.dtype}")
+    if expert_ids.dim() != 1:
+        raise ValueError(f"expected expert_ids of rank 1 but got {expert_ids.dim()}")
+    if expert_start_indices.dtype != torch.uint32:
+        raise TypeError(f"expert_start_indices dtype must be uint32, but got {expert_start_indices.dtype}")
+    if expert_start_indices.dim() != 1:
+        raise ValueError(f"expected expert_start_indices of rank 1 but got {expert_start_indices.dim()}")
+    if a_scales.dim() != 2 or b_scales.dim() != 3:
+        raise ValueError(
+            f"expected a_scales of rank 2 and b_scales of rank 3 but got {a_scales.dim()} and {b_scales.dim()}")
+
+    if input_scale_spec.is_block and weight_scale_spec.is_block:
+        if input_scale_spec.block_size is None or weight_scale_spec.block_size is None:
+            raise ValueError("both input block_size and weight block_size must be set for grouped blockwise scaling")
+        if input_scale_spec.block_size[0] != 1 or input_scale_spec.block_size[1] != 128:
+            raise ValueError("grouped blockwise scaling only supports (1,128) granularity for input")
+        if weight_scale_spec.block_size[0] != 128 or weight_scale_spec.block_size[1] != 128:
+            raise ValueError("grouped blockwise scaling only supports (128,128) granularity for weight")
+    else:
+        raise ValueError("grouped FP8 matmul only supports blockwise scaling")
+    if a_scales.dtype != torch.float32:
+        raise TypeError("this build executes float32 scales only for the grouped matmul")
+
+    T, K = hidden_states.shape
+    E, N, _ = weight.shape
+    kb, nb = -(-K // 128), -(-N // 128)
+    if a_scales.shape[0] != kb or a_scales.shape[1] < T:
+        raise ValueError(f"a_scales shape {tuple(a_scales.shape)} does not cover hidden_states {tuple(hidden_states.shape)}")
+    if tuple(b_scales.shape) != (E, nb, kb):
+        raise ValueError(f"b_scales shape {tuple(b_scales.shape)} is not {(E, nb, kb)}")
+    stats = expert_usage_stats_host
+    if stats.is_cuda:
+        raise ValueError("expert_usage_stats_host must live on the CPU")
+    max_tokens, num_active = int(stats[0]), int(stats[1])
+    if expert_start_indices.shape[0] < num_active + 1:
+        raise ValueError("expert_start_indices is shorter than num_active_experts + 1")
+
+    _require_gpu(hidden_states, weight, a_scales, b_scales, expert_start_indices, expert_ids)
+    hidden_states = hidden_states.contiguous()
+    weight = weight.contiguous()
+    a_scales = a_scales if a_scales.stride(1) == 1 else a_scales.contiguous()
+    b_scales = b_scales.contiguous()
+    c = torch.empty((T, N), dtype=out_type, device=hidden_states.device)
+    a_ld = a_scales.stride(0) if a_scales.shape[0] > 1 else a_scales.shape[1]
+    st = _lib.lib().maxfp8_grouped_matmul_dynamic_scaled_fp8(
+        c.data_ptr(), hidden_states.data_ptr(), weight.data_ptr(), a_scales.data_ptr(), b_scales.data_ptr(),
+        expert_start_indices.data_ptr(), expert_ids.data_ptr(), T, N, K, E, max_tokens, num_active, a_ld,
+        _DT[out_type], _DT[a_scales.dtype], _ALGOS[algo], _stream(hidden_states))
+    _lib.check(st)
+    return c
+
+
+# ---- utilities exposed for tests and calibration ------------------------------------
+
+def cast_f32_to_e4m3fn(x: torch.Tensor) -> torch.Tensor:
+    _require_gpu(x)
+    x = x.contiguous().to(torch.float32)
+    out = torch.empty(x.shape, dtype=_FP8, device=x.device)
+    _lib.check(_lib.lib().maxfp8_cast_f32_to_e4m3fn(out.data_ptr(), x.data_ptr(), x.numel(), _stream(x)))
+    return out
+
+
+def cast_e4m3fn_to_f32(x: torch.Tensor) -> torch.Tensor:
+    _require_gpu(x)
+    x = x.contiguous()
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.lib().maxfp8_cast_e4m3fn_to_f32(out.data_ptr(), x.data_ptr(), x.numel(), _stream(x)))
+    return out
+
+
+def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
+    _require_gpu(dst, src)
+    n = src.numel() * src.element_size()
+    _lib.check(_lib.lib().maxfp8_copy_bytes(dst.data_ptr(), src.data_ptr(), n, _stream(src)))

@@ -1,0 +1,61 @@
+"""FP8 dispatch of a quantised linear, mirroring `quantized_matmul` /
+`_matmul_float8` (max/python/max/nn/quant_ops.py:516-592, 336-481) for the
+dynamic-scale branches this package executes on the MI355X.
+"""
+from __future__ import annotations
+
+import torch
+
+from .kernels import dynamic_scaled_matmul, quantize_dynamic_scaled_float8
+from .quant_config import InputScaleSpec, QuantConfig, ScaleGranularity, WeightScaleSpec
+
+
+def matmul_float8(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    weight_scale: torch.Tensor,
+    input_scale: torch.Tensor | None,
+    quant_config: QuantConfig,
+) -> torch.Tensor:
+    """x @ weight.T with float8 quantisation; x [M, K] bf16, weight [N, K] e4m3fn."""
+    if input_scale is not None:
+        # static activation scales (quant_ops.py:384-417) are a different operator
+        raise NotImplementedError("static FP8 activation scales are outside the dynamic FP8 linear path")
+
+    if quant_config.input_scale.is_tensor and quant_config.weight_scale.is_tensor:
+        # Dynamic tensor-wise FP8 is executed as per-token x per-channel with the
+        # scalar weight scale broadcast to [N, 1] (quant_ops.py:418-461).
+        n_out = weight.shape[0]
+        if weight_scale.dim() < 2:
+            weight_scale = weight_scale.reshape(1, 1).expand(n_out, 1).contiguous()
+        weight_scale = weight_scale.to(x.device)
+        in_spec = InputScaleSpec(ScaleGranularity.COLWISE, quant_config.input_scale.origin, weight_scale.dtype)
+        w_spec = WeightScaleSpec(ScaleGranularity.ROWWISE, weight_scale.dtype)
+        xq, x_scales = quantize_dynamic_scaled_float8(x, in_spec, w_spec, scales_type=weight_scale.dtype,
+                                                      out_type=weight.dtype)
+        return dynamic_scaled_matmul(xq, weight, x_scales, weight_scale, in_spec, w_spec,
+                                     out_type=torch.bfloat16)
+
+    # dynamic per-row / block scaling (quant_ops.py:462-481)
+    xq, x_scale = quantize_dynamic_scaled_float8(
+        x, quant_config.input_scale, quant_config.weight_scale,
+        scales_type=weight_scale.dtype, out_type=weight.dtype)
+    weight_scale = weight_scale.to(x.device)
+    return dynamic_scaled_matmul(xq, weight, x_scale, weight_scale, quant_config.input_scale,
+                                 quant_config.weight_scale, out_type=torch.bfloat16)
+
+
+def quantized_matmul(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    weight_scale: torch.Tensor,
+    input_scale: torch.Tensor | None = None,
+    quant_config: QuantConfig | None = None,
+) -> torch.Tensor:
+    """Entry point of the quantised linear (quant_ops.py:516-592): only the FP8
+    formats are in this package."""
+    if quant_config is None:
+        raise ValueError("quant_config is required for a quantized matmul")
+    if weight.dtype != torch.float8_e4m3fn:
+        raise TypeError(f"weight dtype {weight.dtype} is not float8_e4m3fn")
+    return matmul_float8(x, weight, weight_scale, input_scale, quant_config)

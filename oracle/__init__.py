@@ -1,0 +1,187 @@
+"""ctypes front end of the CPU oracle (oracle/maxfp8_oracle.c).
+
+TEST INFRASTRUCTURE ONLY.  Importable from tests/, ``__graft_entry__.smoke()``
+and the ``cpu_baseline`` leg of ``bench.py``; the product package never imports
+it.  Arrays are numpy: bf16 travels as ``uint16`` bit patterns, e4m3fn as
+``uint8`` bytes.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libmaxfp8_oracle.so")
+
+BF16, F16, F32 = 0, 1, 2
+
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (seconds).  Returns the path of the .so."""
+    src = os.path.join(_HERE, "maxfp8_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libmaxfp8_oracle.so"],
+                              stdout=subprocess.DEVNULL)
+    return _SO
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_SO)
+        L.orc_e4m3fn_to_f32.restype = ctypes.c_float
+        L.orc_e4m3fn_to_f32.argtypes = [ctypes.c_uint8]
+        L.orc_f32_to_e4m3fn.restype = ctypes.c_uint8
+        L.orc_f32_to_e4m3fn.argtypes = [ctypes.c_float]
+        L.orc_f32_to_e4m3fn_array.restype = None
+        L.orc_f32_to_e4m3fn_array.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+        L.orc_dynamic_scale.restype = None
+        L.orc_dynamic_scale.argtypes = [ctypes.c_float, ctypes.c_float, ctypes.c_int,
+                                        ctypes.POINTER(ctypes.c_float),
+                                        ctypes.POINTER(ctypes.c_float)]
+        i64, vp, ci, cf = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+        L.orc_quantize_dynamic_scaled_fp8.restype = ci
+        L.orc_quantize_dynamic_scaled_fp8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64,
+                                                      i64, ci, ci, cf, ci]
+        L.orc_matmul_blockwise.restype = ci
+        L.orc_matmul_blockwise.argtypes = [vp, vp, vp, vp, vp] + [i64] * 11 + [ci, ci, ci]
+        L.orc_matmul_rowwise.restype = ci
+        L.orc_matmul_rowwise.argtypes = [vp, vp, vp, vp, vp] + [i64] * 8 + [ci, ci, ci]
+        L.orc_grouped_matmul.restype = ci
+        L.orc_grouped_matmul.argtypes = [vp] * 7 + [i64] * 7 + [ci, ci, ci]
+        L.orc_max_threads.restype = ci
+        _lib = L
+    return _lib
+
+
+def _p(a: np.ndarray) -> ctypes.c_void_p:
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def default_threads() -> int:
+    try:
+        return max(1, len(os.sched_getaffinity(0)))
+    except AttributeError:  # pragma: no cover
+        return os.cpu_count() or 1
+
+
+# ---- codec -----------------------------------------------------------------
+
+def e4m3fn_decode_table() -> np.ndarray:
+    L = lib()
+    return np.array([L.orc_e4m3fn_to_f32(i) for i in range(256)], dtype=np.float32)
+
+
+def e4m3fn_decode(b: np.ndarray) -> np.ndarray:
+    return e4m3fn_decode_table()[np.asarray(b, dtype=np.uint8)]
+
+
+def e4m3fn_encode(x: np.ndarray) -> np.ndarray:
+    """Encode f32 values (round to nearest even, saturating, NaN -> 0x7f)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint8)
+    lib().orc_f32_to_e4m3fn_array(_p(out), _p(x), x.size)
+    return out
+
+
+def dynamic_scale(amax: float, scale_ub: float = 1200.0, scales_dtype: int = F32):
+    s, r = ctypes.c_float(), ctypes.c_float()
+    lib().orc_dynamic_scale(amax, scale_ub, scales_dtype, ctypes.byref(s), ctypes.byref(r))
+    return np.float32(s.value), np.float32(r.value)
+
+
+# ---- operators ---------------------------------------------------------------
+
+def quantize_dynamic_scaled_fp8(x: np.ndarray, group_size: int, *, in_dtype: int = BF16,
+                                scales_dtype: int = F32, scale_ub: float = 1200.0,
+                                scales_ld: int | None = None, threads: int = 1):
+    """x: [M, K] (uint16 bits for bf16/f16, float32 for f32).  Returns
+    (q uint8 [M, K], scales [K/G, scales_ld]); unwritten scale columns hold NaN
+    bit patterns (f32) / 0xFFFF (bf16) so a test can see they stay untouched."""
+    x = np.ascontiguousarray(x)
+    M, K = x.shape
+    G = K if group_size == -1 else group_size
+    ld = M if scales_ld is None else scales_ld
+    q = np.zeros((M, K), dtype=np.uint8)
+    if scales_dtype == F32:
+        sc = np.full((K // G, ld), np.nan, dtype=np.float32)
+    else:
+        sc = np.full((K // G, ld), 0xFFFF, dtype=np.uint16)
+    rc = lib().orc_quantize_dynamic_scaled_fp8(_p(q), _p(sc), _p(x), M, K, K, K, G, ld,
+                                               in_dtype, scales_dtype, scale_ub, threads)
+    if rc:
+        raise ValueError(f"oracle quantize failed: {rc}")
+    return q, sc
+
+
+def matmul_blockwise(a: np.ndarray, b: np.ndarray, a_scales: np.ndarray, b_scales: np.ndarray,
+                     *, gmnk=(1, 128, 128), c_dtype: int = F32, mode: int = 0,
+                     threads: int = 1) -> np.ndarray:
+    a = np.ascontiguousarray(a, dtype=np.uint8)
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    a_scales = np.ascontiguousarray(a_scales, dtype=np.float32)
+    b_scales = np.ascontiguousarray(b_scales, dtype=np.float32)
+    M, K = a.shape
+    N = b.shape[0]
+    c = np.zeros((M, N), dtype=np.float32 if c_dtype == F32 else np.uint16)
+    rc = lib().orc_matmul_blockwise(_p(c), _p(a), _p(b), _p(a_scales), _p(b_scales),
+                                    M, N, K, K, K, N, gmnk[0], gmnk[1], gmnk[2],
+                                    a_scales.shape[1], b_scales.shape[1], c_dtype, mode, threads)
+    if rc:
+        raise ValueError(f"oracle blockwise matmul failed: {rc}")
+    return c
+
+
+def matmul_rowwise(a: np.ndarray, b: np.ndarray, a_scales: np.ndarray, b_scales: np.ndarray,
+                   *, c_dtype: int = F32, tensor_scales: bool = False,
+                   threads: int = 1) -> np.ndarray:
+    """a_scales [1, M] (or [1,1]), b_scales [N, 1] (or [1,1]); f32."""
+    a = np.ascontiguousarray(a, dtype=np.uint8)
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    a_scales = np.ascontiguousarray(a_scales, dtype=np.float32)
+    b_scales = np.ascontiguousarray(b_scales, dtype=np.float32)
+    M, K = a.shape
+    N = b.shape[0]
+    c = np.zeros((M, N), dtype=np.float32 if c_dtype == F32 else np.uint16)
+    st = 0 if tensor_scales else 1
+    rc = lib().orc_matmul_rowwise(_p(c), _p(a), _p(b), _p(a_scales), _p(b_scales),
+                                  M, N, K, K, K, N, st, st, c_dtype, F32, threads)
+    if rc:
+        raise ValueError(f"oracle rowwise matmul failed: {rc}")
+    return c
+
+
+def grouped_matmul(a: np.ndarray, b: np.ndarray, a_scales: np.ndarray, b_scales: np.ndarray,
+                   offsets: np.ndarray, expert_ids: np.ndarray, max_tokens: int,
+                   num_active: int, *, c_dtype: int = F32, mode: int = 0, threads: int = 1,
+                   fill: float = np.nan) -> np.ndarray:
+    """Rows no active slot owns keep `fill` (f32 output) so a test can see that
+    they are not written."""
+    a = np.ascontiguousarray(a, dtype=np.uint8)
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    a_scales = np.ascontiguousarray(a_scales, dtype=np.float32)
+    b_scales = np.ascontiguousarray(b_scales, dtype=np.float32)
+    offsets = np.ascontiguousarray(offsets, dtype=np.uint32)
+    expert_ids = np.ascontiguousarray(expert_ids, dtype=np.int32)
+    T, K = a.shape
+    E, N, _ = b.shape
+    if c_dtype == F32:
+        c = np.full((T, N), fill, dtype=np.float32)
+    else:
+        c = np.full((T, N), 0x7FC0, dtype=np.uint16)
+    rc = lib().orc_grouped_matmul(_p(c), _p(a), _p(b), _p(a_scales), _p(b_scales),
+                                  _p(offsets), _p(expert_ids), T, N, K, E, max_tokens,
+                                  num_active, a_scales.shape[1], c_dtype, mode, threads)
+    if rc:
+        raise ValueError(f"oracle grouped matmul failed: {rc}")
+    return c
+
+
+def bf16_bits_to_f32(u: np.ndarray) -> np.ndarray:
+    return (np.asarray(u, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)

@@ -1,0 +1,51 @@
+"""End-to-end FP8 linear (quantise + matmul through `Linear`) against the CPU oracle on
+BASELINE's first configuration: x bf16 [64, 4096] with outlier channels, W [4096, 4096]
+block-quantised offline, bf16 out."""
+import numpy as np
+import pytest
+import torch
+
+import modular_amd as mx
+import oracle
+from modular_amd import synth
+from util import assert_rel, bf16_bits, f32_np, fp8_bytes
+
+pytestmark = pytest.mark.gpu
+NT = oracle.default_threads()
+
+
+def test_config0_single_linear(dev):
+    M, K, N = 64, 4096, 4096
+    cfg = mx.blockwise_fp8_config()
+    x = synth.activations(M, K, seed=0)
+    wq, ws = synth.quantize_weight_block(synth.weights_f32(N, K, seed=0))
+    lin = mx.Linear(K, N, cfg, device=dev)
+    lin.weight.copy_(wq.to(dev))
+    lin.weight_scale.copy_(ws.to(dev))
+    y = lin(x.to(dev).reshape(2, 32, K))
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (2, 32, N) and y.dtype == torch.bfloat16
+    q, sa = oracle.quantize_dynamic_scaled_fp8(bf16_bits(x), 128, threads=NT)
+    ref = oracle.matmul_blockwise(q, fp8_bytes(wq), sa, ws.numpy(), threads=NT)
+    assert_rel(f32_np(y.reshape(M, N)), ref, 1e-2, "config 0")
+    # against the unquantised product the error is the quantisation noise, a few percent of the row rms
+    full = x.float() @ synth.weights_f32(N, K, seed=0).t()
+    err = (y.reshape(M, N).float().cpu() - full).norm() / full.norm()
+    assert err < 0.08
+
+
+def test_rowwise_linear_and_bias(dev):
+    M, K, N = 5, 1024, 768
+    cfg = mx.rowwise_fp8_config()
+    x = synth.activations(M, K, seed=2, outlier_frac=0.0)
+    wq, ws = synth.quantize_weight_rowwise(synth.weights_f32(N, K, seed=3))
+    lin = mx.Linear(K, N, cfg, device=dev, has_bias=True)
+    lin.weight.copy_(wq.to(dev))
+    lin.weight_scale.copy_(ws.to(dev))
+    lin.bias.copy_(torch.linspace(-1, 1, N).to(torch.bfloat16))
+    y = lin(x.to(dev))
+    torch.cuda.synchronize()
+    q, sa = oracle.quantize_dynamic_scaled_fp8(bf16_bits(x), K, threads=NT)
+    ref = oracle.matmul_rowwise(q, fp8_bytes(wq), sa, ws.numpy(), threads=NT)
+    ref_b = torch.from_numpy(ref).to(torch.bfloat16) + torch.linspace(-1, 1, N).to(torch.bfloat16)
+    assert_rel(f32_np(y), ref_b.float().numpy(), 1.5e-2, "rowwise linear with bias")

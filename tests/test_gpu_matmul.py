@@ -1,0 +1,221 @@
+"""GPU parity of the scaled FP8 matmuls.
+
+  naive kernels  == CPU oracle bit for bit (f32 out): same summation order
+  MFMA kernels   within max rel err 1e-2 of the oracle (bf16 and f32 out), and bit-exact
+                 where the arithmetic is exact (small integers, power-of-two scales)
+Shapes follow the reference's tests (test_naive_blockwise_fp8_matmul.mojo:194-200,
+test_scaled_matmul.mojo:332-377, test_fp8_matmul_gpu.py:40-442) and BASELINE's configs;
+at sizes the CPU cannot finish, the bit-exact-to-oracle naive kernel checks sampled rows."""
+import numpy as np
+import pytest
+import torch
+
+import modular_amd as mx
+import oracle
+from modular_amd import synth
+from modular_amd.quant_config import InputScaleSpec, QuantConfig, ScaleGranularity, ScaleOrigin, WeightScaleSpec
+from util import assert_rel, bf16_bits, f32_np, fp8_bytes, fp8_from_bytes, rel_err
+
+pytestmark = pytest.mark.gpu
+BLK, ROW = mx.blockwise_fp8_config(), mx.rowwise_fp8_config()
+NT = oracle.default_threads()
+TOL = 1e-2  # BASELINE: max |rel err| <= 1e-2 against the fp32-accumulated reference result
+
+
+def block_cfg(gm, gn, gk):
+    return QuantConfig(InputScaleSpec(ScaleGranularity.BLOCK, ScaleOrigin.DYNAMIC, torch.float32, block_size=(gm, gk)),
+                       WeightScaleSpec(ScaleGranularity.BLOCK, torch.float32, block_size=(gn, gk)))
+
+
+def mm(a, b, sa, sb, cfg, dev, out=torch.float32, algo="auto"):
+    c = mx.dynamic_scaled_matmul(a.to(dev), b.to(dev), sa.to(dev), sb.to(dev), cfg.input_scale, cfg.weight_scale,
+                                 out_type=out, algo=algo)
+    torch.cuda.synchronize()
+    return c
+
+
+def make_block(M, N, K, seed, g=(1, 128, 128), pad_ld=True):
+    gm, gn, gk = g
+    a, b = synth.random_fp8((M, K), seed), synth.random_fp8((N, K), seed + 1)
+    ld = -(-(-(-M // gm)) // 4) * 4 if pad_ld else -(-M // gm)
+    sa = synth.random_scales((-(-K // gk), ld), seed + 2)
+    sb = synth.random_scales((-(-N // gn), -(-K // gk)), seed + 3)
+    return a, b, sa, sb
+
+
+def oracle_block(a, b, sa, sb, g=(1, 128, 128), mode=0):
+    return oracle.matmul_blockwise(fp8_bytes(a), fp8_bytes(b), sa.numpy(), sb.numpy(), gmnk=g, mode=mode, threads=NT)
+
+
+# ---- naive kernel == oracle, bit for bit -------------------------------------------------
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (120, 128, 128), (128, 129, 128), (128, 128, 129), (33, 70, 385)])
+@pytest.mark.parametrize("g", [(1, 128, 128), (1, 64, 128), (1, 64, 16), (32, 128, 64)])
+def test_naive_blockwise_is_the_oracle(dev, M, N, K, g):
+    a, b, sa, sb = make_block(M, N, K, seed=M + N + K + g[1], g=g)
+    c = mm(a, b, sa, sb, block_cfg(*g), dev, algo="naive")
+    assert np.array_equal(f32_np(c), oracle_block(a, b, sa, sb, g))
+    cb = mm(a, b, sa, sb, block_cfg(*g), dev, out=torch.bfloat16, algo="naive")
+    want = oracle.matmul_blockwise(fp8_bytes(a), fp8_bytes(b), sa.numpy(), sb.numpy(), gmnk=g, c_dtype=oracle.BF16)
+    assert np.array_equal(bf16_bits(cb), want)
+
+
+def test_naive_rowwise_is_the_oracle(dev):
+    for (M, N, K) in [(17, 512, 256), (124, 96, 512), (3, 40, 2050)]:
+        a, b = synth.random_fp8((M, K), 1), synth.random_fp8((N, K), 2)
+        sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+        c = mm(a, b, sa, sb, ROW, dev, algo="naive")
+        assert np.array_equal(f32_np(c), oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), sa.numpy(), sb.numpy(), threads=NT))
+
+
+# ---- MFMA kernels: exact cases --------------------------------------------------------------
+
+def exact_case(M, N, K, seed):
+    rng = np.random.default_rng(seed)
+    ai, bi = rng.integers(-4, 5, (M, K)), rng.integers(-4, 5, (N, K))
+    a = fp8_from_bytes(oracle.e4m3fn_encode(ai.astype(np.float32)))
+    b = fp8_from_bytes(oracle.e4m3fn_encode(bi.astype(np.float32)))
+    kb, nb = -(-K // 128), -(-N // 128)
+    ea, eb = rng.integers(-3, 4, (kb, -(-M // 4) * 4)), rng.integers(-3, 4, (nb, kb))
+    want = np.zeros((M, N))
+    for j in range(kb):
+        part = ai[:, j * 128:(j + 1) * 128] @ bi[:, j * 128:(j + 1) * 128].T
+        want += part * np.exp2(ea[j, :M])[:, None] * np.exp2(eb[np.arange(N) // 128, j])[None, :]
+    return a, b, torch.from_numpy(np.exp2(ea).astype(np.float32)), torch.from_numpy(np.exp2(eb).astype(np.float32)), want
+
+
+@pytest.mark.parametrize("algo,M,N,K", [
+    ("tiled", 128, 128, 128), ("tiled", 130, 272, 512), ("tiled", 57, 100, 1040), ("tiled", 256, 384, 2048),
+    ("skinny", 1, 64, 128), ("skinny", 8, 160, 512), ("skinny", 16, 100, 1040), ("skinny", 33, 48, 256),
+    ("skinny", 64, 272, 640),
+])
+def test_mfma_blockwise_exact(dev, algo, M, N, K):
+    a, b, sa, sb, want = exact_case(M, N, K, seed=M * 3 + N + K)
+    c = mm(a, b, sa, sb, BLK, dev, algo=algo)
+    got = f32_np(c).astype(np.float64)
+    bad = np.argwhere(got != want)
+    assert bad.size == 0, f"{len(bad)} mismatches, first at {bad[:4].tolist()}: got {got[tuple(bad[0])]}, want {want[tuple(bad[0])]}"
+    cb = mm(a, b, sa, sb, BLK, dev, out=torch.bfloat16, algo=algo)
+    assert torch.equal(cb.cpu(), torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("algo,M", [("tiled", 150), ("skinny", 5), ("skinny", 40)])
+def test_mfma_rowwise_exact(dev, algo, M):
+    rng = np.random.default_rng(M)
+    N, K = 200, 768
+    ai, bi = rng.integers(-4, 5, (M, K)), rng.integers(-4, 5, (N, K))
+    a = fp8_from_bytes(oracle.e4m3fn_encode(ai.astype(np.float32)))
+    b = fp8_from_bytes(oracle.e4m3fn_encode(bi.astype(np.float32)))
+    sa = torch.from_numpy(np.exp2(rng.integers(-3, 3, (1, M))).astype(np.float32))
+    sb = torch.from_numpy(np.exp2(rng.integers(-3, 3, (N, 1))).astype(np.float32))
+    want = (ai @ bi.T) * sa.numpy().reshape(-1, 1) * sb.numpy().reshape(1, -1)
+    c = mm(a, b, sa, sb, ROW, dev, algo=algo)
+    assert np.array_equal(f32_np(c).astype(np.float64), want)
+
+
+# ---- MFMA kernels: tolerance against the oracle ------------------------------------------
+
+@pytest.mark.parametrize("algo,M,N,K", [
+    ("tiled", 128, 128, 128), ("tiled", 120, 129, 128), ("tiled", 81, 1024, 2048), ("tiled", 300, 576, 1024),
+    ("tiled", 257, 640, 3072), ("tiled", 64, 512, 4096),
+    ("skinny", 1, 1024, 2048), ("skinny", 32, 1024, 2048), ("skinny", 2, 129, 512), ("skinny", 16, 640, 4096),
+    ("skinny", 64, 256, 4096), ("auto", 81, 1024, 2048), ("auto", 7, 576, 7168),
+])
+@pytest.mark.parametrize("out", [torch.float32, torch.bfloat16])
+def test_mfma_blockwise_vs_oracle(dev, algo, M, N, K, out):
+    a, b, sa, sb = make_block(M, N, K, seed=M + N + K)
+    ref = oracle_block(a, b, sa, sb)
+    c = mm(a, b, sa, sb, BLK, dev, out=out, algo=algo)
+    assert_rel(f32_np(c), ref, TOL, f"{algo} {M}x{N}x{K} {out}")
+    if out == torch.float32:
+        # reference kernel test tolerance (test_naive_blockwise_fp8_matmul.mojo: atol = rtol = 1e-4)
+        np.testing.assert_allclose(f32_np(c), ref, rtol=1e-4, atol=1e-4 * np.sqrt(K))
+
+
+@pytest.mark.parametrize("algo,M,N,K", [
+    ("tiled", 17, 512, 256), ("tiled", 124, 512, 512), ("tiled", 300, 1040, 1024),
+    ("skinny", 1, 512, 256), ("skinny", 8, 1000, 8192), ("skinny", 17, 512, 256), ("auto", 3000, 512, 512),
+])
+def test_mfma_rowwise_vs_oracle(dev, algo, M, N, K):
+    a, b = synth.random_fp8((M, K), M), synth.random_fp8((N, K), N)
+    sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+    ref = oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), sa.numpy(), sb.numpy(), threads=NT)
+    for out in (torch.float32, torch.bfloat16):
+        c = mm(a, b, sa, sb, ROW, dev, out=out, algo=algo)
+        assert_rel(f32_np(c), ref, TOL, f"rowwise {algo} {M}x{N}x{K} {out}")
+
+
+def test_tensor_scales(dev):
+    cfg = QuantConfig(InputScaleSpec(ScaleGranularity.TENSOR, ScaleOrigin.DYNAMIC, torch.float32),
+                      WeightScaleSpec(ScaleGranularity.TENSOR, torch.float32))
+    a, b = synth.random_fp8((20, 256), 1), synth.random_fp8((144, 256), 2)
+    sa, sb = torch.tensor([[0.031]]), torch.tensor([[0.0047]])
+    ref = oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), sa.numpy(), sb.numpy(), tensor_scales=True)
+    for algo in ("naive", "skinny", "tiled"):
+        assert_rel(f32_np(mm(a, b, sa, sb, cfg, dev, algo=algo)), ref, TOL, algo)
+
+
+def test_pathological_weight_scale_column(dev):
+    # test_scaled_matmul_pathological_bscale.mojo:14-38: a denormal weight scale gives finite ~0
+    a, b = synth.random_fp8((17, 512), 1), synth.random_fp8((64, 512), 2)
+    sa, sb = synth.random_scales((1, 17), 3), synth.random_scales((64, 1), 4)
+    sb[5, 0] = 1e-40
+    for algo in ("skinny", "tiled"):
+        c = f32_np(mm(a, b, sa, sb, ROW, dev, out=torch.bfloat16, algo=algo))
+        assert np.all(np.isfinite(c)) and np.all(np.abs(c[:, 5]) < 1e-30)
+
+
+def test_row_strided_operands(dev):
+    a_wide, b_wide = synth.random_fp8((40, 1024), 1).to(dev), synth.random_fp8((200, 1024), 2).to(dev)
+    a, b = a_wide[:, 256:768], b_wide[:, 512:]
+    sa, sb = synth.random_scales((4, 40), 3), synth.random_scales((2, 4), 4)
+    ref = oracle_block(a.cpu().contiguous(), b.cpu().contiguous(), sa, sb)
+    for algo in ("skinny", "tiled"):
+        assert_rel(f32_np(mm(a, b, sa, sb, BLK, dev, algo=algo)), ref, TOL, algo)
+
+
+def test_empty(dev):
+    a, b, sa, sb = make_block(0, 128, 256, 1)
+    assert tuple(mm(a, b, sa, sb, BLK, dev).shape) == (0, 128)
+
+
+# ---- configuration-sized problems, checked on sampled rows by the naive kernel ----------------
+
+@pytest.mark.parametrize("M,K,N", [
+    (2048, 4096, 6144),     # Llama-3.1-8B QKV
+    (128, 14336, 4096),     # Llama-3.1-8B down, M = 128
+    (1024, 7168, 1536),     # DeepSeek-V3 q_a
+    (256, 7168, 576),       # DeepSeek-V3 kv_a (N not a multiple of 128)
+    (4096, 512, 32768),     # DeepSeek-V3 kv_b
+    (16, 4096, 28672),      # Llama-3.1-8B gate_up, decode-like
+])
+def test_config_shapes_blockwise(dev, M, K, N):
+    x = synth.activations(M, K, seed=0, device=dev)
+    w, sb = synth.quantize_weight_block(synth.weights_f32(N, K, seed=1, device=dev))
+    q, sa = mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32)
+    c = mx.dynamic_scaled_matmul(q, w, sa, sb, BLK.input_scale, BLK.weight_scale)
+    rows = torch.arange(0, M, max(1, M // 24), device=dev)[:24]
+    ref = mx.dynamic_scaled_matmul(q[rows].contiguous(), w, sa[:, rows].contiguous(), sb, BLK.input_scale,
+                                   BLK.weight_scale, out_type=torch.float32, algo="naive")
+    torch.cuda.synchronize()
+    assert_rel(f32_np(c[rows]), f32_np(ref), TOL, f"config {M}x{N}x{K}")
+    # one row against the CPU oracle itself
+    r0 = int(rows[-1])
+    cpu = oracle.matmul_blockwise(fp8_bytes(q[r0:r0 + 1]), fp8_bytes(w), f32_np(sa[:, r0:r0 + 1]), f32_np(sb), threads=NT)
+    assert np.array_equal(f32_np(ref[-1:]), cpu)
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 8192, 10240), (8, 8192, 10240), (4, 28672, 8192), (2, 8192, 57344)])
+def test_config_shapes_decode_rowwise(dev, M, K, N):
+    x = synth.activations(M, K, seed=0, outlier_frac=0.0, device=dev)
+    w, sb = synth.quantize_weight_rowwise(synth.weights_f32(N, K, seed=1, device=dev))
+    q, sa = mx.quantize_dynamic_scaled_float8(x, ROW.input_scale, ROW.weight_scale, scales_type=torch.float32)
+    assert tuple(sa.shape) == (1, M)
+    c = mx.dynamic_scaled_matmul(q, w, sa, sb, ROW.input_scale, ROW.weight_scale)
+    cols = torch.arange(0, N, 37, device=dev)
+    ref = oracle.matmul_rowwise(fp8_bytes(q), fp8_bytes(w[cols]), f32_np(sa), f32_np(sb[cols]), threads=NT)
+    torch.cuda.synchronize()
+    assert_rel(f32_np(c[:, cols]), ref, TOL, f"decode {M}x{N}x{K}")
+    # linearity in the activation scale: doubling a_s doubles C exactly (power of two)
+    c2 = mx.dynamic_scaled_matmul(q, w, sa * 2, sb, ROW.input_scale, ROW.weight_scale)
+    assert torch.equal(c2.float(), c.float() * 2)

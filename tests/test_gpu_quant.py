@@ -1,0 +1,181 @@
+"""GPU parity of the dynamic quantisation kernels against the CPU oracle: bytes and
+scales must be bit-exact (same tests as the reference's
+max/kernels/test/gpu/quantization/test_scaled_fp8_quantization.mojo plus exhaustive
+checks of the hardware convert and of the two f32 divisions)."""
+import numpy as np
+import pytest
+import torch
+
+import modular_amd as mx
+import oracle
+from modular_amd import kernels, synth
+from util import bf16_bits, fp8_bytes, f32_np
+
+pytestmark = pytest.mark.gpu
+BLK, ROW = mx.blockwise_fp8_config(), mx.rowwise_fp8_config()
+NT = oracle.default_threads()
+
+
+def gpu_quant(x, cfg, scales_type=torch.float32, **kw):
+    q, s = mx.quantize_dynamic_scaled_float8(x, cfg.input_scale, cfg.weight_scale, scales_type=scales_type, **kw)
+    torch.cuda.synchronize()
+    return q, s
+
+
+def check(x_cpu, cfg, dev, group, in_dtype=oracle.BF16, **kw):
+    M, K = x_cpu.shape
+    q, s = gpu_quant(x_cpu.to(dev), cfg, **kw)
+    G = K if group == -1 else group
+    src = bf16_bits(x_cpu) if in_dtype == oracle.BF16 else (
+        x_cpu.view(torch.int16).numpy().view(np.uint16) if in_dtype == oracle.F16 else x_cpu.numpy())
+    q_ref, s_ref = oracle.quantize_dynamic_scaled_fp8(src, G, in_dtype=in_dtype, threads=NT,
+                                                      scale_ub=kw.get("scale_ub", 1200.0))
+    assert s.shape[0] == K // G and s.shape[1] >= M
+    assert np.array_equal(f32_np(s)[:, :M].view(np.uint32), s_ref.view(np.uint32)), "scales differ"
+    assert np.array_equal(fp8_bytes(q), q_ref), "quantized bytes differ"
+
+
+def test_hardware_convert_is_the_oracle_encode(dev):
+    rng = np.random.default_rng(0)
+    allbf16 = (np.arange(65536, dtype=np.uint32) << 16).view(np.float32)
+    rnd = rng.integers(0, 2 ** 32, size=1 << 22, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    mags = rng.standard_normal(1 << 22).astype(np.float32) * np.exp2(rng.integers(-14, 9, size=1 << 22)).astype(np.float32)
+    ties = np.concatenate([oracle.e4m3fn_decode_table()[[b for b in range(127)]]] * 1)
+    ties = (ties[:-1] + ties[1:]) / 2  # every midpoint between adjacent codes
+    x = np.concatenate([allbf16, rnd, mags, ties, -ties]).astype(np.float32)
+    x = x[~np.isnan(x)]
+    got = fp8_bytes(kernels.cast_f32_to_e4m3fn(torch.from_numpy(x).to(dev)))
+    want = oracle.e4m3fn_encode(np.clip(x, -448.0, 448.0))
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, [(float(x[i]), int(got[i]), int(want[i])) for i in bad[:8]]
+
+
+def test_hardware_decode_is_the_oracle_decode(dev):
+    codes = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).to(dev)
+    got = f32_np(kernels.cast_e4m3fn_to_f32(codes))
+    want = oracle.e4m3fn_decode_table()
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32)) and np.all(np.isnan(got[~ok]))
+
+
+# test_scaled_fp8_quantization.mojo:707-750
+@pytest.mark.parametrize("M,K", [(1, 256), (2, 1024), (4, 16384), (2, 260), (4, 264), (1, 576), (4, 576)])
+@pytest.mark.parametrize("group", [-1, 128])
+def test_reference_shapes(dev, M, K, group):
+    if group == 128 and K % 128:
+        pytest.skip("group 128 needs K % 128 == 0")
+    g = torch.Generator().manual_seed(M * 100003 + K)
+    x = (torch.rand((M, K), generator=g) * 2 - 1).to(torch.bfloat16)
+    check(x, BLK if group == 128 else ROW, dev, group)
+
+
+def test_every_bf16_amax_divides_exactly(dev):
+    # one group per positive finite bf16 value v: amax = v.  Pins both divisions on the GPU.
+    vals = (np.arange(1, 0x7F80, dtype=np.uint32) << 16).view(np.float32)
+    n = vals.size
+    x = np.zeros((n, 128), dtype=np.float32)
+    x[:, 3] = vals
+    x[:, 77] = -vals * 0.37
+    x[:, 100] = vals * 0.0123
+    pad = (-n) % 3
+    x = np.concatenate([x, np.zeros((pad, 128), dtype=np.float32)])
+    xb = torch.from_numpy(x).to(torch.bfloat16).reshape(-1, 128 * 3)   # three groups per row
+    check(xb.contiguous(), BLK, dev, 128)
+    check(xb.contiguous(), ROW, dev, -1)
+
+
+def test_near_zero_and_zero_groups(dev):
+    # test_scaled_fp8_quantization.mojo:421-512
+    x = torch.full((4, 512), 1e-38, dtype=torch.float32).to(torch.bfloat16)
+    x[:, ::128] = 0.0
+    q, s = gpu_quant(x.to(dev), BLK)
+    assert np.all(fp8_bytes(q) == 0)
+    check(x, BLK, dev, 128)
+    z = torch.zeros((3, 256), dtype=torch.bfloat16)
+    z[1, 130] = -0.0
+    z[2, 5] = 1e-20
+    check(z, BLK, dev, 128)
+    check(z, ROW, dev, -1)
+
+
+def test_scale_ub_and_saturation(dev):
+    x = synth.activations(16, 1024, seed=3).float()
+    x[:, 7] *= 400.0  # well past 1200
+    xb = x.to(torch.bfloat16)
+    check(xb, BLK, dev, 128)
+    check(xb, ROW, dev, -1)
+    check(xb, BLK, dev, 128, scale_ub=3.0)
+
+
+def test_padding_columns_are_never_written(dev):
+    M, K = 81, 2048  # M_pad = 84
+    x = synth.activations(M, K, seed=5).to(dev)
+    sentinel = torch.full((K // 128, 84), float("nan"), device=dev)
+    # the wrapper allocates; call the C ABI directly on a pre-filled buffer
+    from modular_amd import _lib
+    q = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=dev)
+    st = _lib.lib().maxfp8_quantize_dynamic_scaled_fp8(q.data_ptr(), sentinel.data_ptr(), x.data_ptr(), M, K, K, K,
+                                                       128, 84, _lib.BF16, _lib.F32, 1200.0, None)
+    assert st == 0
+    torch.cuda.synchronize()
+    s = f32_np(sentinel)
+    assert np.all(np.isnan(s[:, M:])) and not np.any(np.isnan(s[:, :M]))
+    _, s2 = gpu_quant(x, BLK)
+    assert tuple(s2.shape) == (16, 84)
+
+
+def test_other_dtypes_and_generic_path(dev):
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn((5, 768), generator=g)
+    check(x, BLK, dev, 128, in_dtype=oracle.F32)
+    check(x.to(torch.float16), BLK, dev, 128, in_dtype=oracle.F16)
+    check(x.to(torch.bfloat16), ROW, dev, 64, group_size_or_per_token=64)
+    check(x.to(torch.bfloat16), ROW, dev, 12, group_size_or_per_token=12)   # not a multiple of 8
+    # bf16 scales dtype
+    q, s = gpu_quant(x.to(torch.bfloat16).to(dev), BLK, scales_type=torch.bfloat16)
+    q_ref, s_ref = oracle.quantize_dynamic_scaled_fp8(bf16_bits(x.to(torch.bfloat16)), 128, scales_dtype=oracle.BF16)
+    assert tuple(s.shape) == (6, 8)
+    assert np.array_equal(bf16_bits(s)[:, :5], s_ref) and np.array_equal(fp8_bytes(q), q_ref)
+    # row-strided input (a column slice of a wider matrix)
+    wide = torch.randn((6, 1024), generator=g).to(torch.bfloat16)
+    q, s = gpu_quant(wide.to(dev)[:, 256:768], BLK)
+    q_ref, s_ref = oracle.quantize_dynamic_scaled_fp8(bf16_bits(wide[:, 256:768].contiguous()), 128)
+    assert np.array_equal(fp8_bytes(q), q_ref) and np.array_equal(f32_np(s)[:, :6], s_ref)
+
+
+def test_empty_input(dev):
+    x = torch.zeros((0, 256), dtype=torch.bfloat16, device=dev)
+    q, s = gpu_quant(x, BLK)
+    assert tuple(q.shape) == (0, 256) and tuple(s.shape) == (2, 0)
+
+
+@pytest.mark.parametrize("M,K,cfg,group", [
+    (64, 4096, "blk", 128),        # configs[0]
+    (2048, 14336, "blk", 128),     # Llama-8B down projection input
+    (4096, 7168, "blk", 128),      # DeepSeek-V3 hidden
+    (8, 28672, "row", -1),         # 70B decode, per token
+    (300, 8192, "row", -1),
+    (1, 4096, "blk", 128),
+])
+def test_config_sizes_bit_exact(dev, M, K, cfg, group):
+    x = synth.activations(M, K, seed=0, outlier_frac=0.01 if cfg == "blk" else 0.0)
+    check(x, BLK if cfg == "blk" else ROW, dev, group)
+
+
+def test_moe_size_properties(dev):
+    # 32768 x 7168 (every routed row of the MoE config), generated on the GPU: a slice is
+    # checked bit-exactly against the oracle, the whole against what the arithmetic fixes
+    M, K = 32768, 7168
+    x = synth.activations(M, K, seed=0, device=dev)
+    q, s = gpu_quant(x, BLK)
+    rows = torch.arange(0, M, 257, device=dev)
+    q_ref, s_ref = oracle.quantize_dynamic_scaled_fp8(bf16_bits(x[rows]), 128, threads=NT)
+    assert np.array_equal(fp8_bytes(q[rows]), q_ref)
+    assert np.array_equal(f32_np(s[:, rows]), s_ref)
+    # scale == min(amax, 1200) / 448 and every group holds a +-448 byte unless clamped
+    amax = x.float().reshape(M, K // 128, 128).abs().amax(-1)
+    assert torch.equal(s[:, :M].t(), torch.minimum(amax, torch.tensor(1200.0, device=dev)) / 448.0)
+    mag = (q.view(torch.uint8) & 0x7F).reshape(M, K // 128, 128).amax(-1)
+    assert bool(torch.all(mag[amax > 0] == 0x7E))
+    # idempotence of the byte pattern: dequantise * scale, requantise with the same scales -> same bytes
+    assert not bool(torch.any((q.view(torch.uint8) & 0x7F) == 0x7F))
