@@ -14,7 +14,7 @@ import modular_amd as mx
 import oracle
 from modular_amd import synth
 from modular_amd.quant_config import InputScaleSpec, QuantConfig, ScaleGranularity, ScaleOrigin, WeightScaleSpec
-from util import assert_rel, bf16_bits, f32_np, fp8_bytes, fp8_from_bytes, rel_err
+from util import F32_BUDGET, assert_rel, bf16_bits, f32_np, fp8_bytes, fp8_from_bytes, rel_err
 
 pytestmark = pytest.mark.gpu
 BLK, ROW = mx.blockwise_fp8_config(), mx.rowwise_fp8_config()
@@ -126,10 +126,7 @@ def test_mfma_blockwise_vs_oracle(dev, algo, M, N, K, out):
     a, b, sa, sb = make_block(M, N, K, seed=M + N + K)
     ref = oracle_block(a, b, sa, sb)
     c = mm(a, b, sa, sb, BLK, dev, out=out, algo=algo)
-    assert_rel(f32_np(c), ref, TOL, f"{algo} {M}x{N}x{K} {out}")
-    if out == torch.float32:
-        # reference kernel test tolerance (test_naive_blockwise_fp8_matmul.mojo: atol = rtol = 1e-4)
-        np.testing.assert_allclose(f32_np(c), ref, rtol=1e-4, atol=1e-4 * np.sqrt(K))
+    assert_rel(f32_np(c), ref, TOL, f"{algo} {M}x{N}x{K} {out}", F32_BUDGET if out == torch.float32 else None)
 
 
 @pytest.mark.parametrize("algo,M,N,K", [
@@ -142,7 +139,22 @@ def test_mfma_rowwise_vs_oracle(dev, algo, M, N, K):
     ref = oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), sa.numpy(), sb.numpy(), threads=NT)
     for out in (torch.float32, torch.bfloat16):
         c = mm(a, b, sa, sb, ROW, dev, out=out, algo=algo)
-        assert_rel(f32_np(c), ref, TOL, f"rowwise {algo} {M}x{N}x{K} {out}")
+        assert_rel(f32_np(c), ref, TOL, f"rowwise {algo} {M}x{N}x{K} {out}", F32_BUDGET if out == torch.float32 else None)
+
+
+def test_mfma_keeps_13_bits_below_the_largest_product(dev):
+    # Known answer that documents the hardware: 448*448 + 1*1 = 200705 is an exact f32, the
+    # scalar kernel returns it, the matrix instruction drops the 1 (truncation inside the
+    # instruction, not in this library's code).  The loss is bounded by 2^-12 of the largest product.
+    a = torch.zeros((16, 128), dtype=torch.float32)
+    b = torch.zeros((16, 128), dtype=torch.float32)
+    a[:, 0], b[:, 0], a[:, 1], b[:, 1] = 448.0, 448.0, 1.0, 1.0
+    a8, b8 = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
+    one = torch.ones((1, 16))
+    assert float(mm(a8, b8, one, one[:, :1], BLK, dev, algo="naive")[0, 0]) == 200705.0
+    for algo in ("tiled", "skinny"):
+        got = float(mm(a8, b8, one, one[:, :1], BLK, dev, algo=algo)[0, 0])
+        assert 200704.0 <= got <= 200705.0 and abs(got - 200705.0) <= 200704.0 * 2.0 ** -12, got
 
 
 def test_tensor_scales(dev):
@@ -152,7 +164,7 @@ def test_tensor_scales(dev):
     sa, sb = torch.tensor([[0.031]]), torch.tensor([[0.0047]])
     ref = oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), sa.numpy(), sb.numpy(), tensor_scales=True)
     for algo in ("naive", "skinny", "tiled"):
-        assert_rel(f32_np(mm(a, b, sa, sb, cfg, dev, algo=algo)), ref, TOL, algo)
+        assert_rel(f32_np(mm(a, b, sa, sb, cfg, dev, algo=algo)), ref, TOL, algo, F32_BUDGET)
 
 
 def test_pathological_weight_scale_column(dev):
@@ -171,7 +183,7 @@ def test_row_strided_operands(dev):
     sa, sb = synth.random_scales((4, 40), 3), synth.random_scales((2, 4), 4)
     ref = oracle_block(a.cpu().contiguous(), b.cpu().contiguous(), sa, sb)
     for algo in ("skinny", "tiled"):
-        assert_rel(f32_np(mm(a, b, sa, sb, BLK, dev, algo=algo)), ref, TOL, algo)
+        assert_rel(f32_np(mm(a, b, sa, sb, BLK, dev, algo=algo)), ref, TOL, algo, F32_BUDGET)
 
 
 def test_empty(dev):

@@ -174,7 +174,8 @@ def test_moe_size_properties(dev):
     assert np.array_equal(f32_np(s[:, rows]), s_ref)
     # scale == min(amax, 1200) / 448 and every group holds a +-448 byte unless clamped
     amax = x.float().reshape(M, K // 128, 128).abs().amax(-1)
-    assert torch.equal(s[:, :M].t(), torch.minimum(amax, torch.tensor(1200.0, device=dev)) / 448.0)
+    # (the division is done on the CPU: it must be the correctly rounded IEEE quotient)
+    assert torch.equal(s[:, :M].t().cpu(), torch.minimum(amax.cpu(), torch.tensor(1200.0)) / 448.0)
     mag = (q.view(torch.uint8) & 0x7F).reshape(M, K // 128, 128).amax(-1)
     assert bool(torch.all(mag[amax > 0] == 0x7E))
     # idempotence of the byte pattern: dequantise * scale, requantise with the same scales -> same bytes
