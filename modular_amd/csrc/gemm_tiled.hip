@@ -1,79 +1,91 @@
 // LDS-staged MFMA GEMM for scaled FP8 on gfx950:  C[M,N] = A[M,K] . B[N,K]^T.
 //
-// One block owns a BM x BN tile of C and walks K in slabs of 128 bytes (one scale
-// group).  Per slab the block copies BM + BN rows of 128 fp8 bytes into LDS
-// (16-byte chunks, chunk index XOR-swizzled with (row >> 1) & 7 so that the
-// 16-lane MFMA fragment reads hit 64 distinct banks), and every wave issues
-// v_mfma_f32_16x16x128_f8f6f4 on its (BM/WAVES_M) x (BN/WAVES_N) sub-tile.
+// One block owns a BM x BN tile of C and walks K in slabs of 128 bytes (one scale group).
 //
-// The weight fragment is the MFMA's row operand and the activation fragment its
-// column operand, so a lane ends up with 4 consecutive n for ONE m: the
-// per-token scale is a single register per 16-row group and the bf16 results
-// leave as 8-byte stores.
+//   * global -> LDS copies are `buffer_load_dwordx4 ... lds` (LDS DMA): no staging registers,
+//     no ds_write.  A wave-instruction moves 8 tile rows x 128 bytes; lane (r = lane >> 3,
+//     p = lane & 7) fetches the logical 16-byte chunk p ^ (row & 7) of its row, so the bytes
+//     land in LDS already swizzled for conflict-free MFMA fragment reads.  Rows past the tile
+//     edge read as zero through the buffer descriptor, so partial tiles need no branches.
+//   * NS LDS stages (2 or 3), one barrier per slab, DMA issued NS-1 slabs ahead.
+//   * every wave issues v_mfma_f32_16x16x128_f8f6f4 on its (BM/WAVES_M) x (BN/WAVES_N)
+//     sub-tile.  The weight fragment is the MFMA's row operand and the activation fragment its
+//     column operand, so a lane ends up with 4 consecutive n for ONE m: the per-token scale is
+//     a single register per 16-row group and bf16 results leave as 8-byte stores.  Weight
+//     fragments of the slab stay in registers; activation fragments stream 16 rows at a time,
+//     one step ahead of the MFMAs that use them.
 //
-// Block scaling (1x128 activation groups, 128x128 weight blocks): each slab's
-// product is formed in a fresh accumulator P (MFMA with C = 0) and promoted with
+// Block scaling (1x128 activation groups, 128x128 weight blocks): each slab's product is formed
+// in a fresh accumulator P (MFMA with C = 0) and promoted with
 // acc += P * (a_s[slab, m] * b_s[n/128, slab]) -- the per-slab promotion of
-// max/kernels/src/linalg/matmul/gpu/sm100/blockwise_fp8.mojo:376-392, which sums
-// the same terms as the reference's naive kernel
-// (max/kernels/src/linalg/fp8_quantization.mojo:1576-1624) in a different order.
-// Row/tensor scaling: acc accumulates over all of K inside the MFMA and is scaled
-// once, (acc * a_s[m]) * b_s[n]  (fp8_quantization.mojo:1218-1240).
+// max/kernels/src/linalg/matmul/gpu/sm100/blockwise_fp8.mojo:376-392, which sums the same terms
+// as the reference's naive kernel (max/kernels/src/linalg/fp8_quantization.mojo:1576-1624) in a
+// different order.  The slab's activation scales travel through LDS with the tile (one more
+// LDS-DMA instruction per wave).  Row/tensor scaling: acc accumulates over all of K inside the
+// MFMA and is scaled once, (acc * a_s[m]) * b_s[n]  (fp8_quantization.mojo:1218-1240).
 //
-// Grouped (MoE) mode maps blocks to (expert slot, m-tile, n-tile) from the
-// device-resident offsets, so no host synchronisation is needed
+// Grouped (MoE) mode maps blocks to (expert slot, m-tile, n-tile) from the device-resident
+// offsets with a block-wide prefix sum, so no host synchronisation is needed
 // (semantics: fp8_quantization.mojo:1745-1865).
+//
+// Why the tiles are what they are (measured on MI355X): LDS serves ~128 B/clk/CU to
+// ds_read_b128 and LDS-DMA together, the L1 -> LDS path ~50 B/clk/CU, and an MFMA retires in
+// 32 clocks per SIMD, so a 64 x 64 wave tile is LDS-bound at two thirds of the MFMA rate and a
+// 128 x 64 wave tile is balanced.  Accumulators must be ordinary VGPRs for the promotion, which
+// caps the wave tile at 128 x 64 with two waves per SIMD.
+#include <stdlib.h>
+
 #include "common.h"
 #include "gemm_args.h"
 
 namespace maxfp8 {
 
-// raw buffer descriptor: out-of-range offsets read as zero, which handles the
-// M and N edges of partial tiles.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t t2_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
-
-__device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff) {
-  return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
-}
-
-__device__ __forceinline__ uint32_t clamp_u32(int64_t v) {
+__device__ __forceinline__ uint32_t t2_clamp_u32(int64_t v) {
   return v > 0xfffffff0ll ? 0xfffffff0u : (v < 0 ? 0u : (uint32_t)v);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE, bool GROUPED>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (BM * BN <= 128 * 128) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
-  constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmArgs p) {
+  constexpr int NWAVES = WAVES_M * WAVES_N;
+  constexpr int NTHREADS = NWAVES * 64;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 16, TN = WN / 16;
-  constexpr int CA = BM * 8 / NTHREADS, CB = BN * 8 / NTHREADS;
-  constexpr int STAGE_BYTES = (BM + BN) * 128;
-  static_assert(CA >= 1 && CB >= 1, "tile too small for the block");
+  constexpr int IA = BM / 8 / NWAVES, IB = BN / 8 / NWAVES;  // LDS-DMA instructions per wave and slab
+  // one stage: A rows, B rows, then (block scaling) the slab's BM activation scales
+  constexpr int SCALE_BYTES = BLOCKSCALE ? BM * 4 : 0;
+  constexpr int STAGE_BYTES = (BM + BN) * 128 + SCALE_BYTES;
+  constexpr int PER = IA + IB + (BLOCKSCALE ? 1 : 0);  // LDS-DMA instructions per wave and slab
+  static_assert(NWAVES % 2 == 0 && IA >= 1 && IB >= 1, "tile / wave layout");
+  static_assert(NS == 2 || NS == 3, "two or three LDS stages");
+  static_assert(!BLOCKSCALE || BM % 64 == 0, "scale rows are copied 64 at a time");
   static_assert(!BLOCKSCALE || (WN <= 128 && 128 % WN == 0), "a wave's columns must sit inside one 128-wide scale block");
 
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-  // ---- block -> tile --------------------------------------------------------
-  int64_t row_begin, row_end;  // rows of A/C this block may touch: [row_begin, row_end)
+  // ---- block -> tile ----------------------------------------------------------------
+  int64_t row_begin, row_end;
   int n0;
   const uint8_t* bptr = p.b;
   const float* bs_ptr = p.b_scales;
   bool zero_fill = false;
   if constexpr (GROUPED) {
-    // blockIdx.y walks the m-tiles of all active slots in slot order: a block-wide
-    // prefix sum over the slots' tile counts locates (slot, tile) without the host.
-    __shared__ int s_slot, s_tile, s_wave_sum[NTHREADS / 64], s_carry;
+    __shared__ int s_slot, s_tile, s_wave_sum[NWAVES], s_carry;
     if (tid == 0) { s_slot = -1; s_tile = 0; s_carry = 0; }
     __syncthreads();
     for (int z0 = 0; z0 < p.num_active; z0 += NTHREADS) {
       const int z = z0 + tid;
       int t = 0;
       if (z < p.num_active) t = ((int)(p.offsets[z + 1] - p.offsets[z]) + BM - 1) / BM;
-      int incl = t;  // inclusive scan inside the wave
+      int incl = t;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
         const int up = __shfl_up(incl, o, 64);
@@ -102,9 +114,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (BM * BN <= 128 * 128) ? 2 :
       bs_ptr += (int64_t)e * p.bs_expert_stride;
     }
   } else {
-    // 1-D grid.  Consecutive block ids land on different XCDs (8 of them, each
-    // with its own L2), so give each XCD a contiguous run of tiles, and walk the
-    // tiles in column-major groups of GROUP_M rows for L2 reuse of A and B.
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     const int total = tiles_m * tiles_n;
     int pid = blockIdx.x;
@@ -113,7 +122,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (BM * BN <= 128 * 128) ? 2 :
       const int base = total >> 3, rem = total & 7;
       pid = xcd * base + (xcd < rem ? xcd : rem) + local;
     }
-    constexpr int GROUP_M = 8;
+    constexpr int GROUP_M = 4;
     const int per_group = GROUP_M * tiles_n;
     const int group = pid / per_group;
     const int first_m = group * GROUP_M;
@@ -128,10 +137,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (BM * BN <= 128 * 128) ? 2 :
   const int rows_here = (int)((row_end - row_begin) < BM ? (row_end - row_begin) : BM);
   const int cols_here = (p.N - n0) < BN ? (p.N - n0) : BN;
 
-  // ---- epilogue helpers --------------------------------------------------------
   const int lm = lane & 15, lq = lane >> 4;
   auto store4 = [&](int64_t m, int n, float v0, float v1, float v2, float v3) {
-    // caller guarantees m is valid; n..n+3 may cross N
     if (p.c_dtype == MAXFP8_BF16) {
       uint16_t* dst = reinterpret_cast<uint16_t*>(p.c) + m * p.ldc + n;
       if (p.c_vec_ok && n + 3 < p.N) {
@@ -171,48 +178,68 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (BM * BN <= 128 * 128) ? 2 :
     return;
   }
 
-  // ---- global -> LDS copy plan ---------------------------------------------------
-  // chunk q = tid + i*NTHREADS: row q>>3 of the tile, 16-byte chunk q&7 of the slab.
+  // ---- global -> LDS copy plan (LDS DMA) ------------------------------------------------
   const uint8_t* a_tile = p.a + row_begin * p.lda;
   const uint8_t* b_tile = bptr + (int64_t)n0 * p.ldb;
-  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_tile, clamp_u32((int64_t)(rows_here - 1) * p.lda + p.K));
-  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_tile, clamp_u32((int64_t)(cols_here - 1) * p.ldb + p.K));
-  const int crow = tid >> 3, cchunk = tid & 7;
-  constexpr int ROWS_PER_PASS = NTHREADS / 8;
-  const uint32_t a_voff = (uint32_t)crow * (uint32_t)p.lda + cchunk * 16;
-  const uint32_t b_voff = (uint32_t)crow * (uint32_t)p.ldb + cchunk * 16;
-  const uint32_t a_step = (uint32_t)ROWS_PER_PASS * (uint32_t)p.lda;
-  const uint32_t b_step = (uint32_t)ROWS_PER_PASS * (uint32_t)p.ldb;
-  // ROWS_PER_PASS is a multiple of 16, so the swizzle term does not depend on i
-  const uint32_t lds_wr = crow * 128 + ((cchunk ^ ((crow >> 1) & 7)) << 4);
+  const __amdgpu_buffer_rsrc_t a_rsrc = t2_rsrc(a_tile, t2_clamp_u32((int64_t)(rows_here - 1) * p.lda + p.K));
+  const __amdgpu_buffer_rsrc_t b_rsrc = t2_rsrc(b_tile, t2_clamp_u32((int64_t)(cols_here - 1) * p.ldb + p.K));
+  const int cr = lane >> 3, cp = lane & 7;
+  // tile row of instruction i is (i*NWAVES + wave)*8 + cr, so row & 7 == cr
+  const int cchunk = cp ^ cr;
+  const uint32_t a_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.lda + cchunk * 16;
+  const uint32_t b_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.ldb + cchunk * 16;
+  const uint32_t a_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.lda;
+  const uint32_t b_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.ldb;
   const bool k_tail = (p.K & 127) != 0;
+  const int nslab = (p.K + 127) / 128;
+  // activation scales of the tile: element (slab, row_begin + r); rows past the tile read as 0
+  const int s_chunk = wave % (BM / 64);
+  __amdgpu_buffer_rsrc_t s_rsrc = t2_rsrc(nullptr, 0);
+  uint32_t s_voff = 0, s_slab_step = 0;
+  if constexpr (BLOCKSCALE) {
+    s_rsrc = t2_rsrc(p.a_scales + row_begin, t2_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + rows_here) * 4));
+    const int r = s_chunk * 64 + lane;
+    s_voff = r < rows_here ? (uint32_t)r * 4u : 0x80000000u;
+    s_slab_step = (uint32_t)p.a_scales_ld * 4u;
+  }
 
-  v4i ra[CA], rb[CB];
-  auto gload = [&](int slab) {
-    uint32_t koff = (uint32_t)slab * 128u;
+  auto dma = [&](int slab, int buf) {
+    const uint32_t koff = (uint32_t)slab * 128u;
     uint32_t kill = 0;
-    if (k_tail && koff + cchunk * 16 >= (uint32_t)p.K) kill = 0x80000000u;  // past K: force out of range
-#pragma unroll
-    for (int i = 0; i < CA; ++i) ra[i] = buffer_load16(a_rsrc, (a_voff + i * a_step + koff) | kill);
-#pragma unroll
-    for (int i = 0; i < CB; ++i) rb[i] = buffer_load16(b_rsrc, (b_voff + i * b_step + koff) | kill);
-  };
-  auto sstore = [&](int buf) {
-    uint8_t* sa = smem + buf * STAGE_BYTES;
+    if (k_tail && koff + cchunk * 16 >= (uint32_t)p.K) kill = 0x80000000u;
+    uint8_t* sa = smem + buf * STAGE_BYTES + wave * 1024;
     uint8_t* sb = sa + BM * 128;
 #pragma unroll
-    for (int i = 0; i < CA; ++i) *reinterpret_cast<v4i*>(sa + lds_wr + i * ROWS_PER_PASS * 128) = ra[i];
+    for (int i = 0; i < IA; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(sa + i * NWAVES * 1024), 16, a_voff | kill,
+                                               koff + i * a_istep, 0, 0);
 #pragma unroll
-    for (int i = 0; i < CB; ++i) *reinterpret_cast<v4i*>(sb + lds_wr + i * ROWS_PER_PASS * 128) = rb[i];
+    for (int i = 0; i < IB; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(sb + i * NWAVES * 1024), 16, b_voff | kill,
+                                               koff + i * b_istep, 0, 0);
+    if constexpr (BLOCKSCALE) {
+      // 64 scales of the slab's row of the transposed scale matrix per wave; with more waves
+      // than 64-row chunks the extra waves repeat a chunk (same bytes to the same place), so
+      // every wave issues the same number of DMA instructions per slab.
+      uint8_t* ss = smem + buf * STAGE_BYTES + (BM + BN) * 128 + s_chunk * 256;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(s_rsrc, (lds_ptr_t)ss, 4, s_voff, (uint32_t)slab * s_slab_step, 0, 0);
+    }
   };
 
-  // ---- fragment read plan ----------------------------------------------------------
-  // lane (lm, lq) reads row lm of a 16-row group, logical chunks 2*lq and 2*lq+1.
-  const int sw = (lm >> 1) & 7;
-  const uint32_t frag0 = lm * 128 + (((2 * lq) ^ sw) << 4);
-  const uint32_t frag1 = lm * 128 + (((2 * lq + 1) ^ sw) << 4);
+  // ---- fragment read plan -------------------------------------------------------------------
+  // lane (lm, lq) holds K bytes [16*lq, +16) and [64 + 16*lq, +16) of row lm: logical chunks
+  // lq and lq + 4, stored at chunk ^ (row & 7).  (Both MFMA operands use the same K order,
+  // which is all the dot product needs; measured conflict-free, unlike chunks 2*lq, 2*lq+1.)
+  const int sw = lm & 7;
+  const uint32_t frag0 = lm * 128 + ((lq ^ sw) << 4);
+  const uint32_t frag1 = lm * 128 + (((lq + 4) ^ sw) << 4);
   const uint32_t a_frag_base = (uint32_t)(wm * WM) * 128;
   const uint32_t b_frag_base = (uint32_t)(BM + wn * WN) * 128;
+  auto read_frag = [&](const uint8_t* base) -> v8i {
+    const v4i lo = *reinterpret_cast<const v4i*>(base + frag0);
+    const v4i hi = *reinterpret_cast<const v4i*>(base + frag1);
+    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
 
   v4f acc[TM][TN];
 #pragma unroll
@@ -220,78 +247,70 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (BM * BN <= 128 * 128) ? 2 :
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  const int nslab = (p.K + 127) / 128;
-
-  // per-slab scales: a_s for this lane's TM rows, b_s for the wave's 128-block
-  float as_cur[TM], as_nxt[TM];
-  float bs_cur = 1.f, bs_nxt = 1.f;
-  int64_t as_col[TM];
   const float* bs_row = nullptr;
-  if constexpr (BLOCKSCALE) {
-#pragma unroll
-    for (int mt = 0; mt < TM; ++mt) {
-      int ml = wm * WM + mt * 16 + lm;
-      if (ml >= rows_here) ml = rows_here - 1;  // stay inside the scale matrix
-      as_col[mt] = row_begin + ml;
-    }
-    bs_row = bs_ptr + (int64_t)((n0 + wn * WN) / 128) * p.b_scales_ld;
-#pragma unroll
-    for (int mt = 0; mt < TM; ++mt) as_nxt[mt] = p.a_scales[as_col[mt]];
-    bs_nxt = bs_row[0];
-  }
+  if constexpr (BLOCKSCALE) bs_row = bs_ptr + (int64_t)((n0 + wn * WN) / 128) * p.b_scales_ld;
+  const uint32_t s_rd = (uint32_t)((BM + BN) * 128 + (wm * WM + lm) * 4);
 
-  gload(0);
-  sstore(0);
-  __syncthreads();
+  // NS LDS stages, one barrier per slab, DMA issued NS-1 slabs ahead.  At the top of slab j a
+  // wave waits until its own DMA of slab j has landed (the younger ones may stay in flight:
+  // LDS-DMA is the only VMEM traffic of the loop, so the count is exact), then the barrier makes
+  // every wave's part of slab j visible and proves that slab j-1's buffer is no longer read, and
+  // the DMA of slab j+NS-1 is sent into that buffer.
+#pragma unroll
+  for (int st = 0; st < NS - 1; ++st)
+    if (st < nslab) dma(st, st);
 
+  // the weight-block scale of the NEXT slab is fetched before this slab's DMA is issued, so
+  // that waiting for it never waits for the youngest DMA
+  float bs_nxt = 1.f;
+  if constexpr (BLOCKSCALE) bs_nxt = bs_row[0];
+
+  int buf = 0;
   for (int slab = 0; slab < nslab; ++slab) {
-    const int buf = slab & 1;
-    const bool more = slab + 1 < nslab;
-    if (more) gload(slab + 1);
-    if constexpr (BLOCKSCALE) {
-#pragma unroll
-      for (int mt = 0; mt < TM; ++mt) as_cur[mt] = as_nxt[mt] * bs_nxt;
-      bs_cur = bs_nxt;
-      (void)bs_cur;
-      if (more) {
-#pragma unroll
-        for (int mt = 0; mt < TM; ++mt) as_nxt[mt] = p.a_scales[(int64_t)(slab + 1) * p.a_scales_ld + as_col[mt]];
-        bs_nxt = bs_row[slab + 1];
-      }
+    if (NS == 3 && slab + 1 < nslab) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const float bs = bs_nxt;
+    if constexpr (BLOCKSCALE) {
+      if (slab + 1 < nslab) bs_nxt = bs_row[slab + 1];
+    }
+    asm volatile("" ::: "memory");
+    if (slab + NS - 1 < nslab) dma(slab + NS - 1, buf == 0 ? NS - 1 : buf - 1);
 
     const uint8_t* sa = smem + buf * STAGE_BYTES;
-    v8i af[TM], bf[TN];
+    float s_cur[TM];
+    if constexpr (BLOCKSCALE) {
 #pragma unroll
-    for (int t = 0; t < TM; ++t) {
-      const v4i lo = *reinterpret_cast<const v4i*>(sa + a_frag_base + t * 2048 + frag0);
-      const v4i hi = *reinterpret_cast<const v4i*>(sa + a_frag_base + t * 2048 + frag1);
-      af[t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      for (int mt = 0; mt < TM; ++mt) s_cur[mt] = *reinterpret_cast<const float*>(sa + s_rd + mt * 64) * bs;
     }
+    v8i bf[TN];
 #pragma unroll
-    for (int t = 0; t < TN; ++t) {
-      const v4i lo = *reinterpret_cast<const v4i*>(sa + b_frag_base + t * 2048 + frag0);
-      const v4i hi = *reinterpret_cast<const v4i*>(sa + b_frag_base + t * 2048 + frag1);
-      bf[t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    }
+    for (int t = 0; t < TN; ++t) bf[t] = read_frag(sa + b_frag_base + t * 2048);
+    v8i af = read_frag(sa + a_frag_base);
 #pragma unroll
-    for (int nt = 0; nt < TN; ++nt) {
+    for (int mt = 0; mt < TM; ++mt) {
+      v8i af_next = af;
+      if (mt + 1 < TM) af_next = read_frag(sa + a_frag_base + (mt + 1) * 2048);
 #pragma unroll
-      for (int mt = 0; mt < TM; ++mt) {
+      for (int nt = 0; nt < TN; ++nt) {
         if constexpr (BLOCKSCALE) {
           const v4f zero = {0.f, 0.f, 0.f, 0.f};
-          const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af[mt], zero, 0, 0, 0, 0, 0, 0);
-          acc[mt][nt] += part * as_cur[mt];
+          const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
+          acc[mt][nt] += part * s_cur[mt];
         } else {
-          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af[mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
+          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
         }
       }
+      af = af_next;
     }
-    if (more) sstore(buf ^ 1);
-    __syncthreads();
+    buf = buf + 1 == NS ? 0 : buf + 1;
   }
 
-  // ---- epilogue ------------------------------------------------------------------
+  // ---- epilogue -----------------------------------------------------------------------------
 #pragma unroll
   for (int mt = 0; mt < TM; ++mt) {
     const int ml = wm * WM + mt * 16 + lm;
@@ -317,11 +336,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (BM * BN <= 128 * 128) ? 2 :
   }
 }
 
-// ---------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE, bool GROUPED>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED>
 static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
-  constexpr int smem = 2 * (BM + BN) * 128;
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE, GROUPED>;
+  constexpr int smem = NS * ((BM + BN) * 128 + (BLOCKSCALE ? BM * 4 : 0));
+  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, GROUPED>;
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -332,20 +350,62 @@ static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const 
   return launch_status(name);
 }
 
+// ---- kernel selection ------------------------------------------------------------------------
+// Three tile shapes.  `t_slab` is the measured time one block spends per 128-byte K slab when
+// the whole chip is busy (microseconds); the cost of a shape is rounds * t_slab, with
+// rounds = ceil(tiles / resident blocks).
+struct TileShape { int bm, bn, slots; float t_slab_block, t_slab_row; };
+static const TileShape kShapes[3] = {
+    {256, 256, 256, 2.05f, 1.70f},   // 8 waves, 2 stages
+    {256, 128, 256, 1.10f, 1.00f},   // 8 waves, 3 stages
+    {128, 128, 512, 1.20f, 1.05f},   // 4 waves, 2 stages, two blocks per CU
+};
+
+// MAXFP8_TILE=1/2/3 forces a shape (for tuning runs); anything else lets the cost model pick.
+static int tile_override() {
+  const char* e = getenv("MAXFP8_TILE");
+  const int v = e ? atoi(e) : 0;
+  return (v >= 1 && v <= 3) ? v : 0;
+}
+
+static int pick_shape(int64_t M, int64_t N, bool blockscale) {
+  int best = 0;
+  float best_cost = 0.f;
+  for (int i = 0; i < 3; ++i) {
+    const TileShape& t = kShapes[i];
+    const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+    const float cost = (float)ceil_div(tiles, t.slots) * (blockscale ? t.t_slab_block : t.t_slab_row);
+    if (i == 0 || cost < best_cost) { best = i; best_cost = cost; }
+  }
+  return best + 1;
+}
+
 int gemm_tiled_dispatch(const GemmArgs& p, bool blockscale, hipStream_t stream) {
-  const int64_t tiles = ceil_div(p.M, 128) * ceil_div(p.N, 128);
+  int variant = tile_override();
+  if (!variant) variant = pick_shape(p.M, p.N, blockscale);
+  const TileShape& t = kShapes[variant - 1];
+  const int64_t tiles = ceil_div(p.M, t.bm) * ceil_div(p.N, t.bn);
   if (tiles >= ((int64_t)1 << 31)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "tiled matmul: too many tiles");
   const dim3 grid((unsigned)tiles);
-  if (blockscale) return launch_tiled<128, 128, 2, 2, true, false>(p, grid, stream, "gemm_tiled_block");
-  return launch_tiled<128, 128, 2, 2, false, false>(p, grid, stream, "gemm_tiled_row");
+  if (blockscale) {
+    if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, true, false>(p, grid, stream, "gemm_tiled_block_256x256");
+    if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, true, false>(p, grid, stream, "gemm_tiled_block_256x128");
+    return launch_tiled<128, 128, 2, 2, 2, true, false>(p, grid, stream, "gemm_tiled_block_128x128");
+  }
+  if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false, false>(p, grid, stream, "gemm_tiled_row_256x256");
+  if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, false, false>(p, grid, stream, "gemm_tiled_row_256x128");
+  return launch_tiled<128, 128, 2, 2, 2, false, false>(p, grid, stream, "gemm_tiled_row_128x128");
 }
 
 int gemm_grouped_dispatch(const GemmArgs& p, int64_t T, hipStream_t stream) {
-  // every active slot owns at most ceil(cnt/128) m-tiles: sum <= T/128 + num_active
-  const int64_t m_tiles = T / 128 + p.num_active;
+  // every active slot owns at most ceil(rows / BM) m-tiles: their sum is <= T / BM + num_active
+  const bool big = tile_override() == 2;
+  const int bm = big ? 256 : 128;
+  const int64_t m_tiles = T / bm + p.num_active;
   if (m_tiles > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: %lld row tiles exceed the launch limit", (long long)m_tiles);
   const dim3 grid((unsigned)ceil_div(p.N, 128), (unsigned)m_tiles);
-  return launch_tiled<128, 128, 2, 2, true, true>(p, grid, stream, "gemm_grouped_block");
+  if (big) return launch_tiled<256, 128, 4, 2, 3, true, true>(p, grid, stream, "gemm_grouped_block_256x128");
+  return launch_tiled<128, 128, 2, 2, 2, true, true>(p, grid, stream, "gemm_grouped_block_128x128");
 }
 
 }  // namespace maxfp8
