@@ -21,7 +21,7 @@ SOURCES = ["api.hip", "quant.hip", "naive.hip", "gemm_tiled.hip", "gemm_skinny.h
 
 # packed-fp32 VALU ops are switched off for every kernel (they are not used by hand either)
 COMMON = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]

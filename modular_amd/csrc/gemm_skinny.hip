@@ -1,40 +1,76 @@
 // Weight-streaming scaled FP8 matmul for small M (decode): C[M,N] = A[M,K] . B[N,K]^T,
 // M <= 16 * MT.
 //
-// The bytes that matter are the N*K weight bytes, read exactly once.  A block owns
-// 16*NTW consecutive weight rows; its 4 waves take the 128-byte K slabs round-robin
-// (so the block reads 512 contiguous bytes of every row per step).  A lane loads 32
-// bytes of one weight row per slab straight into the MFMA row-operand registers
-// (no LDS staging: nothing is reused), the activations are the MFMA column operand
-// (tokens >= M read as zero through the buffer descriptor), and
-// v_mfma_f32_16x16x128_f8f6f4 does the dot products: 16 weight rows x 16 token
-// columns per instruction, so no M-padding to a 128-row tile.  Partial sums of the
-// 4 waves meet in LDS; wave-ordered summation keeps the result deterministic.
+// The bytes that matter are the N*K weight bytes, read exactly once, so the kernel is
+// shaped by what HBM likes (measured on MI355X with read-only kernels: whole 128-byte lines
+// per row and long runs per wave reach ~6.2 TB/s on these shapes; half lines taken by
+// alternating waves stay at ~4.6 TB/s):
+//
+//   * a block owns 16*NTW consecutive weight rows; each of its 4 or 8 waves owns a contiguous
+//     share of K and walks it in 128-byte slabs;
+//   * weight slabs travel by LDS-DMA (`buffer_load_dwordx4 ... lds`), one instruction per
+//     8 rows x 128 bytes (whole cache lines), into a ring of DEPTH slots that is private to
+//     the wave -- no barrier in the loop, DEPTH slabs of weights in flight per wave;
+//   * the MFMA row operand (16 weight rows x 128 K bytes) is read back from LDS with the
+//     same conflict-free chunk swizzle as the tiled kernel; the activations are the column
+//     operand, loaded straight from global memory / L2 (tokens >= M read as zero through the
+//     buffer descriptor): v_mfma_f32_16x16x128_f8f6f4 computes 16 weight rows x 16 tokens
+//     per instruction, so M is never padded to a 128-row tile;
+//   * the waves' partial sums meet in LDS in a fixed order (deterministic result).
 //
 // Scaling follows gemm_tiled.hip: block mode promotes every slab with
 // a_s[slab, m] * b_s[n/128, slab]; row/tensor mode scales once at the end
 // (max/kernels/src/linalg/fp8_quantization.mojo:1218-1240, 1576-1624).
+#include <stdlib.h>
+
+#include <type_traits>
+#include <utility>
+
 #include "common.h"
 #include "gemm_args.h"
 
 namespace maxfp8 {
 
+typedef __attribute__((address_space(3))) void* sk_lds_ptr_t;
+
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t sk_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
-__device__ __forceinline__ v4i sk_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff) {
-  return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+__device__ __forceinline__ v4i sk_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ float sk_load_f32(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
 }
 __device__ __forceinline__ uint32_t sk_clamp_u32(int64_t v) {
   return v > 0xfffffff0ll ? 0xfffffff0u : (v < 0 ? 0u : (uint32_t)v);
 }
 
-template <int NTW, int MT, bool BLOCKSCALE>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(GemmArgs p) {
-  constexpr int WAVES = 4;
-  __shared__ float red[WAVES][MT * NTW * 4][64];
+template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
+struct SkinnyCfg {
+  static constexpr int WAVES = NWAVES;
+  static constexpr int SLOT = NTW * 2048;                    // one slab of the block's rows
+  // VMEM instructions a wave issues per slab, in this order: activations, scales, weight DMA
+  static constexpr int PER = 2 * MT + (BLOCKSCALE ? MT + 1 : 0) + 2 * NTW;
+  // slabs in flight per wave: RING_KB of weights, limited by the 6-bit vmcnt counter and by the
+  // registers the activation fragments of the in-flight slabs take (96)
+  static constexpr int D_BYTES = RING_KB * 1024 / SLOT, D_CNT = 63 / PER + 1, D_REGS = 96 / (MT * 8);
+  static constexpr int D_MIN = D_BYTES < D_CNT ? (D_BYTES < D_REGS ? D_BYTES : D_REGS) : (D_CNT < D_REGS ? D_CNT : D_REGS);
+  static constexpr int DEPTH = D_MIN < 2 ? 2 : D_MIN;
+  static constexpr int RING = DEPTH * SLOT;                  // per wave
+  static constexpr int RED = WAVES * MT * NTW * 4 * 64 * 4;  // reduction buffer (reuses the rings)
+  static constexpr int SMEM = WAVES * RING > RED ? WAVES * RING : RED;
+};
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
+__global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p) {
+  using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
+  constexpr int WAVES = Cfg::WAVES, DEPTH = Cfg::DEPTH, SLOT = Cfg::SLOT, PER = Cfg::PER;
+  static_assert((DEPTH - 1) * PER < 64, "vmcnt is a 6-bit counter");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lm = lane & 15, lq = lane >> 4;
   const int n0 = blockIdx.x * (16 * NTW);
   const int cols_here = (p.N - n0) < 16 * NTW ? (p.N - n0) : 16 * NTW;
@@ -43,15 +79,40 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(GemmArgs p) {
   const __amdgpu_buffer_rsrc_t b_rsrc = sk_rsrc(b_tile, sk_clamp_u32((int64_t)(cols_here - 1) * p.ldb + p.K));
   const __amdgpu_buffer_rsrc_t a_rsrc = sk_rsrc(p.a, sk_clamp_u32((int64_t)(p.M - 1) * p.lda + p.K));
 
-  // lane's two 16-byte chunks of a slab: bytes [16*lq, +16) and [64 + 16*lq, +16)
-  uint32_t b_off[NTW], a_off[MT];
-#pragma unroll
-  for (int t = 0; t < NTW; ++t) b_off[t] = (uint32_t)(t * 16 + lm) * (uint32_t)p.ldb + lq * 16;
-#pragma unroll
-  for (int t = 0; t < MT; ++t) a_off[t] = (uint32_t)(t * 16 + lm) * (uint32_t)p.lda + lq * 16;
-
   const int nslab = (p.K + 127) / 128;
   const bool k_tail = (p.K & 127) != 0;
+  // this wave's slabs: [s_begin, s_end)
+  const int per_wave = (nslab + WAVES - 1) / WAVES;
+  const int s_begin = wave * per_wave;
+  const int s_end = (s_begin + per_wave) < nslab ? (s_begin + per_wave) : nslab;
+
+  // weight DMA: lane (cr = lane >> 3, cp = lane & 7) moves logical chunk cp ^ cr of row cr (then
+  // row 8 + cr) of a 16-row group to LDS position lane * 16: row r, chunk c is stored at c ^ (r & 7)
+  const int cr = lane >> 3, cp = lane & 7;
+  const int cchunk = cp ^ cr;
+  const uint32_t w_voff = (uint32_t)cr * (uint32_t)p.ldb + cchunk * 16;
+  const uint32_t w_half = 8u * (uint32_t)p.ldb;
+  const uint32_t w_tile = 16u * (uint32_t)p.ldb;
+  // activation operand: lane (m = lm, lq) holds K bytes [16*lq, +16) and [64 + 16*lq, +16) of token m
+  uint32_t a_off[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) a_off[t] = (uint32_t)(t * 16 + lm) * (uint32_t)p.lda + lq * 16;
+  // fragment read: row lm of a 16-row group, logical chunks lq and lq + 4
+  const uint32_t frag0 = lm * 128 + ((lq ^ (lm & 7)) << 4);
+  const uint32_t frag1 = lm * 128 + (((lq + 4) ^ (lm & 7)) << 4);
+  uint8_t* ring = smem + wave * Cfg::RING;
+
+  __amdgpu_buffer_rsrc_t as_rsrc = sk_rsrc(nullptr, 0), bs_rsrc = sk_rsrc(nullptr, 0);
+  uint32_t as_voff[MT];
+  if constexpr (BLOCKSCALE) {
+    as_rsrc = sk_rsrc(p.a_scales, sk_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + p.M) * 4));
+    bs_rsrc = sk_rsrc(p.b_scales + (int64_t)(n0 / 128) * p.b_scales_ld, (uint32_t)nslab * 4u);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = t * 16 + lm;
+      as_voff[t] = (uint32_t)(m < p.M ? m : p.M - 1) * 4u;
+    }
+  }
 
   v4f acc[MT][NTW];
 #pragma unroll
@@ -59,73 +120,94 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(GemmArgs p) {
 #pragma unroll
     for (int j = 0; j < NTW; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  int as_m[MT];
-  const float* bs_row = nullptr;
-  if constexpr (BLOCKSCALE) {
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const int m = t * 16 + lm;
-      as_m[t] = m < p.M ? m : p.M - 1;
-    }
-    bs_row = p.b_scales + (int64_t)(n0 / 128) * p.b_scales_ld;
-  }
+  v8i af[DEPTH][MT];
+  float as_v[DEPTH][MT], bs_v[DEPTH];
 
-  v8i wf[NTW], af[MT];
-  float sc[MT];
-  auto load_slab = [&](int slab) {
-    const uint32_t koff = (uint32_t)slab * 128u;
-    uint32_t kill0 = 0, kill1 = 0;
+  // Issues the PER loads of one slab into pipeline slot d.  Slabs past the wave's range are
+  // issued "out of range" (zeros, no traffic), so every slot always carries exactly PER
+  // instructions and the wait counts below are exact.
+  auto issue = [&](int slab, auto d_c) {
+    constexpr int d = decltype(d_c)::value;
+    const bool live = slab < s_end;
+    const int sl = live ? slab : s_begin;
+    const uint32_t koff = (uint32_t)sl * 128u;
+    uint32_t kill0 = live ? 0u : 0x80000000u, kill1 = kill0, killw = kill0;
     if (k_tail) {
       if (koff + lq * 16 >= (uint32_t)p.K) kill0 = 0x80000000u;
       if (koff + 64 + lq * 16 >= (uint32_t)p.K) kill1 = 0x80000000u;
-    }
-#pragma unroll
-    for (int t = 0; t < NTW; ++t) {
-      const v4i lo = sk_load16(b_rsrc, (b_off[t] + koff) | kill0);
-      const v4i hi = sk_load16(b_rsrc, (b_off[t] + koff + 64) | kill1);
-      wf[t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      if (koff + cchunk * 16 >= (uint32_t)p.K) killw = 0x80000000u;
     }
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      const v4i lo = sk_load16(a_rsrc, (a_off[t] + koff) | kill0);
-      const v4i hi = sk_load16(a_rsrc, (a_off[t] + koff + 64) | kill1);
-      af[t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      const v4i lo = sk_load16(a_rsrc, a_off[t] | kill0, koff);
+      const v4i hi = sk_load16(a_rsrc, a_off[t] | kill1, koff + 64);
+      af[d][t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
     if constexpr (BLOCKSCALE) {
-      const float bs = bs_row[slab];
 #pragma unroll
-      for (int t = 0; t < MT; ++t) sc[t] = p.a_scales[(int64_t)slab * p.a_scales_ld + as_m[t]] * bs;
+      for (int t = 0; t < MT; ++t)
+        as_v[d][t] = sk_load_f32(as_rsrc, as_voff[t], (uint32_t)sl * (uint32_t)p.a_scales_ld * 4u);
+      bs_v[d] = sk_load_f32(bs_rsrc, 0, (uint32_t)sl * 4u);
+    }
+    uint8_t* slot = ring + d * SLOT;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (sk_lds_ptr_t)(slot + t * 2048), 16, w_voff | killw,
+                                               koff + t * w_tile, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (sk_lds_ptr_t)(slot + t * 2048 + 1024), 16, w_voff | killw,
+                                               koff + t * w_tile + w_half, 0, 0);
     }
   };
-
-  // The compiler software-pipelines this loop (the loads of the next slab do not
-  // depend on the MFMAs of this one); UNROLL slabs are in flight per wave.
-  constexpr int UNROLL = (NTW * 2 + MT * 2) <= 8 ? 4 : 2;
-#pragma unroll UNROLL
-  for (int slab = wave; slab < nslab; slab += WAVES) {
-    load_slab(slab);
+  auto compute = [&](auto d_c) {
+    constexpr int d = decltype(d_c)::value;
+    // the slot's loads are the oldest in flight: everything issued for the DEPTH-1 younger slots may stay
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * PER) : "memory");
+    const uint8_t* slot = ring + d * SLOT;
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
+      const v4i lo = *reinterpret_cast<const v4i*>(slot + nt * 2048 + frag0);
+      const v4i hi = *reinterpret_cast<const v4i*>(slot + nt * 2048 + frag1);
+      const v8i wf = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         if constexpr (BLOCKSCALE) {
           const v4f zero = {0.f, 0.f, 0.f, 0.f};
-          const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], af[mt], zero, 0, 0, 0, 0, 0, 0);
-          acc[mt][nt] += part * sc[mt];
+          const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af[d][mt], zero, 0, 0, 0, 0, 0, 0);
+          acc[mt][nt] += part * (as_v[d][mt] * bs_v[d]);
         } else {
-          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], af[mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
+          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af[d][mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
         }
       }
     }
+    // the fragment reads must have left LDS before the slot is refilled
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
+  auto for_each_slot = [&](auto&& f) {
+    [&]<int... D>(std::integer_sequence<int, D...>) { (f(std::integral_constant<int, D>{}), ...); }
+    (std::make_integer_sequence<int, DEPTH>{});
+  };
+
+  for_each_slot([&](auto d_c) { issue(s_begin + decltype(d_c)::value, d_c); });
+  for (int base = s_begin; base < s_end; base += DEPTH) {
+    for_each_slot([&](auto d_c) {
+      constexpr int d = decltype(d_c)::value;
+      compute(d_c);
+      issue(base + DEPTH + d, d_c);
+    });
   }
+  // drain: the last DEPTH issues were out of range, but they still target LDS slots
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
 
   // ---- reduce the 4 waves' partial sums (fixed order) and store ----------------------
+  float* red = reinterpret_cast<float*>(smem);  // [WAVES][MT*NTW*4][64]
+  constexpr int RSTRIDE = MT * NTW * 4 * 64;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) red[wave][(mt * NTW + nt) * 4 + v][lane] = acc[mt][nt][v];
+      for (int v = 0; v < 4; ++v) red[wave * RSTRIDE + ((mt * NTW + nt) * 4 + v) * 64 + lane] = acc[mt][nt][v];
   __syncthreads();
 
   // (mt, nt) pairs are dealt to the waves round-robin
@@ -136,8 +218,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(GemmArgs p) {
     float v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int r = pair * 4 + i;
-      v[i] = ((red[0][r][lane] + red[1][r][lane]) + red[2][r][lane]) + red[3][r][lane];
+      const int r = (pair * 4 + i) * 64 + lane;
+      float sum = red[r];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) sum += red[w * RSTRIDE + r];
+      v[i] = sum;
     }
     if (m >= p.M || n >= p.N) continue;
     if constexpr (!BLOCKSCALE) {
@@ -169,20 +254,39 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(GemmArgs p) {
   }
 }
 
-template <int NTW, int MT, bool BLOCKSCALE>
-static int launch_skinny(const GemmArgs& p, hipStream_t stream) {
+template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
+static int launch_skinny_r(const GemmArgs& p, hipStream_t stream) {
+  using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
+  auto kern = gemm_skinny_kernel<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM);
+    if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "gemm_skinny: cannot reserve %d bytes of LDS: %s", Cfg::SMEM, hipGetErrorString(e));
+    attr_done = true;
+  }
   const int64_t blocks = ceil_div(p.N, 16 * NTW);
-  hipLaunchKernelGGL((gemm_skinny_kernel<NTW, MT, BLOCKSCALE>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NWAVES * 64), Cfg::SMEM, stream, p);
   return launch_status("gemm_skinny");
 }
 
+// Shape choice (measured on the Llama-70B decode shapes):
+//   N >= 16384: 32 rows per block (an activation fragment feeds two MFMAs), 16 KB of weights
+//               in flight per wave;
+//   smaller N:  16 rows per block, 8 KB per wave: twice the blocks, and more of them per CU.
+// (8 waves per block were tried for the small-N shapes and were slower.)
+// MAXFP8_SKINNY=<ntw>4<ringKB>, e.g. 1408 or 2416, forces a shape for tuning runs.
 template <int MT, bool BLOCKSCALE>
 static int pick_ntw(const GemmArgs& p, hipStream_t stream) {
-  // enough blocks to keep 256 CUs streaming: prefer >= 4 blocks per CU
-  const int64_t n16 = ceil_div(p.N, 16);
-  if (MT <= 2 && n16 >= 4 * 1024 * 4 / 4) return launch_skinny<4, MT, BLOCKSCALE>(p, stream);
-  if (n16 >= 2 * 1024) return launch_skinny<2, MT, BLOCKSCALE>(p, stream);
-  return launch_skinny<1, MT, BLOCKSCALE>(p, stream);
+  const char* e = getenv("MAXFP8_SKINNY");
+  int sel = e ? atoi(e) : 0;
+  if (!sel) sel = (p.N >= 16384 && MT <= 2) ? 2416 : 1408;
+  switch (sel) {
+    case 1408: return launch_skinny_r<1, MT, BLOCKSCALE, 8, 4>(p, stream);
+    case 1416: return launch_skinny_r<1, MT, BLOCKSCALE, 16, 4>(p, stream);
+    case 2416: return launch_skinny_r<2, MT, BLOCKSCALE, 16, 4>(p, stream);
+    case 2408: return launch_skinny_r<2, MT, BLOCKSCALE, 8, 4>(p, stream);
+    default: MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "skinny matmul: unknown shape selector %d", sel);
+  }
 }
 
 int gemm_skinny_max_m() { return 64; }
