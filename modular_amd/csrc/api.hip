@@ -35,7 +35,8 @@ int naive_rowwise_dispatch(void*, const void*, const void*, const void*, const v
                            int64_t, int64_t, int64_t, int64_t, int64_t, int, int, hipStream_t);
 int naive_grouped_dispatch(void*, const void*, const void*, const void*, const void*, const uint32_t*,
                            const int32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int, hipStream_t);
-int gemm_tiled_dispatch(const GemmArgs&, bool, hipStream_t);
+int gemm_tiled_dispatch(const GemmArgs&, bool, size_t, hipStream_t);
+size_t gemm_tiled_workspace_bytes(int64_t, int64_t, int64_t);
 int gemm_grouped_dispatch(const GemmArgs&, int64_t, hipStream_t);
 int gemm_skinny_dispatch(const GemmArgs&, bool, hipStream_t);
 int gemm_skinny_max_m();
@@ -75,8 +76,8 @@ int maxfp8_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const vo
 }
 
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  (void)M; (void)N; (void)K;
-  return 0;  // no kernel of this version needs scratch memory
+  if (M <= 0 || N <= 0 || K <= 0 || M <= gemm_skinny_max_m()) return 0;
+  return gemm_tiled_workspace_bytes(M, N, K);  // split-K partial sums; 0 when no split would be used
 }
 
 int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
@@ -85,7 +86,6 @@ int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, cons
                                      int64_t gm, int64_t gn, int64_t gk, int64_t a_scales_ld, int64_t b_scales_ld,
                                      int c_dtype, int scales_dtype, int algo, void* workspace,
                                      size_t workspace_bytes, void* stream) {
-  (void)workspace; (void)workspace_bytes;
   if (c_dtype != MAXFP8_BF16 && c_dtype != MAXFP8_F32)
     MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "matmul: output dtype %d is not bf16 or f32", c_dtype);
   if (M < 0 || N < 0 || K < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: negative size");
@@ -147,7 +147,9 @@ int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, cons
   p.c_dtype = c_dtype;
   p.c_vec_ok = (ldc % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
   if (algo == MAXFP8_ALGO_SKINNY) return gemm_skinny_dispatch(p, block, st);
-  return gemm_tiled_dispatch(p, block, st);
+  if (workspace && !is_aligned(workspace, 16)) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "matmul: workspace must be 16-byte aligned");
+  p.workspace = (float*)workspace;
+  return gemm_tiled_dispatch(p, block, workspace_bytes, st);
 }
 
 int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,

@@ -192,6 +192,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
   const uint32_t b_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.ldb;
   const bool k_tail = (p.K & 127) != 0;
   const int nslab = (p.K + 127) / 128;
+  // split-K (dense only): blockIdx.y takes a contiguous share of the slabs and leaves raw f32
+  // partial sums in the workspace for the reduction kernel
+  int slab_begin = 0, slab_end = nslab;
+  bool partial_out = false;
+  if constexpr (!GROUPED) {
+    if (p.splits > 1) {
+      const int per = (nslab + p.splits - 1) / p.splits;
+      slab_begin = blockIdx.y * per;
+      slab_end = (slab_begin + per) < nslab ? (slab_begin + per) : nslab;
+      partial_out = true;
+    }
+  }
   // activation scales of the tile: element (slab, row_begin + r); rows past the tile read as 0
   const int s_chunk = wave % (BM / 64);
   __amdgpu_buffer_rsrc_t s_rsrc = t2_rsrc(nullptr, 0);
@@ -258,16 +270,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
   // the DMA of slab j+NS-1 is sent into that buffer.
 #pragma unroll
   for (int st = 0; st < NS - 1; ++st)
-    if (st < nslab) dma(st, st);
+    if (slab_begin + st < slab_end) dma(slab_begin + st, st);
 
   // the weight-block scale of the NEXT slab is fetched before this slab's DMA is issued, so
   // that waiting for it never waits for the youngest DMA
   float bs_nxt = 1.f;
-  if constexpr (BLOCKSCALE) bs_nxt = bs_row[0];
+  if constexpr (BLOCKSCALE) bs_nxt = bs_row[slab_begin];
 
   int buf = 0;
-  for (int slab = 0; slab < nslab; ++slab) {
-    if (NS == 3 && slab + 1 < nslab) {
+  for (int slab = slab_begin; slab < slab_end; ++slab) {
+    if (NS == 3 && slab + 1 < slab_end) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -276,10 +288,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
     asm volatile("" ::: "memory");
     const float bs = bs_nxt;
     if constexpr (BLOCKSCALE) {
-      if (slab + 1 < nslab) bs_nxt = bs_row[slab + 1];
+      if (slab + 1 < slab_end) bs_nxt = bs_row[slab + 1];
     }
     asm volatile("" ::: "memory");
-    if (slab + NS - 1 < nslab) dma(slab + NS - 1, buf == 0 ? NS - 1 : buf - 1);
+    if (slab + NS - 1 < slab_end) dma(slab + NS - 1, buf == 0 ? NS - 1 : buf - 1);
 
     const uint8_t* sa = smem + buf * STAGE_BYTES;
     float s_cur[TM];
@@ -311,6 +323,29 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
   }
 
   // ---- epilogue -----------------------------------------------------------------------------
+  if (partial_out) {
+    float* ws = p.workspace + (int64_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) {
+      const int ml = wm * WM + mt * 16 + lm;
+      if (ml >= rows_here) continue;
+      float* row = ws + (row_begin + ml) * p.N;
+#pragma unroll
+      for (int nt = 0; nt < TN; ++nt) {
+        const int n = n0 + wn * WN + nt * 16 + lq * 4;
+        if (n >= p.N) continue;
+        const v4f v = acc[mt][nt];
+        if ((p.N & 3) == 0) {
+          *reinterpret_cast<float4*>(row + n) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < p.N) row[n + i] = v[i];
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int mt = 0; mt < TM; ++mt) {
     const int ml = wm * WM + mt * 16 + lm;
@@ -350,46 +385,134 @@ static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const 
   return launch_status(name);
 }
 
+// Sums the split-K partial results in split order (deterministic), applies the row / tensor
+// scales where the matmul has them, converts and stores.
+template <bool BLOCKSCALE>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
+  const int64_t total = (int64_t)p.M * p.N;
+  const int64_t stride = (int64_t)gridDim.x * 256 * 4;
+  for (int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4; i < total; i += stride) {
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    const int cnt = (total - i) < 4 ? (int)(total - i) : 4;
+    for (int sp = 0; sp < p.splits; ++sp) {
+      const float* src = p.workspace + (int64_t)sp * total + i;
+      if (cnt == 4 && (total & 3) == 0) {
+        const float4 t = *reinterpret_cast<const float4*>(src);
+        v[0] += t.x; v[1] += t.y; v[2] += t.z; v[3] += t.w;
+      } else {
+        for (int j = 0; j < cnt; ++j) v[j] += src[j];
+      }
+    }
+    for (int j = 0; j < cnt; ++j) {
+      const int64_t m = (i + j) / p.N;
+      const int64_t n = (i + j) - m * p.N;
+      float r = v[j];
+      if constexpr (!BLOCKSCALE) {
+        r = r * p.a_scales[m * p.a_scale_stride];
+        r = r * p.b_scales[n * p.b_scale_stride];
+      }
+      if (p.c_dtype == MAXFP8_BF16) reinterpret_cast<uint16_t*>(p.c)[m * p.ldc + n] = (uint16_t)f32_to_bf16_bits(r);
+      else reinterpret_cast<float*>(p.c)[m * p.ldc + n] = r;
+    }
+  }
+}
+
 // ---- kernel selection ------------------------------------------------------------------------
 // Three tile shapes.  `t_slab` is the measured time one block spends per 128-byte K slab when
 // the whole chip is busy (microseconds); the cost of a shape is rounds * t_slab, with
 // rounds = ceil(tiles / resident blocks).
 struct TileShape { int bm, bn, slots; float t_slab_block, t_slab_row; };
-static const TileShape kShapes[3] = {
+static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, dim3 grid, hipStream_t stream);
+
+static const TileShape kShapes[4] = {
     {256, 256, 256, 2.05f, 1.70f},   // 8 waves, 2 stages
     {256, 128, 256, 1.10f, 1.00f},   // 8 waves, 3 stages
     {128, 128, 512, 1.20f, 1.05f},   // 4 waves, 2 stages, two blocks per CU
+    {128, 128, 256, 9.99f, 9.99f},   // 4 waves, 3 stages, one block per CU (tuning only)
 };
 
 // MAXFP8_TILE=1/2/3 forces a shape (for tuning runs); anything else lets the cost model pick.
 static int tile_override() {
   const char* e = getenv("MAXFP8_TILE");
   const int v = e ? atoi(e) : 0;
-  return (v >= 1 && v <= 3) ? v : 0;
+  return (v >= 1 && v <= 4) ? v : 0;
 }
 
-static int pick_shape(int64_t M, int64_t N, bool blockscale) {
+// Split-K: when the tiles of a matmul cover only part of the chip, K is cut into `splits` shares
+// (each at least 4 slabs) until the grid fills the resident-block slots.  Needs
+// splits * M * N * 4 bytes of workspace; without workspace the matmul runs unsplit.
+static int pick_splits(int64_t tiles, int slots, int nslab) {
+  const char* e = getenv("MAXFP8_SPLITK");
+  int splits = e ? atoi(e) : 0;
+  if (splits <= 0) {
+    splits = 1;
+    if (tiles * 2 <= slots) splits = (int)(slots / tiles);
+    if (splits > 16) splits = 16;
+  }
+  if (splits > nslab / 4) splits = nslab / 4;
+  if (splits < 1) splits = 1;
+  const int per = (nslab + splits - 1) / splits;
+  return (nslab + per - 1) / per;  // no empty share
+}
+
+// cost of a shape (microseconds) = rounds of resident blocks * slabs per block * time per slab
+static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can_split) {
   int best = 0;
   float best_cost = 0.f;
   for (int i = 0; i < 3; ++i) {
     const TileShape& t = kShapes[i];
     const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
-    const float cost = (float)ceil_div(tiles, t.slots) * (blockscale ? t.t_slab_block : t.t_slab_row);
+    const int sp = can_split ? pick_splits(tiles, t.slots, nslab) : 1;
+    float cost = (float)ceil_div(tiles * sp, t.slots) * (float)ceil_div(nslab, sp) *
+                 (blockscale ? t.t_slab_block : t.t_slab_row);
+    // a split pays a second launch and one write + one read of sp * M * N f32 partial sums (~4 TB/s)
+    if (sp > 1) cost += 5.0f + (float)sp * (float)M * (float)N * 8.0f / 4.0e6f;
     if (i == 0 || cost < best_cost) { best = i; best_cost = cost; }
   }
   return best + 1;
 }
 
-int gemm_tiled_dispatch(const GemmArgs& p, bool blockscale, hipStream_t stream) {
+size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  // the largest split count any shape could choose for this problem
+  size_t worst = 0;
+  const int nslab = (int)ceil_div(K, 128);
+  for (int i = 0; i < 3; ++i) {
+    const TileShape& t = kShapes[i];
+    const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+    const int sp = pick_splits(tiles, t.slots, nslab);
+    if (sp > 1 && (size_t)sp > worst) worst = sp;
+  }
+  return worst * (size_t)M * (size_t)N * 4;
+}
+
+int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, hipStream_t stream) {
+  GemmArgs p = p_in;
+  const int nslab = (p.K + 127) / 128;
   int variant = tile_override();
-  if (!variant) variant = pick_shape(p.M, p.N, blockscale);
+  if (!variant) variant = pick_shape(p.M, p.N, nslab, blockscale, p.workspace != nullptr);
   const TileShape& t = kShapes[variant - 1];
   const int64_t tiles = ceil_div(p.M, t.bm) * ceil_div(p.N, t.bn);
   if (tiles >= ((int64_t)1 << 31)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "tiled matmul: too many tiles");
-  const dim3 grid((unsigned)tiles);
+  p.splits = 1;
+  if (p.workspace) {
+    const int sp = pick_splits(tiles, t.slots, (p.K + 127) / 128);
+    if (sp > 1 && (size_t)sp * p.M * p.N * 4 <= workspace_bytes) p.splits = sp;
+  }
+  const dim3 grid((unsigned)tiles, (unsigned)p.splits);
+  const int rc = gemm_tiled_launch(p, blockscale, variant, grid, stream);
+  if (rc != MAXFP8_OK || p.splits == 1) return rc;
+  const int64_t quads = ceil_div((int64_t)p.M * p.N, 4);
+  const unsigned rblocks = (unsigned)(ceil_div(quads, 256) < 4096 ? ceil_div(quads, 256) : 4096);
+  if (blockscale) hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3(rblocks), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3(rblocks), dim3(256), 0, stream, p);
+  return launch_status("splitk_reduce");
+}
+
+static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, dim3 grid, hipStream_t stream) {
   if (blockscale) {
     if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, true, false>(p, grid, stream, "gemm_tiled_block_256x256");
     if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, true, false>(p, grid, stream, "gemm_tiled_block_256x128");
+    if (variant == 4) return launch_tiled<128, 128, 2, 2, 3, true, false>(p, grid, stream, "gemm_tiled_block_128x128x3");
     return launch_tiled<128, 128, 2, 2, 2, true, false>(p, grid, stream, "gemm_tiled_block_128x128");
   }
   if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false, false>(p, grid, stream, "gemm_tiled_row_256x256");

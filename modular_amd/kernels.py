@@ -183,10 +183,13 @@ def dynamic_scaled_matmul(
     ldb = b.stride(0) if N > 1 else K
     a_ld = a_scales.stride(0) if a_scales.shape[0] > 1 else a_scales.shape[1]
     b_ld = b_scales.stride(0) if b_scales.shape[0] > 1 else b_scales.shape[1]
+    # split-K scratch for problems whose tiles would cover only part of the chip (0 bytes otherwise)
+    ws_bytes = _lib.lib().maxfp8_matmul_workspace_bytes(M, N, K) if algo in ("auto", "tiled") else 0
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=a.device) if ws_bytes else None
     st = _lib.lib().maxfp8_matmul_dynamic_scaled_fp8(
         c.data_ptr(), a.data_ptr(), b.data_ptr(), a_scales.data_ptr(), b_scales.data_ptr(), M, N, K,
         lda, ldb, N, gin, gw, gm, gn, gk, a_ld, b_ld, _DT[out_type], _DT[a_scales.dtype], _ALGOS[algo],
-        None, 0, _stream(a))
+        ws.data_ptr() if ws is not None else None, ws_bytes, _stream(a))
     _lib.check(st)
     return c
 
