@@ -63,6 +63,19 @@ WORKLOADS = {
 DEFAULT = "llama8b_gate_up_m2048"
 
 
+def measured_traffic(name):
+    """HBM bytes per launch of the workload's matmul kernel, measured with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE (profiles/hbm_traffic_pmc.txt); None when it was not measured."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", "hbm_traffic_pmc.txt")):
+            parts = line.split()
+            if len(parts) == 3 and parts[0] == "traffic" and parts[1] == name:
+                return int(parts[2])
+    except OSError:
+        pass
+    return None
+
+
 def algorithmic(kind, M, K, N):
     """(flops, HBM bytes) of one step's matmul, and bytes of the quantisation."""
     flops = 2.0 * M * N * K
@@ -201,7 +214,9 @@ def result_line(name, steps, warmup, with_cpu=True):
     kind, M, K, N = wl.kind, wl.M, wl.K, wl.N
     flops, mm_bytes, q_bytes = algorithmic(kind, M, K, N)
     if kind == "grouped":
-        mm_bytes += 255 * N * K  # every expert's weights are streamed once
+        # weights of every expert that received tokens are streamed once (experts without tokens are never read)
+        active = int((wl.counts > 0).sum())
+        mm_bytes += (active - 1) * N * K + 4 * (active - 1) * math.ceil(N / 128) * (K // 128)
     hbm_bound = kind == "row" or M <= 16
     if hbm_bound:
         value, unit = (mm_bytes + q_bytes) / (ms_step * 1e-3) / 1e9, "GB/s"
@@ -210,8 +225,9 @@ def result_line(name, steps, warmup, with_cpu=True):
         value, unit = flops / (ms_step * 1e-3) / 1e12, "TFLOP/s"
         roof = {"bound": "mfma", "achieved": flops / (mm_avg * 1e-3) / 1e12, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
-    roof["kernel"] = {"grouped": "gemm_tiled_kernel<grouped>", "row": "gemm_skinny_kernel"}.get(
+    roof["traffic"] = measured_traffic(name)
+    roof["algorithmic_bytes"] = mm_bytes
+    roof["kernel"] = {"grouped": "gemm_tiled_kernel<128,128,...,grouped>", "row": "gemm_skinny_kernel"}.get(
         kind, "gemm_skinny_kernel" if M <= 64 else "gemm_tiled_kernel")
     roof["kernel_ms_avg"], roof["kernel_ms_median"], roof["kernel_ms_min"] = mm_avg, mm_med, mm_min
     out = {
@@ -237,6 +253,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--table", action="store_true", help="run every workload, write gpurun_out/bench_table.json")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch the plain copy kernel on 256 MiB three times (the known-size unit that "
+                         "hardware byte counters of a rocprofv3 --pmc run are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collective); run with --gpus 1",
@@ -261,6 +280,13 @@ def main():
                 json.dump(rows, f, indent=1)
             torch.cuda.empty_cache()
         return
+    if args.calibrate:
+        from modular_amd import kernels
+        src = torch.ones((256 << 20,), dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            kernels.copy_bytes(dst, src)
+        torch.cuda.synchronize()
     print(json.dumps(result_line(args.workload, args.steps, args.warmup, with_cpu=not args.no_cpu)))
 
 
