@@ -50,7 +50,7 @@ __device__ __forceinline__ uint32_t t2_clamp_u32(int64_t v) {
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmArgs p) {
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
   constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int NTHREADS = NWAVES * 64;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -190,7 +190,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
   const uint32_t b_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.ldb + cchunk * 16;
   const uint32_t a_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.lda;
   const uint32_t b_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.ldb;
-  const bool k_tail = (p.K & 127) != 0;
   const int nslab = (p.K + 127) / 128;
   // split-K (dense only): blockIdx.y takes a contiguous share of the slabs and leaves raw f32
   // partial sums in the workspace for the reduction kernel
@@ -215,27 +214,34 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
     s_slab_step = (uint32_t)p.a_scales_ld * 4u;
   }
 
-  auto dma = [&](int slab, int buf) {
+  // LDS-DMA instruction idx (0 .. PER-1) of a wave's share of a slab
+  // (dead = 0x80000000 puts every lane out of range: nothing is fetched and the copy only writes
+  // zeros into a stage that is not read again; that keeps the loop free of branches)
+  auto dma_one = [&](int slab, int buf, int idx, uint32_t dead) {
     const uint32_t koff = (uint32_t)slab * 128u;
-    uint32_t kill = 0;
-    if (k_tail && koff + cchunk * 16 >= (uint32_t)p.K) kill = 0x80000000u;
+    uint32_t kill = dead;
+    if (koff + cchunk * 16 >= (uint32_t)p.K) kill = 0x80000000u;
     uint8_t* sa = smem + buf * STAGE_BYTES + wave * 1024;
     uint8_t* sb = sa + BM * 128;
-#pragma unroll
-    for (int i = 0; i < IA; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(sa + i * NWAVES * 1024), 16, a_voff | kill,
-                                               koff + i * a_istep, 0, 0);
-#pragma unroll
-    for (int i = 0; i < IB; ++i)
+    if (idx < IA) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(sa + idx * NWAVES * 1024), 16, a_voff | kill,
+                                               koff + idx * a_istep, 0, 0);
+    } else if (idx < IA + IB) {
+      const int i = idx - IA;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(sb + i * NWAVES * 1024), 16, b_voff | kill,
                                                koff + i * b_istep, 0, 0);
-    if constexpr (BLOCKSCALE) {
+    } else if constexpr (BLOCKSCALE) {
       // 64 scales of the slab's row of the transposed scale matrix per wave; with more waves
       // than 64-row chunks the extra waves repeat a chunk (same bytes to the same place), so
       // every wave issues the same number of DMA instructions per slab.
       uint8_t* ss = smem + buf * STAGE_BYTES + (BM + BN) * 128 + s_chunk * 256;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(s_rsrc, (lds_ptr_t)ss, 4, s_voff, (uint32_t)slab * s_slab_step, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(s_rsrc, (lds_ptr_t)ss, 4, s_voff | dead,
+                                               (uint32_t)slab * s_slab_step, 0, 0);
     }
+  };
+  auto dma = [&](int slab, int buf, uint32_t dead) {
+#pragma unroll
+    for (int idx = 0; idx < PER; ++idx) dma_one(slab, buf, idx, dead);
   };
 
   // ---- fragment read plan -------------------------------------------------------------------
@@ -270,7 +276,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
   // the DMA of slab j+NS-1 is sent into that buffer.
 #pragma unroll
   for (int st = 0; st < NS - 1; ++st)
-    if (slab_begin + st < slab_end) dma(slab_begin + st, st);
+    dma(slab_begin + st, st, slab_begin + st < slab_end ? 0u : 0x80000000u);
 
   // the weight-block scale of the NEXT slab is fetched before this slab's DMA is issued, so
   // that waiting for it never waits for the youngest DMA
@@ -279,7 +285,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
 
   int buf = 0;
   for (int slab = slab_begin; slab < slab_end; ++slab) {
-    if (NS == 3 && slab + 1 < slab_end) {
+    if (NS == 3) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -291,7 +297,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
       if (slab + 1 < slab_end) bs_nxt = bs_row[slab + 1];
     }
     asm volatile("" ::: "memory");
-    if (slab + NS - 1 < slab_end) dma(slab + NS - 1, buf == 0 ? NS - 1 : buf - 1);
+    // The DMA of slab + NS - 1 is issued in pieces between the MFMA groups below: a wave that
+    // sends its whole share at once sits in the VMEM issue queue for most of the copy's
+    // duration, and since the barrier lines all waves up, the matrix pipe idles meanwhile.
+    const uint32_t dead = slab + NS - 1 < slab_end ? 0u : 0x80000000u;
+    const int dma_slab = slab + NS - 1, dma_buf = buf == 0 ? NS - 1 : buf - 1;
+#ifndef MAXFP8_DMA_SPREAD
+#define MAXFP8_DMA_SPREAD TM
+#endif
+    constexpr int SPREAD = MAXFP8_DMA_SPREAD < 1 ? 1 : (MAXFP8_DMA_SPREAD > TM ? TM : MAXFP8_DMA_SPREAD);
 
     const uint8_t* sa = smem + buf * STAGE_BYTES;
     float s_cur[TM];
@@ -318,6 +332,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmA
         }
       }
       af = af_next;
+#pragma unroll
+      for (int idx = 0; idx < PER; ++idx)
+        if (idx * SPREAD / PER == mt) dma_one(dma_slab, dma_buf, idx, dead);
+#ifdef MAXFP8_SCHED_BARRIER
+      __builtin_amdgcn_sched_barrier(0);
+#endif
     }
     buf = buf + 1 == NS ? 0 : buf + 1;
   }
