@@ -20,6 +20,7 @@ struct GemmArgs {
   const uint32_t* offsets;
   const int32_t* expert_ids;
   int num_active;
+  int small_rows;            // slots with at most this many rows use the small tile (0: none do)
   int64_t b_expert_stride;   // bytes between experts in b
   int64_t bs_expert_stride;  // elements between experts in b_scales
   // split-K / skinny only

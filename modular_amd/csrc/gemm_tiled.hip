@@ -49,91 +49,29 @@ __device__ __forceinline__ uint32_t t2_clamp_u32(int64_t v) {
   return v > 0xfffffff0ll ? 0xfffffff0u : (v < 0 ? 0u : (uint32_t)v);
 }
 
+// One BM x BN tile of C: rows [row_begin, row_end) (at most BM of them are used) by columns
+// [n0, n0 + BN) of the weight matrix at bptr / scales at bs_ptr.  Called by every thread of a
+// block of WAVES_M * WAVES_N waves with `smem` = the block's dynamic LDS.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
+__device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, const int64_t row_begin, const int64_t row_end,
+                                          const int n0, const uint8_t* bptr, const float* bs_ptr) {
   constexpr int NWAVES = WAVES_M * WAVES_N;
-  constexpr int NTHREADS = NWAVES * 64;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 16, TN = WN / 16;
   constexpr int IA = BM / 8 / NWAVES, IB = BN / 8 / NWAVES;  // LDS-DMA instructions per wave and slab
-  // one stage: A rows, B rows, then (block scaling) the slab's BM activation scales
-  constexpr int SCALE_BYTES = BLOCKSCALE ? BM * 4 : 0;
+  // one stage: A rows, B rows, then (block scaling) the slab's activation scales, 64 per copy
+  constexpr int SCALE_ROWS = BM < 64 ? 64 : BM;
+  constexpr int SCALE_BYTES = BLOCKSCALE ? SCALE_ROWS * 4 : 0;
   constexpr int STAGE_BYTES = (BM + BN) * 128 + SCALE_BYTES;
   constexpr int PER = IA + IB + (BLOCKSCALE ? 1 : 0);  // LDS-DMA instructions per wave and slab
   static_assert(NWAVES % 2 == 0 && IA >= 1 && IB >= 1, "tile / wave layout");
   static_assert(NS == 2 || NS == 3, "two or three LDS stages");
-  static_assert(!BLOCKSCALE || BM % 64 == 0, "scale rows are copied 64 at a time");
+  static_assert(!BLOCKSCALE || SCALE_ROWS % 64 == 0, "scale rows are copied 64 at a time");
   static_assert(!BLOCKSCALE || (WN <= 128 && 128 % WN == 0), "a wave's columns must sit inside one 128-wide scale block");
-
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-
-  // ---- block -> tile ----------------------------------------------------------------
-  int64_t row_begin, row_end;
-  int n0;
-  const uint8_t* bptr = p.b;
-  const float* bs_ptr = p.b_scales;
-  bool zero_fill = false;
-  if constexpr (GROUPED) {
-    __shared__ int s_slot, s_tile, s_wave_sum[NWAVES], s_carry;
-    if (tid == 0) { s_slot = -1; s_tile = 0; s_carry = 0; }
-    __syncthreads();
-    for (int z0 = 0; z0 < p.num_active; z0 += NTHREADS) {
-      const int z = z0 + tid;
-      int t = 0;
-      if (z < p.num_active) t = ((int)(p.offsets[z + 1] - p.offsets[z]) + BM - 1) / BM;
-      int incl = t;
-#pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int up = __shfl_up(incl, o, 64);
-        if (lane >= o) incl += up;
-      }
-      if (lane == 63) s_wave_sum[wave] = incl;
-      __syncthreads();
-      int before = s_carry;
-      for (int w = 0; w < wave; ++w) before += s_wave_sum[w];
-      const int excl = before + incl - t;
-      if (t > 0 && (int)blockIdx.y >= excl && (int)blockIdx.y < excl + t) { s_slot = z; s_tile = blockIdx.y - excl; }
-      __syncthreads();
-      if (tid == NTHREADS - 1) s_carry = before + incl;
-      __syncthreads();
-      if (s_slot >= 0 || (int)blockIdx.y < s_carry) break;
-    }
-    const int slot = s_slot;
-    if (slot < 0) return;
-    row_begin = (int64_t)p.offsets[slot] + (int64_t)s_tile * BM;
-    row_end = p.offsets[slot + 1];
-    n0 = blockIdx.x * BN;
-    const int e = p.expert_ids[slot];
-    if (e < 0) zero_fill = true;
-    else {
-      bptr += (int64_t)e * p.b_expert_stride;
-      bs_ptr += (int64_t)e * p.bs_expert_stride;
-    }
-  } else {
-    const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-    const int total = tiles_m * tiles_n;
-    int pid = blockIdx.x;
-    {
-      const int xcd = pid & 7, local = pid >> 3;
-      const int base = total >> 3, rem = total & 7;
-      pid = xcd * base + (xcd < rem ? xcd : rem) + local;
-    }
-    constexpr int GROUP_M = 4;
-    const int per_group = GROUP_M * tiles_n;
-    const int group = pid / per_group;
-    const int first_m = group * GROUP_M;
-    const int gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-    const int in_group = pid - group * per_group;
-    const int tm = first_m + in_group % gsize;
-    const int tn = in_group / gsize;
-    row_begin = (int64_t)tm * BM;
-    row_end = p.M;
-    n0 = tn * BN;
-  }
   const int rows_here = (int)((row_end - row_begin) < BM ? (row_end - row_begin) : BM);
   const int cols_here = (p.N - n0) < BN ? (p.N - n0) : BN;
 
@@ -164,20 +102,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
     }
   };
 
-  if (GROUPED && zero_fill) {
-#pragma unroll
-    for (int mt = 0; mt < TM; ++mt) {
-      const int ml = wm * WM + mt * 16 + lm;
-      if (ml >= rows_here) continue;
-#pragma unroll
-      for (int nt = 0; nt < TN; ++nt) {
-        const int n = n0 + wn * WN + nt * 16 + lq * 4;
-        if (n < p.N) store4(row_begin + ml, n, 0.f, 0.f, 0.f, 0.f);
-      }
-    }
-    return;
-  }
-
   // ---- global -> LDS copy plan (LDS DMA) ------------------------------------------------
   const uint8_t* a_tile = p.a + row_begin * p.lda;
   const uint8_t* b_tile = bptr + (int64_t)n0 * p.ldb;
@@ -204,7 +128,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
     }
   }
   // activation scales of the tile: element (slab, row_begin + r); rows past the tile read as 0
-  const int s_chunk = wave % (BM / 64);
+  const int s_chunk = wave % (SCALE_ROWS / 64);
   __amdgpu_buffer_rsrc_t s_rsrc = t2_rsrc(nullptr, 0);
   uint32_t s_voff = 0, s_slab_step = 0;
   if constexpr (BLOCKSCALE) {
@@ -265,6 +189,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
+  // number of this wave's 16-row groups that hold rows of the tile (wave-uniform)
+  constexpr bool SKIP_ROWS = GROUPED && BM <= 64;  // (in big tiles the branches cost more than the MFMAs saved)
+  int mt_live = TM;
+  if constexpr (SKIP_ROWS) {
+    const int left = __builtin_amdgcn_readfirstlane(rows_here) - wm * WM;
+    mt_live = left <= 0 ? 0 : ((left + 15) >> 4 < TM ? (left + 15) >> 4 : TM);
+  }
   const float* bs_row = nullptr;
   if constexpr (BLOCKSCALE) bs_row = bs_ptr + (int64_t)((n0 + wn * WN) / 128) * p.b_scales_ld;
   const uint32_t s_rd = (uint32_t)((BM + BN) * 128 + (wm * WM + lm) * 4);
@@ -319,19 +250,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
     v8i af = read_frag(sa + a_frag_base);
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) {
-      v8i af_next = af;
-      if (mt + 1 < TM) af_next = read_frag(sa + a_frag_base + (mt + 1) * 2048);
+      // 16-row groups past the end of a short tile (an expert with few tokens) are skipped:
+      // their fragments are not read and their MFMAs not issued
+      if (!SKIP_ROWS || mt < mt_live) {
+        v8i af_next = af;
+        if (mt + 1 < TM) af_next = read_frag(sa + a_frag_base + (mt + 1) * 2048);
 #pragma unroll
-      for (int nt = 0; nt < TN; ++nt) {
-        if constexpr (BLOCKSCALE) {
-          const v4f zero = {0.f, 0.f, 0.f, 0.f};
-          const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
-          acc[mt][nt] += part * s_cur[mt];
-        } else {
-          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
+        for (int nt = 0; nt < TN; ++nt) {
+          if constexpr (BLOCKSCALE) {
+            const v4f zero = {0.f, 0.f, 0.f, 0.f};
+            const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
+            acc[mt][nt] += part * s_cur[mt];
+          } else {
+            acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
+          }
         }
+        af = af_next;
       }
-      af = af_next;
 #pragma unroll
       for (int idx = 0; idx < PER; ++idx)
         if (idx * SPREAD / PER == mt) dma_one(dma_slab, dma_buf, idx, dead);
@@ -391,18 +326,123 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED>
-static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
-  constexpr int smem = NS * ((BM + BN) * 128 + (BLOCKSCALE ? BM * 4 : 0));
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, GROUPED>;
-  static bool attr_done = false;
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  // ---- block -> tile: XCD de-interleave, then groups of GROUP_M row tiles share weight columns
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  {
+    const int xcd = pid & 7, local = pid >> 3;
+    const int base = total >> 3, rem = total & 7;
+    pid = xcd * base + (xcd < rem ? xcd : rem) + local;
+  }
+  constexpr int GROUP_M = 4;
+  const int per_group = GROUP_M * tiles_n;
+  const int group = pid / per_group;
+  const int first_m = group * GROUP_M;
+  const int gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int in_group = pid - group * per_group;
+  const int tm = first_m + in_group % gsize;
+  const int tn = in_group / gsize;
+  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false>(p, smem, (int64_t)tm * BM, p.M, tn * BN, p.b, p.b_scales);
+}
+
+// Grouped (MoE) matmul.  Slot z owns rows [offsets[z], offsets[z+1]).  A slot with at most
+// small_rows (<= SBM) rows is one SBM-row tile per BN columns, computed with a small tile and one more LDS stage
+// (such tiles only stream weights, so what they need is bytes in flight); a larger slot is cut
+// into BM-row tiles.  blockIdx.y counts row tiles over all slots, blockIdx.x is the column tile.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_grouped_kernel(GemmArgs p) {
+  static_assert(WAVES_M * WAVES_N == SWAVES_M * SWAVES_N, "both tile kinds run on the same block");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  constexpr int NWAVES = WAVES_M * WAVES_N, NTHREADS = NWAVES * 64;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  __shared__ int s_slot, s_tile, s_wave_sum[NWAVES], s_carry;
+  if (tid == 0) { s_slot = -1; s_tile = 0; s_carry = 0; }
+  __syncthreads();
+  for (int z0 = 0; z0 < p.num_active; z0 += NTHREADS) {
+    const int z = z0 + tid;
+    int t = 0;
+    if (z < p.num_active) {
+      const int rows = (int)(p.offsets[z + 1] - p.offsets[z]);
+      t = rows <= p.small_rows ? (rows > 0 ? 1 : 0) : (rows + BM - 1) / BM;
+    }
+    int incl = t;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    if (lane == 63) s_wave_sum[wave] = incl;
+    __syncthreads();
+    int before = s_carry;
+    for (int w = 0; w < wave; ++w) before += s_wave_sum[w];
+    const int excl = before + incl - t;
+    if (t > 0 && (int)blockIdx.y >= excl && (int)blockIdx.y < excl + t) { s_slot = z; s_tile = blockIdx.y - excl; }
+    __syncthreads();
+    if (tid == NTHREADS - 1) s_carry = before + incl;
+    __syncthreads();
+    if (s_slot >= 0 || (int)blockIdx.y < s_carry) break;
+  }
+  const int slot = s_slot;
+  if (slot < 0) return;
+  const int64_t slot_begin = p.offsets[slot], row_end = p.offsets[slot + 1];
+  const bool small = row_end - slot_begin <= p.small_rows;
+  const int64_t row_begin = slot_begin + (int64_t)s_tile * BM;
+  const int n0 = blockIdx.x * BN;
+  const int e = p.expert_ids[slot];
+  if (e < 0) {
+    // a slot without an expert writes zeros
+    const int rows_here = (int)((row_end - row_begin) < BM ? (row_end - row_begin) : BM);
+    const int cols_here = (p.N - n0) < BN ? (p.N - n0) : BN;
+    for (int i = tid; i < rows_here * cols_here; i += NTHREADS) {
+      const int64_t m = row_begin + i / cols_here;
+      const int n = n0 + i % cols_here;
+      if (p.c_dtype == MAXFP8_BF16) reinterpret_cast<uint16_t*>(p.c)[m * p.ldc + n] = 0;
+      else reinterpret_cast<float*>(p.c)[m * p.ldc + n] = 0.f;
+    }
+    return;
+  }
+  const uint8_t* bptr = p.b + (int64_t)e * p.b_expert_stride;
+  const float* bs_ptr = p.b_scales + (int64_t)e * p.bs_expert_stride;
+  if (small) tile_body<SBM, BN, SWAVES_M, SWAVES_N, SNS, true, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+  else tile_body<BM, BN, WAVES_M, WAVES_N, NS, true, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+}
+
+template <int BM, int BN, int NS, bool BLOCKSCALE>
+constexpr int tile_lds_bytes() {
+  return NS * ((BM + BN) * 128 + (BLOCKSCALE ? (BM < 64 ? 64 : BM) * 4 : 0));
+}
+
+template <typename Kern>
+static int launch_with_lds(Kern kern, bool& attr_done, int smem, int threads, const GemmArgs& p, dim3 grid, hipStream_t stream,
+                           const char* name) {
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, smem, hipGetErrorString(e));
     attr_done = true;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(WAVES_M * WAVES_N * 64), smem, stream, p);
+  hipLaunchKernelGGL(kern, grid, dim3(threads), smem, stream, p);
   return launch_status(name);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE>
+static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
+  static bool attr_done = false;
+  return launch_with_lds(gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE>, attr_done,
+                         tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), WAVES_M * WAVES_N * 64, p, grid, stream, name);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS>
+static int launch_grouped(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
+  static bool attr_done = false;
+  constexpr int big = tile_lds_bytes<BM, BN, NS, true>(), small = tile_lds_bytes<SBM, BN, SNS, true>();
+  return launch_with_lds(gemm_grouped_kernel<BM, BN, WAVES_M, WAVES_N, NS, SBM, SWAVES_M, SWAVES_N, SNS>, attr_done,
+                         big > small ? big : small, WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
 
 // Sums the split-K partial results in split order (deterministic), applies the row / tensor
@@ -530,25 +570,29 @@ int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_
 
 static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, dim3 grid, hipStream_t stream) {
   if (blockscale) {
-    if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, true, false>(p, grid, stream, "gemm_tiled_block_256x256");
-    if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, true, false>(p, grid, stream, "gemm_tiled_block_256x128");
-    if (variant == 4) return launch_tiled<128, 128, 2, 2, 3, true, false>(p, grid, stream, "gemm_tiled_block_128x128x3");
-    return launch_tiled<128, 128, 2, 2, 2, true, false>(p, grid, stream, "gemm_tiled_block_128x128");
+    if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, true>(p, grid, stream, "gemm_tiled_block_256x256");
+    if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, true>(p, grid, stream, "gemm_tiled_block_256x128");
+    if (variant == 4) return launch_tiled<128, 128, 2, 2, 3, true>(p, grid, stream, "gemm_tiled_block_128x128x3");
+    return launch_tiled<128, 128, 2, 2, 2, true>(p, grid, stream, "gemm_tiled_block_128x128");
   }
-  if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false, false>(p, grid, stream, "gemm_tiled_row_256x256");
-  if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, false, false>(p, grid, stream, "gemm_tiled_row_256x128");
-  return launch_tiled<128, 128, 2, 2, 2, false, false>(p, grid, stream, "gemm_tiled_row_128x128");
+  if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false>(p, grid, stream, "gemm_tiled_row_256x256");
+  if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, false>(p, grid, stream, "gemm_tiled_row_256x128");
+  return launch_tiled<128, 128, 2, 2, 2, false>(p, grid, stream, "gemm_tiled_row_128x128");
 }
 
-int gemm_grouped_dispatch(const GemmArgs& p, int64_t T, hipStream_t stream) {
-  // every active slot owns at most ceil(rows / BM) m-tiles: their sum is <= T / BM + num_active
-  const bool big = tile_override() == 2;
+int gemm_grouped_dispatch(const GemmArgs& p_in, int64_t T, hipStream_t stream) {
+  GemmArgs p = p_in;
+  // a slot owns one small tile or ceil(rows / BM) tiles: their sum is <= T / BM + num_active
+  // MAXFP8_TILE=2: 256-row tiles; MAXFP8_TILE=3: no small tiles (tuning runs)
+  const int tune = tile_override();
+  const bool big = tune == 2;
   const int bm = big ? 256 : 128;
+  p.small_rows = tune == 3 ? 0 : (big ? 64 : 32);
   const int64_t m_tiles = T / bm + p.num_active;
   if (m_tiles > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: %lld row tiles exceed the launch limit", (long long)m_tiles);
   const dim3 grid((unsigned)ceil_div(p.N, 128), (unsigned)m_tiles);
-  if (big) return launch_tiled<256, 128, 4, 2, 3, true, true>(p, grid, stream, "gemm_grouped_block_256x128");
-  return launch_tiled<128, 128, 2, 2, 2, true, true>(p, grid, stream, "gemm_grouped_block_128x128");
+  if (big) return launch_grouped<256, 128, 4, 2, 3, 64, 1, 8, 3>(p, grid, stream, "gemm_grouped_block_256x128");
+  return launch_grouped<128, 128, 2, 2, 2, 32, 1, 4, 3>(p, grid, stream, "gemm_grouped_block_128x128");
 }
 
 }  // namespace maxfp8
