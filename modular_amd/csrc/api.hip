@@ -146,6 +146,7 @@ int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, cons
   p.b_scale_stride = tensor ? 0 : b_scales_ld;
   p.c_dtype = c_dtype;
   p.c_vec_ok = (ldc % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
+  p.c_vec8_ok = (ldc % 8 == 0) && is_aligned(c, 16);
   if (algo == MAXFP8_ALGO_SKINNY) return gemm_skinny_dispatch(p, block, st);
   if (workspace && !is_aligned(workspace, 16)) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "matmul: workspace must be 16-byte aligned");
   p.workspace = (float*)workspace;
@@ -197,6 +198,7 @@ int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void*
   p.b_scales_ld = ceil_div(K, 128);
   p.c_dtype = c_dtype;
   p.c_vec_ok = (N % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
+  p.c_vec8_ok = (N % 8 == 0) && is_aligned(c, 16);
   p.offsets = expert_start_indices;
   p.expert_ids = expert_ids;
   p.num_active = (int)num_active_experts;

@@ -16,6 +16,7 @@ struct GemmArgs {
   int64_t a_scale_stride, b_scale_stride;
   int c_dtype;
   int c_vec_ok;            // C base and ldc allow 4-element vector stores
+  int c_vec8_ok;           // ... and 8-element ones (16-byte aligned rows)
   // grouped only
   const uint32_t* offsets;
   const int32_t* expert_ids;

@@ -76,27 +76,30 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   const int cols_here = (p.N - n0) < BN ? (p.N - n0) : BN;
 
   const int lm = lane & 15, lq = lane >> 4;
-  auto store4 = [&](int64_t m, int n, float v0, float v1, float v2, float v3) {
+  // A lane ends up with 8 consecutive columns of one row (see the weight fragment plan below):
+  // one 16-byte store for bf16, two for f32.
+  auto store8 = [&](int64_t m, int n, const v4f& lo, const v4f& hi) {
+    const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     if (p.c_dtype == MAXFP8_BF16) {
       uint16_t* dst = reinterpret_cast<uint16_t*>(p.c) + m * p.ldc + n;
-      if (p.c_vec_ok && n + 3 < p.N) {
-        const uint32_t lo = f32_to_bf16_bits(v0) | (f32_to_bf16_bits(v1) << 16);
-        const uint32_t hi = f32_to_bf16_bits(v2) | (f32_to_bf16_bits(v3) << 16);
-        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
-      } else {
-        const float v[4] = {v0, v1, v2, v3};
+      if (p.c_vec8_ok && n + 7 < p.N) {
+        uint32_t w[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i) w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+        *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
           if (n + i < p.N) dst[i] = (uint16_t)f32_to_bf16_bits(v[i]);
       }
     } else {
       float* dst = reinterpret_cast<float*>(p.c) + m * p.ldc + n;
-      if (p.c_vec_ok && n + 3 < p.N) {
-        *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
+      if (p.c_vec_ok && n + 7 < p.N) {
+        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
       } else {
-        const float v[4] = {v0, v1, v2, v3};
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 8; ++i)
           if (n + i < p.N) dst[i] = v[i];
       }
     }
@@ -108,10 +111,14 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   const __amdgpu_buffer_rsrc_t a_rsrc = t2_rsrc(a_tile, t2_clamp_u32((int64_t)(rows_here - 1) * p.lda + p.K));
   const __amdgpu_buffer_rsrc_t b_rsrc = t2_rsrc(b_tile, t2_clamp_u32((int64_t)(cols_here - 1) * p.ldb + p.K));
   const int cr = lane >> 3, cp = lane & 7;
-  // tile row of instruction i is (i*NWAVES + wave)*8 + cr, so row & 7 == cr
+  // tile row of instruction i is (i*NWAVES + wave)*8 + cr, so row & 7 == cr and (row >> 3) & 1 ==
+  // wave & 1.  Activation rows keep logical chunk c at c ^ (row & 7); weight rows at
+  // c ^ (4 * ((row >> 3) & 1) + (row & 3)), which is what keeps their fragment reads (rows
+  // 0-3 and 8-11 of a 32-row group in one instruction) free of bank conflicts.
   const int cchunk = cp ^ cr;
+  const int cchunk_b = cp ^ (((wave & 1) << 2) | (cr & 3));
   const uint32_t a_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.lda + cchunk * 16;
-  const uint32_t b_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.ldb + cchunk * 16;
+  const uint32_t b_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.ldb + cchunk_b * 16;
   const uint32_t a_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.lda;
   const uint32_t b_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.ldb;
   const int nslab = (p.K + 127) / 128;
@@ -143,8 +150,9 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   // zeros into a stage that is not read again; that keeps the loop free of branches)
   auto dma_one = [&](int slab, int buf, int idx, uint32_t dead) {
     const uint32_t koff = (uint32_t)slab * 128u;
-    uint32_t kill = dead;
+    uint32_t kill = dead, kill_b = dead;
     if (koff + cchunk * 16 >= (uint32_t)p.K) kill = 0x80000000u;
+    if (koff + cchunk_b * 16 >= (uint32_t)p.K) kill_b = 0x80000000u;
     uint8_t* sa = smem + buf * STAGE_BYTES + wave * 1024;
     uint8_t* sb = sa + BM * 128;
     if (idx < IA) {
@@ -152,7 +160,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
                                                koff + idx * a_istep, 0, 0);
     } else if (idx < IA + IB) {
       const int i = idx - IA;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(sb + i * NWAVES * 1024), 16, b_voff | kill,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(sb + i * NWAVES * 1024), 16, b_voff | kill_b,
                                                koff + i * b_istep, 0, 0);
     } else if constexpr (BLOCKSCALE) {
       // 64 scales of the slab's row of the transposed scale matrix per wave; with more waves
@@ -180,6 +188,20 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   auto read_frag = [&](const uint8_t* base) -> v8i {
     const v4i lo = *reinterpret_cast<const v4i*>(base + frag0);
     const v4i hi = *reinterpret_cast<const v4i*>(base + frag1);
+    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+  // Weight fragments come in pairs (t = 2q, 2q+1) over 32 weight rows: MFMA row i of the even
+  // fragment is weight row 8*(i/4) + i%4 of the group, of the odd fragment 4 more.  The MFMA
+  // leaves rows 4*(lane/16) .. +3 in a lane, so the pair gives a lane 8 consecutive columns of C.
+  static_assert(TN % 2 == 0, "weight fragments are read in pairs");
+  const int wrow = 8 * (lm >> 2) + (lm & 3);                      // row in the 32-row group (even fragment)
+  const int wsw = (((wrow >> 3) & 1) << 2) | (wrow & 3);          // same for the odd fragment (rows + 4)
+  const uint32_t wfrag0 = wrow * 128 + ((lq ^ wsw) << 4);
+  const uint32_t wfrag1 = wrow * 128 + (((lq + 4) ^ wsw) << 4);
+  auto read_wfrag = [&](const uint8_t* base, int t) -> v8i {
+    const uint8_t* g = base + (t >> 1) * 4096 + (t & 1) * 512;
+    const v4i lo = *reinterpret_cast<const v4i*>(g + wfrag0);
+    const v4i hi = *reinterpret_cast<const v4i*>(g + wfrag1);
     return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
 
@@ -234,7 +256,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     const uint32_t dead = slab + NS - 1 < slab_end ? 0u : 0x80000000u;
     const int dma_slab = slab + NS - 1, dma_buf = buf == 0 ? NS - 1 : buf - 1;
 #ifndef MAXFP8_DMA_SPREAD
-#define MAXFP8_DMA_SPREAD TM
+#define MAXFP8_DMA_SPREAD (NS == 2 && TM >= 4 ? TM / 2 : TM)
 #endif
     constexpr int SPREAD = MAXFP8_DMA_SPREAD < 1 ? 1 : (MAXFP8_DMA_SPREAD > TM ? TM : MAXFP8_DMA_SPREAD);
 
@@ -246,7 +268,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     }
     v8i bf[TN];
 #pragma unroll
-    for (int t = 0; t < TN; ++t) bf[t] = read_frag(sa + b_frag_base + t * 2048);
+    for (int t = 0; t < TN; ++t) bf[t] = read_wfrag(sa + b_frag_base, t);
     v8i af = read_frag(sa + a_frag_base);
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) {
@@ -286,15 +308,17 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
       if (ml >= rows_here) continue;
       float* row = ws + (row_begin + ml) * p.N;
 #pragma unroll
-      for (int nt = 0; nt < TN; ++nt) {
-        const int n = n0 + wn * WN + nt * 16 + lq * 4;
+      for (int q = 0; q < TN / 2; ++q) {
+        const int n = n0 + wn * WN + q * 32 + lq * 8;
         if (n >= p.N) continue;
-        const v4f v = acc[mt][nt];
-        if ((p.N & 3) == 0) {
-          *reinterpret_cast<float4*>(row + n) = make_float4(v[0], v[1], v[2], v[3]);
+        const v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
+        if ((p.N & 3) == 0 && n + 7 < p.N) {
+          *reinterpret_cast<float4*>(row + n) = make_float4(lo[0], lo[1], lo[2], lo[3]);
+          *reinterpret_cast<float4*>(row + n + 4) = make_float4(hi[0], hi[1], hi[2], hi[3]);
         } else {
+          const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
+          for (int i = 0; i < 8; ++i)
             if (n + i < p.N) row[n + i] = v[i];
         }
       }
@@ -309,23 +333,24 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     float a_s = 1.f;
     if constexpr (!BLOCKSCALE) a_s = p.a_scales[m * p.a_scale_stride];
 #pragma unroll
-    for (int nt = 0; nt < TN; ++nt) {
-      const int n = n0 + wn * WN + nt * 16 + lq * 4;
+    for (int q = 0; q < TN / 2; ++q) {
+      const int n = n0 + wn * WN + q * 32 + lq * 8;
       if (n >= p.N) continue;
-      v4f v = acc[mt][nt];
+      v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
       if constexpr (!BLOCKSCALE) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int nn = (n + i < p.N) ? n + i : p.N - 1;
-          const float t = v[i] * a_s;
-          v[i] = t * p.b_scales[(int64_t)nn * p.b_scale_stride];
+          const int n_lo = (n + i < p.N) ? n + i : p.N - 1;
+          const int n_hi = (n + 4 + i < p.N) ? n + 4 + i : p.N - 1;
+          const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
+          lo[i] = t_lo * p.b_scales[(int64_t)n_lo * p.b_scale_stride];
+          hi[i] = t_hi * p.b_scales[(int64_t)n_hi * p.b_scale_stride];
         }
       }
-      store4(m, n, v[0], v[1], v[2], v[3]);
+      store8(m, n, lo, hi);
     }
   }
 }
-
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
@@ -591,7 +616,7 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, int64_t T, hipStream_t stream) {
   const int64_t m_tiles = T / bm + p.num_active;
   if (m_tiles > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: %lld row tiles exceed the launch limit", (long long)m_tiles);
   const dim3 grid((unsigned)ceil_div(p.N, 128), (unsigned)m_tiles);
-  if (big) return launch_grouped<256, 128, 4, 2, 3, 64, 1, 8, 3>(p, grid, stream, "gemm_grouped_block_256x128");
+  if (big) return launch_grouped<256, 128, 4, 2, 3, 64, 2, 4, 3>(p, grid, stream, "gemm_grouped_block_256x128");
   return launch_grouped<128, 128, 2, 2, 2, 32, 1, 4, 3>(p, grid, stream, "gemm_grouped_block_128x128");
 }
 
