@@ -503,17 +503,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
 }
 
 // ---- kernel selection ------------------------------------------------------------------------
-// Three tile shapes.  `t_slab` is the measured time one block spends per 128-byte K slab when
-// the whole chip is busy (microseconds); the cost of a shape is rounds * t_slab, with
-// rounds = ceil(tiles / resident blocks).
-struct TileShape { int bm, bn, slots; float t_slab_block, t_slab_row; };
+// Three tile shapes.  A block spends t_slab microseconds per 128-byte K slab and t_tile on the
+// rest of a tile (pipeline fill, the store burst at the end), both measured with the whole chip
+// busy and weights coming from HBM; the cost of a shape is rounds * (slabs * t_slab + t_tile)
+// with rounds = ceil(tiles / resident blocks).
+struct TileShape { int bm, bn, slots; float t_slab_block, t_slab_row, t_tile; };
 static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, dim3 grid, hipStream_t stream);
 
 static const TileShape kShapes[4] = {
-    {256, 256, 256, 2.05f, 1.70f},   // 8 waves, 2 stages
-    {256, 128, 256, 1.10f, 1.00f},   // 8 waves, 3 stages
-    {128, 128, 512, 1.20f, 1.05f},   // 4 waves, 2 stages, two blocks per CU
-    {128, 128, 256, 9.99f, 9.99f},   // 4 waves, 3 stages, one block per CU (tuning only)
+    {256, 256, 256, 1.63f, 1.40f, 11.4f},   // 8 waves, 2 stages
+    {256, 128, 256, 0.92f, 0.82f, 9.0f},    // 8 waves, 3 stages
+    {128, 128, 512, 0.96f, 0.86f, 11.4f},   // 4 waves, 2 stages, two blocks per CU
+    {128, 128, 256, 9.99f, 9.99f, 9.0f},    // 4 waves, 3 stages, one block per CU (tuning only)
 };
 
 // MAXFP8_TILE=1/2/3 forces a shape (for tuning runs); anything else lets the cost model pick.
@@ -540,7 +541,7 @@ static int pick_splits(int64_t tiles, int slots, int nslab) {
   return (nslab + per - 1) / per;  // no empty share
 }
 
-// cost of a shape (microseconds) = rounds of resident blocks * slabs per block * time per slab
+// cost of a shape (microseconds) = rounds of resident blocks * time of one tile
 static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can_split) {
   int best = 0;
   float best_cost = 0.f;
@@ -548,8 +549,8 @@ static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can
     const TileShape& t = kShapes[i];
     const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
     const int sp = can_split ? pick_splits(tiles, t.slots, nslab) : 1;
-    float cost = (float)ceil_div(tiles * sp, t.slots) * (float)ceil_div(nslab, sp) *
-                 (blockscale ? t.t_slab_block : t.t_slab_row);
+    float cost = (float)ceil_div(tiles * sp, t.slots) *
+                 ((float)ceil_div(nslab, sp) * (blockscale ? t.t_slab_block : t.t_slab_row) + t.t_tile);
     // a split pays a second launch and one write + one read of sp * M * N f32 partial sums (~4 TB/s)
     if (sp > 1) cost += 5.0f + (float)sp * (float)M * (float)N * 8.0f / 4.0e6f;
     if (i == 0 || cost < best_cost) { best = i; best_cost = cost; }
