@@ -35,7 +35,8 @@ typedef enum maxfp8_status {
   MAXFP8_ERR_GRANULARITY = -4, /* unsupported scaling granularity combination  */
   MAXFP8_ERR_LAUNCH = -5,      /* HIP reported an error at launch              */
   MAXFP8_ERR_NULL = -6,        /* required pointer was NULL                    */
-  MAXFP8_ERR_WORKSPACE = -7    /* workspace missing or too small               */
+  MAXFP8_ERR_WORKSPACE = -7    /* reserved: a missing or short workspace is not an
+                                  error, the matmul then runs without split-K  */
 } maxfp8_status;
 
 typedef enum maxfp8_dtype {
@@ -110,8 +111,12 @@ int maxfp8_quantize_dynamic_scaled_fp8(
  *
  *   scales_dtype MAXFP8_F32 (block requires it) or MAXFP8_BF16 (rowwise/tensor).
  *   algo        a maxfp8_algo value.
- *   workspace   optional device scratch for split-K (may be NULL: then kernels
- *               that need none are used).
+ *   workspace   optional device scratch for split-K, 16-byte aligned, of
+ *               workspace_bytes bytes (maxfp8_matmul_workspace_bytes gives the
+ *               size that allows every split the library would choose).  NULL
+ *               or too small: the matmul runs unsplit, which is slower only
+ *               when its tiles cover a small part of the chip.  The contents
+ *               are scratch: overwritten by the call, meaningless afterwards.
  */
 int maxfp8_matmul_dynamic_scaled_fp8(
     void* c, const void* a, const void* b,

@@ -1,0 +1,160 @@
+"""Every tile shape, the split-K path and the workspace contract of the tiled MFMA matmul,
+and the two tile kinds of the grouped kernel, on cases whose arithmetic is exact (small
+integers, power-of-two scales: any summation order gives the same f32) plus tolerance checks
+against the CPU oracle.  The shapes cut tiles in M, N and K and leave N off the 8-column store
+width, which is where the edge handling of the kernels lives."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import modular_amd as mx
+import oracle
+from modular_amd import _lib, synth
+from test_gpu_matmul import BLK, ROW, TOL, exact_case, make_block, mm, oracle_block
+from test_gpu_grouped import make as make_grouped, ref as ref_grouped, run as run_grouped
+from util import F32_BUDGET, assert_rel, f32_np, fp8_bytes, fp8_from_bytes
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("tile", ["1", "2", "3", "4"])
+@pytest.mark.parametrize("M,N,K", [(300, 392, 1040), (257, 100, 512), (64, 129, 384), (513, 520, 256)])
+def test_each_tile_shape_exact(dev, monkeypatch, tile, M, N, K):
+    monkeypatch.setenv("MAXFP8_TILE", tile)
+    a, b, sa, sb, want = exact_case(M, N, K, seed=M + N + K)
+    got = f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled")).astype(np.float64)
+    bad = np.argwhere(got != want)
+    assert bad.size == 0, f"tile {tile}: {len(bad)} mismatches, first at {bad[:4].tolist()}"
+    cb = mm(a, b, sa, sb, BLK, dev, out=torch.bfloat16, algo="tiled")
+    assert torch.equal(cb.cpu(), torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("tile", ["1", "2", "3"])
+def test_each_tile_shape_rowwise(dev, monkeypatch, tile):
+    monkeypatch.setenv("MAXFP8_TILE", tile)
+    M, N, K = 300, 1044, 1024
+    a, b = synth.random_fp8((M, K), M), synth.random_fp8((N, K), N)
+    sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+    ref = oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), sa.numpy(), sb.numpy())
+    for out in (torch.float32, torch.bfloat16):
+        assert_rel(f32_np(mm(a, b, sa, sb, ROW, dev, out=out, algo="tiled")), ref, TOL, f"tile {tile} {out}",
+                   F32_BUDGET if out == torch.float32 else None)
+
+
+@pytest.mark.parametrize("splits", ["2", "3", "4"])
+@pytest.mark.parametrize("kind", ["block", "row"])
+def test_split_k_exact(dev, monkeypatch, splits, kind):
+    # forced split counts (at most one per 4 slabs); the shares are uneven (17 slabs)
+    monkeypatch.setenv("MAXFP8_SPLITK", splits)
+    M, N, K = 130, 264, 17 * 128
+    if kind == "block":
+        a, b, sa, sb, want = exact_case(M, N, K, seed=int(splits))
+        cfg = BLK
+    else:
+        rng = np.random.default_rng(7)
+        ai, bi = rng.integers(-4, 5, (M, K)), rng.integers(-4, 5, (N, K))
+        a = fp8_from_bytes(oracle.e4m3fn_encode(ai.astype(np.float32)))
+        b = fp8_from_bytes(oracle.e4m3fn_encode(bi.astype(np.float32)))
+        sa = torch.from_numpy(np.exp2(rng.integers(-3, 3, (1, M))).astype(np.float32))
+        sb = torch.from_numpy(np.exp2(rng.integers(-3, 3, (N, 1))).astype(np.float32))
+        want = (ai @ bi.T) * sa.numpy().reshape(-1, 1) * sb.numpy().reshape(1, -1)
+        cfg = ROW
+    assert _lib.lib().maxfp8_matmul_workspace_bytes(M, N, K) >= int(splits) * M * N * 4
+    got = f32_np(mm(a, b, sa, sb, cfg, dev, algo="tiled")).astype(np.float64)
+    assert np.array_equal(got, want)
+    cb = mm(a, b, sa, sb, cfg, dev, out=torch.bfloat16, algo="tiled")
+    assert torch.equal(cb.cpu(), torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16))
+
+
+def test_split_k_chosen_for_a_small_grid(dev):
+    # 2 x 2 tiles of 128 on a 256-CU chip with K = 8192: the cost model splits K when it is
+    # given workspace; with and without it the result meets the tolerance
+    M, N, K = 256, 256, 8192
+    assert _lib.lib().maxfp8_matmul_workspace_bytes(M, N, K) > 0
+    a, b, sa, sb = make_block(M, N, K, seed=5)
+    ref = oracle_block(a, b, sa, sb)
+    c_split = f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled"))
+    assert_rel(c_split, ref, TOL, "split-K", F32_BUDGET)
+    c_plain = f32_np(_call_abi(a, b, sa, sb, dev, workspace=None))
+    assert_rel(c_plain, ref, TOL, "no workspace", F32_BUDGET)
+
+
+def _call_abi(a, b, sa, sb, dev, workspace, workspace_bytes=0, algo=2):
+    """maxfp8_matmul_dynamic_scaled_fp8 through the C ABI, blockwise 1x128 / 128x128, f32 out."""
+    L = _lib.lib()
+    a, b, sa, sb = a.to(dev), b.to(dev), sa.to(dev), sb.to(dev)
+    M, K = a.shape
+    N = b.shape[0]
+    c = torch.empty((M, N), dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = L.maxfp8_matmul_dynamic_scaled_fp8(
+        ctypes.c_void_p(c.data_ptr()), ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()),
+        ctypes.c_void_p(sa.data_ptr()), ctypes.c_void_p(sb.data_ptr()), M, N, K, K, K, N,
+        3, 3, 1, 128, 128, sa.shape[1], sb.shape[1], 2, 2, algo,
+        ctypes.c_void_p(workspace), workspace_bytes, ctypes.c_void_p(stream))
+    torch.cuda.synchronize()
+    if rc != 0:
+        raise RuntimeError((rc, L.maxfp8_last_error().decode()))
+    return c
+
+
+def test_workspace_contract(dev):
+    M, N, K = 256, 256, 8192
+    a, b, sa, sb = make_block(M, N, K, seed=9)
+    need = _lib.lib().maxfp8_matmul_workspace_bytes(M, N, K)
+    ws = torch.empty(need + 64, dtype=torch.uint8, device=dev)
+    full = _call_abi(a, b, sa, sb, dev, ws.data_ptr(), need)
+    # a workspace that is too small is not an error: the matmul runs unsplit
+    small = _call_abi(a, b, sa, sb, dev, ws.data_ptr(), 1024)
+    plain = _call_abi(a, b, sa, sb, dev, None)
+    assert torch.equal(small, plain)
+    assert_rel(f32_np(full), f32_np(plain), 1e-4, "split vs unsplit", F32_BUDGET)
+    # a misaligned workspace is refused
+    with pytest.raises(RuntimeError) as e:
+        _call_abi(a, b, sa, sb, dev, ws.data_ptr() + 4, need)
+    assert e.value.args[0][0] == -3  # MAXFP8_ERR_ALIGN
+
+
+GROUPED = [
+    # small tiles (<= 32 rows), big tiles, their boundaries, empty slots, a slot without expert
+    ([0, 1, 31, 32, 33, 129, 300], [3, 0, 6, 1, -1, 2, 5], 7, 200, 384),
+    ([32] * 6, [5, 4, 3, 2, 1, 0], 6, 100, 256),
+    ([1, 257, 2, 128], [0, 1, 2, 3], 4, 392, 512),
+]
+
+
+@pytest.mark.parametrize("tile", ["0", "2", "3"])
+@pytest.mark.parametrize("counts,ids,E,N,K", GROUPED)
+@pytest.mark.parametrize("out", [torch.float32, torch.bfloat16])
+def test_grouped_tile_kinds(dev, monkeypatch, tile, counts, ids, E, N, K, out):
+    monkeypatch.setenv("MAXFP8_TILE", tile)
+    args = make_grouped(counts, ids, E, N, K, seed=sum(counts) + N)
+    c = run_grouped(*args, max(counts), len(counts), dev, out=out, algo="tiled")
+    assert_rel(f32_np(c), ref_grouped(*args, max(counts), len(counts)), TOL, f"grouped {counts} tile {tile}",
+               F32_BUDGET if out == torch.float32 else None)
+
+
+def test_grouped_small_tiles_exact(dev):
+    # integer data and power-of-two scales through the small-tile path: bit-exact
+    rng = np.random.default_rng(3)
+    counts, E, N, K = [5, 32, 17, 0, 9], 5, 264, 640
+    T = sum(counts)
+    ai, bi = rng.integers(-4, 5, (T, K)), rng.integers(-4, 5, (E, N, K))
+    a = fp8_from_bytes(oracle.e4m3fn_encode(ai.astype(np.float32)))
+    b = fp8_from_bytes(oracle.e4m3fn_encode(bi.astype(np.float32).reshape(E * N, K))).reshape(E, N, K)
+    kb, nb = K // 128, -(-N // 128)
+    ea, eb = rng.integers(-3, 4, (kb, -(-T // 4) * 4)), rng.integers(-3, 4, (E, nb, kb))
+    sa = torch.from_numpy(np.exp2(ea).astype(np.float32))
+    sb = torch.from_numpy(np.exp2(eb).astype(np.float32))
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32)
+    ids = torch.tensor([4, 2, 0, 1, 3], dtype=torch.int32)
+    want = np.zeros((T, N))
+    for z, e in enumerate(ids.tolist()):
+        r0, r1 = int(off[z]), int(off[z + 1])
+        for j in range(kb):
+            part = ai[r0:r1, j * 128:(j + 1) * 128] @ bi[e][:, j * 128:(j + 1) * 128].T
+            want[r0:r1] += part * np.exp2(ea[j, r0:r1])[:, None] * np.exp2(eb[e][np.arange(N) // 128, j])[None, :]
+    c = run_grouped(a, b, sa, sb, off, ids, max(counts), len(counts), dev, algo="tiled")
+    assert np.array_equal(f32_np(c).astype(np.float64), want)
