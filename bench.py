@@ -240,7 +240,7 @@ def result_line(name, steps, warmup, with_cpu=True):
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = measured_traffic(name)
     roof["algorithmic_bytes"] = mm_bytes
-    roof["kernel"] = {"grouped": "gemm_tiled_kernel<128,128,...,grouped>", "row": "gemm_skinny_kernel"}.get(
+    roof["kernel"] = {"grouped": "gemm_grouped_kernel", "row": "gemm_skinny_kernel"}.get(
         kind, "gemm_skinny_kernel" if M <= 64 else "gemm_tiled_kernel")
     roof["kernel_ms_avg"], roof["kernel_ms_median"], roof["kernel_ms_min"] = mm_avg, mm_med, mm_min
     out = {
