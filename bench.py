@@ -59,6 +59,9 @@ WORKLOADS = {
     # configs[4]: DeepSeek-V3 MoE grouped GEMM, 256 experts, 32768 routed rows
     "moe_gate_up": ("grouped", 32768, 7168, 4096),
     "moe_down": ("grouped", 32768, 2048, 7168),
+    # the step before a per-token FP8 linear: RMSNorm fused with the dynamic quantisation (N unused)
+    "rmsnorm_quant_m4096_k7168": ("rmsq", 4096, 7168, 0),
+    "rmsnorm_quant_m32768_k7168": ("rmsq", 32768, 7168, 0),
 }
 DEFAULT = "llama8b_gate_up_m2048"
 
@@ -99,7 +102,15 @@ class Workload:
         self.dev = dev
         self.mx = mx
         kind, M, K, N = self.kind, self.M, self.K, self.N
-        self.cfg = mx.rowwise_fp8_config() if kind == "row" else mx.blockwise_fp8_config()
+        self.cfg = mx.rowwise_fp8_config() if kind in ("row", "rmsq") else mx.blockwise_fp8_config()
+        if kind == "rmsq":
+            self.copies = max(2, min(8, math.ceil(CACHE_BUST_BYTES / (3 * M * K)) + 1))
+            self.x = [synth.activations(M, K, seed=c, outlier_frac=0.01, device=dev) for c in range(self.copies)]
+            g = torch.Generator(device="cpu").manual_seed(7)
+            self.gamma = (1.0 + 0.1 * torch.randn(K, generator=g)).to(torch.bfloat16).to(dev)
+            self.w, self.ws = [None] * self.copies, [None] * self.copies
+            torch.cuda.synchronize()
+            return
         E = 256 if kind == "grouped" else 1
         w_bytes = E * N * K
         per_copy = w_bytes + 2 * M * K + 2 * M * N
@@ -129,11 +140,16 @@ class Workload:
 
     def quantise(self, c):
         import torch
+        if self.kind == "rmsq":
+            return (None, None)
         return self.mx.quantize_dynamic_scaled_float8(self.x[c], self.cfg.input_scale, self.cfg.weight_scale,
                                                       scales_type=torch.float32)
 
     def matmul(self, c, q, sa):
+        """the workload's dominant kernel (the fused norm + quantise itself for the rmsq kind)"""
         mx, cfg = self.mx, self.cfg
+        if self.kind == "rmsq":
+            return mx.rms_norm_fused_quantize_dynamic_scaled_fp8(self.x[c], self.gamma, 1e-6)
         if self.kind == "grouped":
             return mx.grouped_dynamic_scaled_fp8_matmul(q, self.w[c], sa, self.ws[c], self.off, self.ids, self.stats,
                                                         cfg.input_scale, cfg.weight_scale)
@@ -189,6 +205,19 @@ def cpu_baseline(wl, budget_s=15.0):
     threads = oracle.default_threads()
     kind, M, K, N = wl.kind, wl.M, wl.K, wl.N
     x = wl.x[0].cpu()
+    if kind == "rmsq":
+        import torch
+        rows = min(M, 4096)
+        xb = x[:rows].contiguous().view(torch.int16).numpy().view(np.uint16)
+        gb = wl.gamma.cpu().view(torch.int16).numpy().view(np.uint16)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < budget_s / 3 or reps == 0:
+            oracle.rms_norm_fused_quantize(xb, gb, 1e-6, threads=threads)
+            reps += 1
+        t = (time.perf_counter() - t0) / reps
+        return {"value": 3.0 * rows * K / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": f"oracle rms_norm_fused_quantize on rows 0..{rows - 1} of M={M}, K={K}: {t:.3f} s per pass, {reps} passes"}
     w = wl.w[0] if kind != "grouped" else wl.w[0][0]
     ws = wl.ws[0] if kind != "grouped" else wl.ws[0][0]
     wb = w.cpu().view(__import__("torch").uint8).numpy()
@@ -226,11 +255,13 @@ def result_line(name, steps, warmup, with_cpu=True):
     wl, ms_step, mm_avg, mm_med, mm_min = run_gpu(name, steps, warmup)
     kind, M, K, N = wl.kind, wl.M, wl.K, wl.N
     flops, mm_bytes, q_bytes = algorithmic(kind, M, K, N)
+    if kind == "rmsq":
+        flops, mm_bytes, q_bytes = 0.0, 3 * M * K + 2 * K + 4 * M, 0
     if kind == "grouped":
         # weights of every expert that received tokens are streamed once (experts without tokens are never read)
         active = int((wl.counts > 0).sum())
         mm_bytes += (active - 1) * N * K + 4 * (active - 1) * math.ceil(N / 128) * (K // 128)
-    hbm_bound = kind == "row" or M <= 16
+    hbm_bound = kind in ("row", "rmsq") or M <= 16
     if hbm_bound:
         value, unit = (mm_bytes + q_bytes) / (ms_step * 1e-3) / 1e9, "GB/s"
         roof = {"bound": "hbm", "achieved": mm_bytes / (mm_avg * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s"}
@@ -240,7 +271,7 @@ def result_line(name, steps, warmup, with_cpu=True):
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = measured_traffic(name)
     roof["algorithmic_bytes"] = mm_bytes
-    roof["kernel"] = {"grouped": "gemm_grouped_kernel", "row": "gemm_skinny_kernel"}.get(
+    roof["kernel"] = {"grouped": "gemm_grouped_kernel", "row": "gemm_skinny_kernel", "rmsq": "rmsnorm_quant_row_bf16_kernel"}.get(
         kind, "gemm_skinny_kernel" if M <= 64 else "gemm_tiled_kernel")
     roof["kernel_ms_avg"], roof["kernel_ms_median"], roof["kernel_ms_min"] = mm_avg, mm_med, mm_min
     out = {
@@ -248,8 +279,10 @@ def result_line(name, steps, warmup, with_cpu=True):
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8_e4m3fn (f32 accumulate, bf16 out)", "data": "synthetic",
         "config": {"workload": name, "M": M, "K": K, "N": N,
-                   "scaling": "per-token x per-channel" if kind == "row" else "1x128 activations, 128x128 weights",
-                   "step": "dynamic quantise + " + ("grouped " if kind == "grouped" else "") + "scaled matmul",
+                   "scaling": "per-token" if kind == "rmsq" else
+                              "per-token x per-channel" if kind == "row" else "1x128 activations, 128x128 weights",
+                   "step": "RMSNorm fused with dynamic quantise" if kind == "rmsq" else
+                           "dynamic quantise + " + ("grouped " if kind == "grouped" else "") + "scaled matmul",
                    "input_copies": wl.copies},
         "roofline": roof,
     }

@@ -158,6 +158,25 @@ int maxfp8_grouped_matmul_dynamic_scaled_fp8(
     int64_t a_scales_ld, int c_dtype, int scales_dtype, int algo, void* stream);
 
 /*
+ * mo.composite.rms_norm_fused_quantize_dynamic_scaled_fp8
+ *   (op registration: max/kernels/src/graph_compiler/builtin_kernels/quantization.mojo:112-237;
+ *    kernel: max/kernels/src/nn/normalization.mojo:3996-4175)
+ * RMSNorm over the last axis fused with the per-row (per-token) dynamic quantisation:
+ *   inv_rms = 1/sqrt(sum_c x[r,c]^2 / K + epsilon),  g'[c] = gamma[c] + weight_offset
+ *   scales[r] = min(max_c |x*g'| * inv_rms, scale_ub) / 448
+ *   out[r,c]  = e4m3fn(clamp(((x * inv_rms) * g'[c]) / scales[r]))   (as x * (1/scale))
+ * in [rows, K] and gamma [K] share in_dtype; out [rows, K] e4m3fn; out_scales [rows]
+ * (the op's [1, rows] tensor).  epsilon and weight_offset are rounded to in_dtype first,
+ * as the registration does (quantization.mojo:205-213).  Higher-rank inputs are passed
+ * flattened to [rows, K].
+ */
+int maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8(
+    void* out_fp8, void* out_scales, const void* in, const void* gamma,
+    int64_t rows, int64_t K, int64_t in_row_stride, int64_t out_row_stride,
+    int in_dtype, int scales_dtype, float epsilon, float weight_offset,
+    float scale_ub, void* stream);
+
+/*
  * Elementwise f32 -> e4m3fn (clamp to +-448, round to nearest even), the cast
  * inside fp8_quantize (max/kernels/src/internal_utils/fp8_utils.mojo:96-143).
  * Exposed so the hardware convert can be checked exhaustively.

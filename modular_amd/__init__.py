@@ -7,7 +7,7 @@ through the C ABI of include/maxfp8.h; there is no CPU or PyTorch fallback.
 from .quant_config import (InputScaleSpec, QuantConfig, QuantFormat, ScaleGranularity, ScaleOrigin,
                            WeightScaleSpec, blockwise_fp8_config, rowwise_fp8_config)
 from .kernels import (dynamic_scaled_matmul, grouped_dynamic_scaled_fp8_matmul,
-                      quantize_dynamic_scaled_float8)
+                      quantize_dynamic_scaled_float8, rms_norm_fused_quantize_dynamic_scaled_fp8)
 from .quant_ops import matmul_float8, quantized_matmul
 from .linear import Linear
 
@@ -15,5 +15,5 @@ __all__ = [
     "InputScaleSpec", "QuantConfig", "QuantFormat", "ScaleGranularity", "ScaleOrigin", "WeightScaleSpec",
     "blockwise_fp8_config", "rowwise_fp8_config", "dynamic_scaled_matmul",
     "grouped_dynamic_scaled_fp8_matmul", "quantize_dynamic_scaled_float8", "matmul_float8",
-    "quantized_matmul", "Linear",
+    "quantized_matmul", "Linear", "rms_norm_fused_quantize_dynamic_scaled_fp8",
 ]

@@ -25,6 +25,8 @@ int launch_status(const char* what) {
 // kernels (defined in the other translation units)
 int quantize_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, int,
                       float, hipStream_t);
+int rmsnorm_quantize_dispatch(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float,
+                              float, float, hipStream_t);
 int cast_f32_to_e4m3fn_dispatch(void*, const float*, int64_t, hipStream_t);
 int cast_e4m3fn_to_f32_dispatch(float*, const void*, int64_t, hipStream_t);
 int copy_bytes_dispatch(void*, const void*, int64_t, hipStream_t);
@@ -40,6 +42,21 @@ size_t gemm_tiled_workspace_bytes(int64_t, int64_t, int64_t);
 int gemm_grouped_dispatch(const GemmArgs&, int64_t, hipStream_t);
 int gemm_skinny_dispatch(const GemmArgs&, bool, hipStream_t);
 int gemm_skinny_max_m();
+
+// v rounded to bf16 / f16 and widened back: how an op parameter of the input's dtype arrives
+static float round_to_dtype(float v, int dtype) {
+  if (dtype == MAXFP8_BF16) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return v;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    u &= 0xffff0000u;
+    memcpy(&v, &u, 4);
+    return v;
+  }
+  if (dtype == MAXFP8_F16) return (float)(_Float16)v;
+  return v;
+}
 
 static bool is_aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
@@ -73,6 +90,25 @@ int maxfp8_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const vo
   if (!out_fp8 || !out_scales || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize: null pointer");
   return quantize_dispatch(out_fp8, out_scales, in, M, K, in_row_stride, out_row_stride, group_size, scales_ld,
                            in_dtype, scales_dtype, scale_ub, (hipStream_t)stream);
+}
+
+int maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, const void* gamma,
+                                                      int64_t rows, int64_t K, int64_t in_row_stride,
+                                                      int64_t out_row_stride, int in_dtype, int scales_dtype,
+                                                      float epsilon, float weight_offset, float scale_ub, void* stream) {
+  if (in_dtype != MAXFP8_BF16 && in_dtype != MAXFP8_F16 && in_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "rms_norm_fused_quantize: input dtype %d is not bf16, f16 or f32", in_dtype);
+  if (scales_dtype != MAXFP8_F32 && scales_dtype != MAXFP8_BF16)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "rms_norm_fused_quantize: scales dtype should be bfloat16 or float32 (got %d)", scales_dtype);
+  if (rows < 0 || K < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "rms_norm_fused_quantize: negative size");
+  if (rows == 0 || K == 0) return MAXFP8_OK;
+  if (rows >= ((int64_t)1 << 31) || K >= ((int64_t)1 << 31)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "rms_norm_fused_quantize: sizes must fit 31 bits");
+  if (in_row_stride < K || out_row_stride < K)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "rms_norm_fused_quantize: row strides smaller than the row length");
+  if (!out_fp8 || !out_scales || !in || !gamma) MAXFP8_FAIL(MAXFP8_ERR_NULL, "rms_norm_fused_quantize: null pointer");
+  return rmsnorm_quantize_dispatch(out_fp8, out_scales, in, gamma, rows, K, in_row_stride, out_row_stride, in_dtype,
+                                   scales_dtype, round_to_dtype(epsilon, in_dtype), round_to_dtype(weight_offset, in_dtype),
+                                   scale_ub, (hipStream_t)stream);
 }
 
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K) {

@@ -182,6 +182,125 @@ __global__ __launch_bounds__(256) void quant_generic_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// RMSNorm fused with per-row dynamic quantisation (max/kernels/src/nn/normalization.mojo:3996-4175):
+//   inv_rms = rsqrt(sum x^2 / K + eps);  g' = gamma + weight_offset (f32)
+//   row_max = max |x * g'| * inv_rms;  (scale, recip) from row_max
+//   out = e4m3fn(clamp(((x * inv_rms) * g') * recip))
+// One block (256 threads) per row; the row and gamma stay in registers between the two
+// reductions and the convert pass: the activations are read once (2 bytes in, 1 byte out per
+// element -- the unfused pair of kernels moves 2 + 2 + 2 + 1).
+template <int NV>
+__global__ __launch_bounds__(256) void rmsnorm_quant_row_bf16_kernel(
+    uint8_t* __restrict__ out, float* __restrict__ scales, const uint16_t* __restrict__ in,
+    const uint16_t* __restrict__ gamma, int K, int64_t in_stride, int64_t out_stride, float epsilon,
+    float weight_offset, float scale_ub) {
+  __shared__ float red_s[4], red_m[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const uint16_t* src = in + (int64_t)row * in_stride;
+  const int nvec = K >> 3;
+  uint4 v[NV], g[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * 256;
+    v[i] = idx < nvec ? reinterpret_cast<const uint4*>(src)[idx] : make_uint4(0, 0, 0, 0);
+    g[i] = idx < nvec ? reinterpret_cast<const uint4*>(gamma)[idx] : make_uint4(0, 0, 0, 0);
+  }
+  float ssq = 0.0f, amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+    const uint32_t gw[4] = {g[i].x, g[i].y, g[i].z, g[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float x0 = __uint_as_float(w[j] << 16), x1 = __uint_as_float(w[j] & 0xffff0000u);
+      const float g0 = __uint_as_float(gw[j] << 16) + weight_offset, g1 = __uint_as_float(gw[j] & 0xffff0000u) + weight_offset;
+      ssq += x0 * x0;
+      ssq += x1 * x1;
+      amax = fmaxf(amax, fabsf(x0 * g0));
+      amax = fmaxf(amax, fabsf(x1 * g1));
+    }
+  }
+  ssq = wave_sum(ssq);
+  amax = wave_max(amax);
+  if ((tid & 63) == 0) { red_s[tid >> 6] = ssq; red_m[tid >> 6] = amax; }
+  __syncthreads();
+  ssq = (red_s[0] + red_s[1]) + (red_s[2] + red_s[3]);
+  amax = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
+  const float inv_rms = 1.0f / __fsqrt_rn(ssq / (float)K + epsilon);
+  float scale, recip;
+  dynamic_scale_f32(amax * inv_rms, scale_ub, scale, recip);
+  if (tid == 0) scales[row] = scale;
+  uint8_t* dst = out + (int64_t)row * out_stride;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * 256;
+    if (idx < nvec) {
+      const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+      const uint32_t gw[4] = {g[i].x, g[i].y, g[i].z, g[i].w};
+      float f[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float g0 = __uint_as_float(gw[j] << 16) + weight_offset, g1 = __uint_as_float(gw[j] & 0xffff0000u) + weight_offset;
+        f[2 * j] = ((__uint_as_float(w[j] << 16) * inv_rms) * g0) * recip;
+        f[2 * j + 1] = ((__uint_as_float(w[j] & 0xffff0000u) * inv_rms) * g1) * recip;
+      }
+      int lo = 0, hi = 0;
+      lo = cvt_pk_e4m3fn(clamp448(f[0]), clamp448(f[1]), lo, false);
+      lo = cvt_pk_e4m3fn(clamp448(f[2]), clamp448(f[3]), lo, true);
+      hi = cvt_pk_e4m3fn(clamp448(f[4]), clamp448(f[5]), hi, false);
+      hi = cvt_pk_e4m3fn(clamp448(f[6]), clamp448(f[7]), hi, true);
+      reinterpret_cast<uint2*>(dst)[idx] = make_uint2((uint32_t)lo, (uint32_t)hi);
+    }
+  }
+}
+
+// any dtype, alignment and row length: three passes over global memory
+__global__ __launch_bounds__(256) void rmsnorm_quant_generic_kernel(
+    uint8_t* __restrict__ out, void* __restrict__ scales, const void* __restrict__ in, const void* __restrict__ gamma,
+    int K, int64_t in_stride, int64_t out_stride, int in_dtype, int scales_dtype, float epsilon, float weight_offset,
+    float scale_ub) {
+  __shared__ float red_s[4], red_m[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int64_t base = (int64_t)row * in_stride;
+  float ssq = 0.0f, amax = 0.0f;
+  for (int i = tid; i < K; i += 256) {
+    const float x = load_elem(in, in_dtype, base + i);
+    ssq += x * x;
+    amax = fmaxf(amax, fabsf(x * (load_elem(gamma, in_dtype, i) + weight_offset)));
+  }
+  ssq = wave_sum(ssq);
+  amax = wave_max(amax);
+  if ((tid & 63) == 0) { red_s[tid >> 6] = ssq; red_m[tid >> 6] = amax; }
+  __syncthreads();
+  ssq = (red_s[0] + red_s[1]) + (red_s[2] + red_s[3]);
+  amax = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
+  const float inv_rms = 1.0f / __fsqrt_rn(ssq / (float)K + epsilon);
+  const float row_max = amax * inv_rms;
+  float scale, recip;
+  if (scales_dtype == MAXFP8_BF16) {
+    const float a = bf16_bits_to_f32(f32_to_bf16_bits(row_max));
+    const float ub = bf16_bits_to_f32(f32_to_bf16_bits(scale_ub));
+    const uint32_t sb = f32_to_bf16_bits(fminf(a, ub) / 448.0f);
+    scale = bf16_bits_to_f32(sb);
+    float r = 0.0f;
+    if (scale != 0.0f) {
+      r = 1.0f / scale;
+      if (isinf(r) || isnan(r)) r = 0.0f;
+    }
+    recip = r;
+    if (tid == 0) reinterpret_cast<uint16_t*>(scales)[row] = (uint16_t)sb;
+  } else {
+    dynamic_scale_f32(row_max, scale_ub, scale, recip);
+    if (tid == 0) reinterpret_cast<float*>(scales)[row] = scale;
+  }
+  uint8_t* dst = out + (int64_t)row * out_stride;
+  for (int i = tid; i < K; i += 256) {
+    const float gq = load_elem(gamma, in_dtype, i) + weight_offset;
+    dst[i] = encode_one(clamp448(((load_elem(in, in_dtype, base + i) * inv_rms) * gq) * recip));
+  }
+}
+
+// ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void cast_f32_to_e4m3fn_kernel(uint8_t* out, const float* in, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
@@ -247,6 +366,33 @@ int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M
                      out_scales, in, (int)ngroups, (int)G, in_row_stride, out_row_stride, scales_ld, in_dtype,
                      scales_dtype, scale_ub);
   return launch_status("quant_generic");
+}
+
+int rmsnorm_quantize_dispatch(void* out_fp8, void* out_scales, const void* in, const void* gamma, int64_t rows, int64_t K,
+                              int64_t in_row_stride, int64_t out_row_stride, int in_dtype, int scales_dtype, float epsilon,
+                              float weight_offset, float scale_ub, hipStream_t stream) {
+  const bool fast = in_dtype == MAXFP8_BF16 && scales_dtype == MAXFP8_F32 && aligned16(in) && aligned16(gamma) &&
+                    (in_row_stride % 8 == 0) && (reinterpret_cast<uintptr_t>(out_fp8) % 8 == 0) && (out_row_stride % 8 == 0) &&
+                    (K % 8 == 0) && K <= 256 * 8 * 16;
+  if (fast) {
+    const int64_t nv = ceil_div(K / 8, 256);
+    uint8_t* o = (uint8_t*)out_fp8;
+    float* s = (float*)out_scales;
+#define LAUNCH_RMS(NV)                                                                                         \
+  hipLaunchKernelGGL(rmsnorm_quant_row_bf16_kernel<NV>, dim3((unsigned)rows), dim3(256), 0, stream, o, s,      \
+                     (const uint16_t*)in, (const uint16_t*)gamma, (int)K, in_row_stride, out_row_stride, epsilon, \
+                     weight_offset, scale_ub)
+    if (nv <= 1) LAUNCH_RMS(1);
+    else if (nv <= 2) LAUNCH_RMS(2);
+    else if (nv <= 4) LAUNCH_RMS(4);
+    else if (nv <= 8) LAUNCH_RMS(8);
+    else LAUNCH_RMS(16);
+#undef LAUNCH_RMS
+    return launch_status("rmsnorm_quant_row_bf16");
+  }
+  hipLaunchKernelGGL(rmsnorm_quant_generic_kernel, dim3((unsigned)rows), dim3(256), 0, stream, (uint8_t*)out_fp8, out_scales,
+                     in, gamma, (int)K, in_row_stride, out_row_stride, in_dtype, scales_dtype, epsilon, weight_offset, scale_ub);
+  return launch_status("rmsnorm_quant_generic");
 }
 
 int cast_f32_to_e4m3fn_dispatch(void* out, const float* in, int64_t n, hipStream_t stream) {

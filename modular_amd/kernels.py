@@ -97,6 +97,53 @@ def quantize_dynamic_scaled_float8(
     return out, scales
 
 
+def rms_norm_fused_quantize_dynamic_scaled_fp8(
+    input: torch.Tensor,
+    gamma: torch.Tensor,
+    epsilon: float,
+    weight_offset: float = 0.0,
+    scale_ub: float = 1200.0,
+    out_type: torch.dtype = _FP8,
+    scales_type: torch.dtype = torch.float32,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """RMSNorm over the last axis fused with the per-row dynamic fp8 quantisation: the composite op
+    `mo.composite.rms_norm_fused_quantize_dynamic_scaled_fp8` that the reference's graph compiler
+    forms from rms_norm followed by quantize_dynamic_scaled_float8
+    (builtin_kernels/quantization.mojo:112-237).
+
+    Returns (quantized, same shape as input, e4m3fn; scales [1, rows] with rows = input.numel() / K)."""
+    if input.dim() < 1:
+        raise ValueError("input must have at least one axis")
+    if gamma.dim() != 1:
+        raise ValueError("gamma must be rank 1")
+    if gamma.dtype != input.dtype:
+        raise TypeError("gamma dtype must match input dtype")
+    if out_type != _FP8:
+        raise ValueError("output dtype should be float8_e4m3fn or float8_e4m3fnuz")
+    if scales_type not in (torch.float32, torch.bfloat16):
+        raise TypeError("scales dtype should be bfloat16 or float32")
+    if input.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError(f"input dtype {input.dtype} is not bfloat16, float16 or float32")
+    K = input.shape[-1]
+    if gamma.shape[0] != K:
+        raise ValueError(f"gamma has {gamma.shape[0]} elements, the normalised axis has {K}")
+    _require_gpu(input)
+    _require_gpu(gamma)
+    x2 = input.reshape(-1, K)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    gamma = gamma.contiguous()
+    out = torch.empty((rows, K), dtype=_FP8, device=input.device)
+    scales = torch.empty((1, rows), dtype=scales_type, device=input.device)
+    st = _lib.lib().maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8(
+        out.data_ptr(), scales.data_ptr(), x2.data_ptr(), gamma.data_ptr(), rows, K,
+        x2.stride(0) if rows > 1 else K, K, _DT[input.dtype], _DT[scales_type], float(epsilon),
+        float(weight_offset), float(scale_ub), _stream(input))
+    _lib.check(st)
+    return out.reshape(input.shape), scales
+
+
 def dynamic_scaled_matmul(
     a: torch.Tensor,
     b: torch.Tensor,

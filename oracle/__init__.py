@@ -55,6 +55,8 @@ def lib() -> ctypes.CDLL:
         L.orc_matmul_rowwise.argtypes = [vp, vp, vp, vp, vp] + [i64] * 8 + [ci, ci, ci]
         L.orc_grouped_matmul.restype = ci
         L.orc_grouped_matmul.argtypes = [vp] * 7 + [i64] * 7 + [ci, ci, ci]
+        L.orc_rms_norm_fused_quantize.restype = ci
+        L.orc_rms_norm_fused_quantize.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, cf, cf, cf, ci]
         L.orc_max_threads.restype = ci
         _lib = L
     return _lib
@@ -117,6 +119,35 @@ def quantize_dynamic_scaled_fp8(x: np.ndarray, group_size: int, *, in_dtype: int
                                                in_dtype, scales_dtype, scale_ub, threads)
     if rc:
         raise ValueError(f"oracle quantize failed: {rc}")
+    return q, sc
+
+
+def round_to_dtype(v: float, dtype: int) -> float:
+    """v rounded to bf16 / f16 / f32 and widened back (how an op parameter of the input's dtype arrives)."""
+    if dtype == BF16:
+        import torch
+        return float(torch.tensor(v, dtype=torch.float32).to(torch.bfloat16).float())
+    if dtype == F16:
+        return float(np.float32(np.float16(v)))
+    return float(np.float32(v))
+
+
+def rms_norm_fused_quantize(x: np.ndarray, gamma: np.ndarray, epsilon: float, weight_offset: float = 0.0, *,
+                            in_dtype: int = BF16, scales_dtype: int = F32, scale_ub: float = 1200.0,
+                            threads: int = 1):
+    """x: [rows, K], gamma: [K] (uint16 bits for bf16/f16, float32 for f32).  epsilon and
+    weight_offset are rounded to the input dtype first, as the op registration does
+    (builtin_kernels/quantization.mojo:205-213).  Returns (q uint8 [rows, K], scales [1, rows])."""
+    x = np.ascontiguousarray(x)
+    gamma = np.ascontiguousarray(gamma)
+    rows, K = x.shape
+    q = np.zeros((rows, K), dtype=np.uint8)
+    sc = np.zeros((1, rows), dtype=np.float32 if scales_dtype == F32 else np.uint16)
+    rc = lib().orc_rms_norm_fused_quantize(_p(q), _p(sc), _p(x), _p(gamma), rows, K, K, K, in_dtype, scales_dtype,
+                                           round_to_dtype(epsilon, in_dtype), round_to_dtype(weight_offset, in_dtype),
+                                           scale_ub, threads)
+    if rc:
+        raise ValueError(f"oracle rms_norm_fused_quantize failed: {rc}")
     return q, sc
 
 

@@ -188,6 +188,62 @@ int orc_quantize_dynamic_scaled_fp8(uint8_t* out, void* scales, const void* in,
   return 0;
 }
 
+/*
+ * RMSNorm fused with per-row dynamic FP8 quantisation
+ * (max/kernels/src/nn/normalization.mojo:3996-4175; op registration
+ * max/kernels/src/graph_compiler/builtin_kernels/quantization.mojo:112-237;
+ * host procedure of the reference's test, test_rms_norm_fused_fp8.mojo:60-126):
+ *   ssq      = sum_c f32(x[r,c])^2                  (rounded once to f32: see below)
+ *   inv_rms  = 1 / sqrt(ssq / K + eps)              eps already rounded to the input dtype
+ *   g'[c]    = f32(gamma[c]) + f32(weight_offset)
+ *   row_max  = max_c |f32(x) * g'[c]| * inv_rms     (the kernel's form, normalization.mojo:4112-4131)
+ *   (scale, recip) = dynamic scale of row_max       scales[r] = scale
+ *   out[r,c] = e4m3fn(clamp(((f32(x) * inv_rms) * g'[c]) * recip, +-448))
+ * PARITY UNPINNED beyond the reference test's own data: the reference reduces ssq as a tree
+ * of SIMD partial sums and uses the target's rsqrt, neither of which its source fixes, so the
+ * last bits of inv_rms -- and with them a byte here and there -- are not defined by the source.
+ * The oracle therefore takes the one value every f32 summation order approximates: the sum
+ * accumulated in double and rounded to f32 once (the sequential f32 loop of the reference's
+ * host test drifts by up to K * 2^-24 relative on long rows; it gives the same bytes on that
+ * test's data, which tests/test_oracle_rmsnorm.py checks).
+ */
+int orc_rms_norm_fused_quantize(uint8_t* out, void* scales, const void* in, const void* gamma,
+                                int64_t rows, int64_t K, int64_t in_row_stride, int64_t out_row_stride,
+                                int in_dtype, int scales_dtype, float epsilon, float weight_offset,
+                                float scale_ub, int threads) {
+#ifdef _OPENMP
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+#endif
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t base = r * in_row_stride;
+    double ssq_d = 0.0;
+    for (int64_t c = 0; c < K; ++c) {
+      const double x = (double)load_in(in, in_dtype, base + c);
+      ssq_d += x * x;
+    }
+    const float ssq = (float)ssq_d;
+    const float inv_rms = 1.0f / sqrtf(ssq / (float)K + epsilon);
+    float amax = 0.0f;
+    for (int64_t c = 0; c < K; ++c) {
+      const float g = load_in(gamma, in_dtype, c) + weight_offset;
+      const float a = fabsf(load_in(in, in_dtype, base + c) * g);
+      if (a > amax) amax = a;
+    }
+    float scale, recip;
+    orc_dynamic_scale(amax * inv_rms, scale_ub, scales_dtype, &scale, &recip);
+    if (scales_dtype == ORC_BF16) ((uint16_t*)scales)[r] = f32_to_bf16(scale);
+    else ((float*)scales)[r] = scale;
+    for (int64_t c = 0; c < K; ++c) {
+      const float g = load_in(gamma, in_dtype, c) + weight_offset;
+      float v = ((load_in(in, in_dtype, base + c) * inv_rms) * g) * recip;
+      if (v > 448.0f) v = 448.0f;
+      if (v < -448.0f) v = -448.0f;
+      out[r * out_row_stride + c] = orc_f32_to_e4m3fn(v);
+    }
+  }
+  return 0;
+}
+
 /* ---- matmuls ------------------------------------------------------------ */
 
 static float g_lut[256];
