@@ -39,7 +39,7 @@ int naive_grouped_dispatch(void*, const void*, const void*, const void*, const v
                            const int32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int, hipStream_t);
 int gemm_tiled_dispatch(const GemmArgs&, bool, size_t, hipStream_t);
 size_t gemm_tiled_workspace_bytes(int64_t, int64_t, int64_t);
-int gemm_grouped_dispatch(const GemmArgs&, int64_t, hipStream_t);
+int gemm_grouped_dispatch(const GemmArgs&, int64_t, int64_t, hipStream_t);
 int gemm_skinny_dispatch(const GemmArgs&, bool, hipStream_t);
 int gemm_skinny_max_m();
 
@@ -240,7 +240,7 @@ int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void*
   p.num_active = (int)num_active_experts;
   p.b_expert_stride = N * K;
   p.bs_expert_stride = ceil_div(N, 128) * ceil_div(K, 128);
-  return gemm_grouped_dispatch(p, T, st);
+  return gemm_grouped_dispatch(p, T, max_num_tokens_per_expert, st);
 }
 
 int maxfp8_cast_f32_to_e4m3fn(void* out_fp8, const float* in, int64_t n, void* stream) {

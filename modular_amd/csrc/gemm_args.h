@@ -22,6 +22,7 @@ struct GemmArgs {
   const int32_t* expert_ids;
   int num_active;
   int small_rows;            // slots with at most this many rows use the small tile (0: none do)
+  int big_rows, big_bm;      // slots with at least big_rows rows give their full big_bm-row tiles to the large-tile launch (0: none)
   int64_t b_expert_stride;   // bytes between experts in b
   int64_t bs_expert_stride;  // elements between experts in b_scales
   // split-K / skinny only

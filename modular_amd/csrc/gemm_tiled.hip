@@ -375,15 +375,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
   tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false>(p, smem, (int64_t)tm * BM, p.M, tn * BN, p.b, p.b_scales);
 }
 
-// Grouped (MoE) matmul.  Slot z owns rows [offsets[z], offsets[z+1]).  A slot with at most
-// small_rows (<= SBM) rows is one SBM-row tile per BN columns, computed with a small tile and one more LDS stage
-// (such tiles only stream weights, so what they need is bytes in flight); a larger slot is cut
-// into BM-row tiles.  blockIdx.y counts row tiles over all slots, blockIdx.x is the column tile.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_grouped_kernel(GemmArgs p) {
-  static_assert(WAVES_M * WAVES_N == SWAVES_M * SWAVES_N, "both tile kinds run on the same block");
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  constexpr int NWAVES = WAVES_M * WAVES_N, NTHREADS = NWAVES * 64;
+// ---- grouped (MoE) matmul ---------------------------------------------------------------------
+// Slot z owns rows [offsets[z], offsets[z+1]).  blockIdx.y counts row tiles over all slots,
+// blockIdx.x is the column tile; a block finds its (slot, tile) with a block-wide prefix sum of
+// tiles_of(slot) over the device-resident offsets: no host synchronisation, no list of tiles.
+template <int NWAVES, typename TilesOf>
+__device__ __forceinline__ bool grouped_find_tile(const GemmArgs& p, const int by, TilesOf tiles_of, int& slot, int& tile) {
+  constexpr int NTHREADS = NWAVES * 64;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   __shared__ int s_slot, s_tile, s_wave_sum[NWAVES], s_carry;
@@ -392,10 +390,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
   for (int z0 = 0; z0 < p.num_active; z0 += NTHREADS) {
     const int z = z0 + tid;
     int t = 0;
-    if (z < p.num_active) {
-      const int rows = (int)(p.offsets[z + 1] - p.offsets[z]);
-      t = rows <= p.small_rows ? (rows > 0 ? 1 : 0) : (rows + BM - 1) / BM;
-    }
+    if (z < p.num_active) t = tiles_of((int)(p.offsets[z + 1] - p.offsets[z]));
     int incl = t;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
@@ -407,35 +402,83 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
     int before = s_carry;
     for (int w = 0; w < wave; ++w) before += s_wave_sum[w];
     const int excl = before + incl - t;
-    if (t > 0 && (int)blockIdx.y >= excl && (int)blockIdx.y < excl + t) { s_slot = z; s_tile = blockIdx.y - excl; }
+    if (t > 0 && by >= excl && by < excl + t) { s_slot = z; s_tile = by - excl; }
     __syncthreads();
     if (tid == NTHREADS - 1) s_carry = before + incl;
     __syncthreads();
-    if (s_slot >= 0 || (int)blockIdx.y < s_carry) break;
+    if (s_slot >= 0 || by < s_carry) break;
   }
-  const int slot = s_slot;
-  if (slot < 0) return;
+  slot = s_slot;
+  tile = s_tile;
+  return slot >= 0;
+}
+
+// a slot without an expert (id -1) writes zeros
+template <int NTHREADS>
+__device__ __forceinline__ void grouped_zero_tile(const GemmArgs& p, int64_t row_begin, int rows_here, int n0, int bn) {
+  const int cols_here = (p.N - n0) < bn ? (p.N - n0) : bn;
+  for (int i = threadIdx.x; i < rows_here * cols_here; i += NTHREADS) {
+    const int64_t m = row_begin + i / cols_here;
+    const int n = n0 + i % cols_here;
+    if (p.c_dtype == MAXFP8_BF16) reinterpret_cast<uint16_t*>(p.c)[m * p.ldc + n] = 0;
+    else reinterpret_cast<float*>(p.c)[m * p.ldc + n] = 0.f;
+  }
+}
+
+// rows of a slot that the large-tile launch takes: the full big_bm-row tiles of slots with at
+// least big_rows rows
+__device__ __forceinline__ int grouped_head_rows(const GemmArgs& p, int rows) {
+  return (p.big_rows > 0 && rows >= p.big_rows) ? (rows / p.big_bm) * p.big_bm : 0;
+}
+
+// The rows the large-tile launch leaves: BM-row tiles, and one SBM-row tile with one more LDS stage
+// for what is at most small_rows (<= SBM) rows (such tiles only stream weights, so what they need is bytes in
+// flight).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_grouped_kernel(GemmArgs p) {
+  static_assert(WAVES_M * WAVES_N == SWAVES_M * SWAVES_N, "both tile kinds run on the same block");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  constexpr int NWAVES = WAVES_M * WAVES_N;
+  int slot, tile;
+  const int by = blockIdx.y, bx = blockIdx.x;
+  const bool found = grouped_find_tile<NWAVES>(p, by, [&](int rows_total) {
+    const int rows = rows_total - grouped_head_rows(p, rows_total);
+    return rows <= p.small_rows ? (rows > 0 ? 1 : 0) : (rows + BM - 1) / BM;
+  }, slot, tile);
+  if (!found) return;
   const int64_t slot_begin = p.offsets[slot], row_end = p.offsets[slot + 1];
-  const bool small = row_end - slot_begin <= p.small_rows;
-  const int64_t row_begin = slot_begin + (int64_t)s_tile * BM;
-  const int n0 = blockIdx.x * BN;
+  const int64_t rest_begin = slot_begin + grouped_head_rows(p, (int)(row_end - slot_begin));
+  const bool small = row_end - rest_begin <= p.small_rows;
+  const int64_t row_begin = rest_begin + (int64_t)tile * BM;
+  const int n0 = bx * BN;
   const int e = p.expert_ids[slot];
   if (e < 0) {
-    // a slot without an expert writes zeros
-    const int rows_here = (int)((row_end - row_begin) < BM ? (row_end - row_begin) : BM);
-    const int cols_here = (p.N - n0) < BN ? (p.N - n0) : BN;
-    for (int i = tid; i < rows_here * cols_here; i += NTHREADS) {
-      const int64_t m = row_begin + i / cols_here;
-      const int n = n0 + i % cols_here;
-      if (p.c_dtype == MAXFP8_BF16) reinterpret_cast<uint16_t*>(p.c)[m * p.ldc + n] = 0;
-      else reinterpret_cast<float*>(p.c)[m * p.ldc + n] = 0.f;
-    }
+    grouped_zero_tile<NWAVES * 64>(p, row_begin, (int)((row_end - row_begin) < BM ? (row_end - row_begin) : BM), n0, BN);
     return;
   }
   const uint8_t* bptr = p.b + (int64_t)e * p.b_expert_stride;
   const float* bs_ptr = p.b_scales + (int64_t)e * p.bs_expert_stride;
   if (small) tile_body<SBM, BN, SWAVES_M, SWAVES_N, SNS, true, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
   else tile_body<BM, BN, WAVES_M, WAVES_N, NS, true, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+}
+
+// The full BM-row tiles (BM == big_bm) of the slots with at least big_rows rows.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  constexpr int NWAVES = WAVES_M * WAVES_N;
+  int slot, tile;
+  const int by = blockIdx.y, bx = blockIdx.x;
+  if (!grouped_find_tile<NWAVES>(p, by, [&](int rows_total) { return grouped_head_rows(p, rows_total) / BM; }, slot, tile)) return;
+  const int64_t row_begin = (int64_t)p.offsets[slot] + (int64_t)tile * BM;
+  const int n0 = bx * BN;
+  const int e = p.expert_ids[slot];
+  if (e < 0) {
+    grouped_zero_tile<NWAVES * 64>(p, row_begin, BM, n0, BN);
+    return;
+  }
+  tile_body<BM, BN, WAVES_M, WAVES_N, NS, true, true>(p, smem, row_begin, row_begin + BM, n0, p.b + (int64_t)e * p.b_expert_stride,
+                                                       p.b_scales + (int64_t)e * p.bs_expert_stride);
 }
 
 template <int BM, int BN, int NS, bool BLOCKSCALE>
@@ -468,6 +511,13 @@ static int launch_grouped(const GemmArgs& p, dim3 grid, hipStream_t stream, cons
   constexpr int big = tile_lds_bytes<BM, BN, NS, true>(), small = tile_lds_bytes<SBM, BN, SNS, true>();
   return launch_with_lds(gemm_grouped_kernel<BM, BN, WAVES_M, WAVES_N, NS, SBM, SWAVES_M, SWAVES_N, SNS>, attr_done,
                          big > small ? big : small, WAVES_M * WAVES_N * 64, p, grid, stream, name);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS>
+static int launch_grouped_large(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
+  static bool attr_done = false;
+  return launch_with_lds(gemm_grouped_large_kernel<BM, BN, WAVES_M, WAVES_N, NS>, attr_done, tile_lds_bytes<BM, BN, NS, true>(),
+                         WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
 
 // Sums the split-K partial results in split order (deterministic), applies the row / tensor
@@ -606,14 +656,26 @@ static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, di
   return launch_tiled<128, 128, 2, 2, 2, false>(p, grid, stream, "gemm_tiled_row_128x128");
 }
 
-int gemm_grouped_dispatch(const GemmArgs& p_in, int64_t T, hipStream_t stream) {
+int gemm_grouped_dispatch(const GemmArgs& p_in, int64_t T, int64_t max_tokens, hipStream_t stream) {
   GemmArgs p = p_in;
-  // a slot owns one small tile or ceil(rows / BM) tiles: their sum is <= T / BM + num_active
-  // MAXFP8_TILE=2: 256-row tiles; MAXFP8_TILE=3: no small tiles (tuning runs)
+  // Slots with at least 1024 rows (the caller's bound on the largest slot says whether there can
+  // be any) hand their full 256-row tiles to a launch with 256 x 256 tiles; everything else --
+  // their last rows, the other slots -- runs in 128 x 128 tiles, and in 32 x 128 tiles with a
+  // third LDS stage where at most 32 rows are left.
+  // MAXFP8_TILE=2: 256-row tiles in one launch; 3: no small tiles; 4: no large-tile launch (tuning runs)
   const int tune = tile_override();
   const bool big = tune == 2;
   const int bm = big ? 256 : 128;
   p.small_rows = tune == 3 ? 0 : (big ? 64 : 32);
+  p.big_rows = 0;
+  p.big_bm = 256;
+  if (!big && tune != 4 && max_tokens >= 1024 && T / 256 <= 65535) {
+    p.big_rows = 1024;
+    const dim3 lgrid((unsigned)ceil_div(p.N, 256), (unsigned)(T / 256));
+    const int rc = launch_grouped_large<256, 256, 2, 4, 2>(p, lgrid, stream, "gemm_grouped_block_256x256");
+    if (rc != MAXFP8_OK) return rc;
+  }
+  // a slot owns one small tile or ceil(rows / BM) tiles: their sum is <= T / BM + num_active
   const int64_t m_tiles = T / bm + p.num_active;
   if (m_tiles > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: %lld row tiles exceed the launch limit", (long long)m_tiles);
   const dim3 grid((unsigned)ceil_div(p.N, 128), (unsigned)m_tiles);

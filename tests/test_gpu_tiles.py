@@ -122,10 +122,13 @@ GROUPED = [
     ([0, 1, 31, 32, 33, 129, 300], [3, 0, 6, 1, -1, 2, 5], 7, 200, 384),
     ([32] * 6, [5, 4, 3, 2, 1, 0], 6, 100, 256),
     ([1, 257, 2, 128], [0, 1, 2, 3], 4, 392, 512),
+    # slots of 1024 rows and more give their full 256-row tiles to the large-tile launch
+    ([1030, 0, 2050, 31], [2, 1, -1, 0], 4, 392, 256),
+    ([1024, 1279, 5], [1, 0, 2], 3, 264, 384),
 ]
 
 
-@pytest.mark.parametrize("tile", ["0", "2", "3"])
+@pytest.mark.parametrize("tile", ["0", "2", "3", "4"])
 @pytest.mark.parametrize("counts,ids,E,N,K", GROUPED)
 @pytest.mark.parametrize("out", [torch.float32, torch.bfloat16])
 def test_grouped_tile_kinds(dev, monkeypatch, tile, counts, ids, E, N, K, out):
