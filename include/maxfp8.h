@@ -177,6 +177,38 @@ int maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8(
     float scale_ub, void* stream);
 
 /*
+ * mo.moe.create.indices  (wrapper: max/python/max/nn/kernels.py:4980-5060; kernel:
+ * max/kernels/src/nn/moe.mojo:435-720).  Groups the n = tokens * top_k expert assignments
+ * topk_ids[i] (int32 / uint32, values in [0, num_experts)) by expert:
+ *   token_expert_order[n]   assignment indices grouped by expert slot
+ *   expert_start_indices[num_experts + 1]  slot z owns token_expert_order[start[z] .. start[z+1])
+ *   restore_token_order[n]  position of assignment i in token_expert_order
+ *   expert_ids[num_experts] expert of slot z
+ *   expert_usage_stats[2]   {most assignments on one expert, number of slots = num_experts}
+ * The reference assigns slots in the order its blocks reach a lock, so any permutation of the
+ * experts is a valid expert_ids; this library always returns slot z = expert z with the
+ * assignments of a slot in increasing order (deterministic).  No outputs need initialising.
+ */
+int maxfp8_moe_create_indices(
+    uint32_t* token_expert_order, uint32_t* expert_start_indices, uint32_t* restore_token_order,
+    int32_t* expert_ids, uint32_t* expert_usage_stats, const void* topk_ids,
+    int64_t n, int64_t num_experts, void* stream);
+
+/*
+ * ep.fused_silu  (wrapper: max/python/max/nn/comm/ep/ep_kernels.py:1121-1165 and 1168-1290;
+ * kernels: max/kernels/src/shmem/ep_comm.mojo:4409-4500, 4505-4624).
+ * in [max_rows, 2 * inter]: out[m, k] = silu(in[m, k]) * in[m, inter + k] for the
+ * rows m < row_offsets[num_offsets - 1] (read on the device; the other rows are not written).
+ * quantize == 0: out has in_dtype.  quantize != 0: out is e4m3fn with one f32 scale per 128
+ * outputs, out_scales[k / 128, m] (row stride scales_ld), scale = max(amax, 1e-4) / 448 and
+ * out = clamp(value / scale) -- this op's own recipe.  inter % 128 == 0 (quantize) or % 8.
+ */
+int maxfp8_fused_silu(
+    void* out, void* out_scales, const void* in, const uint32_t* row_offsets,
+    int64_t num_offsets, int64_t max_rows, int64_t inter, int64_t in_row_stride,
+    int64_t out_row_stride, int64_t scales_ld, int in_dtype, int quantize, void* stream);
+
+/*
  * Elementwise f32 -> e4m3fn (clamp to +-448, round to nearest even), the cast
  * inside fp8_quantize (max/kernels/src/internal_utils/fp8_utils.mojo:96-143).
  * Exposed so the hardware convert can be checked exhaustively.

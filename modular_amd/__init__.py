@@ -8,6 +8,7 @@ from .quant_config import (InputScaleSpec, QuantConfig, QuantFormat, ScaleGranul
                            WeightScaleSpec, blockwise_fp8_config, rowwise_fp8_config)
 from .kernels import (dynamic_scaled_matmul, grouped_dynamic_scaled_fp8_matmul,
                       quantize_dynamic_scaled_float8, rms_norm_fused_quantize_dynamic_scaled_fp8)
+from .moe_kernels import fused_silu, fused_silu_quantized, moe_create_indices
 from .quant_ops import matmul_float8, quantized_matmul
 from .linear import Linear
 
@@ -16,4 +17,5 @@ __all__ = [
     "blockwise_fp8_config", "rowwise_fp8_config", "dynamic_scaled_matmul",
     "grouped_dynamic_scaled_fp8_matmul", "quantize_dynamic_scaled_float8", "matmul_float8",
     "quantized_matmul", "Linear", "rms_norm_fused_quantize_dynamic_scaled_fp8",
+    "moe_create_indices", "fused_silu", "fused_silu_quantized",
 ]

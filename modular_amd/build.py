@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libmaxfp8.so")
 
-SOURCES = ["api.hip", "quant.hip", "naive.hip", "gemm_tiled.hip", "gemm_skinny.hip"]
+SOURCES = ["api.hip", "quant.hip", "naive.hip", "gemm_tiled.hip", "gemm_skinny.hip", "moe.hip"]
 
 # packed-fp32 VALU ops are switched off for every kernel (they are not used by hand either)
 COMMON = [

@@ -27,6 +27,9 @@ int quantize_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int6
                       float, hipStream_t);
 int rmsnorm_quantize_dispatch(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float,
                               float, float, hipStream_t);
+int moe_create_indices_dispatch(uint32_t*, uint32_t*, uint32_t*, int32_t*, uint32_t*, const int32_t*, int64_t, int64_t, hipStream_t);
+int fused_silu_dispatch(void*, float*, const void*, const uint32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool,
+                        hipStream_t);
 int cast_f32_to_e4m3fn_dispatch(void*, const float*, int64_t, hipStream_t);
 int cast_e4m3fn_to_f32_dispatch(float*, const void*, int64_t, hipStream_t);
 int copy_bytes_dispatch(void*, const void*, int64_t, hipStream_t);
@@ -109,6 +112,38 @@ int maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_s
   return rmsnorm_quantize_dispatch(out_fp8, out_scales, in, gamma, rows, K, in_row_stride, out_row_stride, in_dtype,
                                    scales_dtype, round_to_dtype(epsilon, in_dtype), round_to_dtype(weight_offset, in_dtype),
                                    scale_ub, (hipStream_t)stream);
+}
+
+int maxfp8_moe_create_indices(uint32_t* token_expert_order, uint32_t* expert_start_indices, uint32_t* restore_token_order,
+                              int32_t* expert_ids, uint32_t* expert_usage_stats, const void* topk_ids, int64_t n,
+                              int64_t num_experts, void* stream) {
+  if (n < 0 || num_experts < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "moe_create_indices: negative size");
+  if (n >= ((int64_t)1 << 31) || num_experts > 65535)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "moe_create_indices: %lld assignments / %lld experts exceed the limits", (long long)n,
+                (long long)num_experts);
+  if (!expert_usage_stats || !expert_start_indices) MAXFP8_FAIL(MAXFP8_ERR_NULL, "moe_create_indices: null pointer");
+  if (num_experts == 0) return MAXFP8_OK;
+  if (!expert_ids || (n > 0 && (!token_expert_order || !restore_token_order || !topk_ids)))
+    MAXFP8_FAIL(MAXFP8_ERR_NULL, "moe_create_indices: null pointer");
+  return moe_create_indices_dispatch(token_expert_order, expert_start_indices, restore_token_order, expert_ids,
+                                     expert_usage_stats, (const int32_t*)topk_ids, n, num_experts, (hipStream_t)stream);
+}
+
+int maxfp8_fused_silu(void* out, void* out_scales, const void* in, const uint32_t* row_offsets, int64_t num_offsets,
+                      int64_t max_rows, int64_t inter, int64_t in_row_stride, int64_t out_row_stride, int64_t scales_ld,
+                      int in_dtype, int quantize, void* stream) {
+  if (in_dtype != MAXFP8_BF16) MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "fused_silu: input dtype %d is not bf16", in_dtype);
+  if (max_rows < 0 || inter < 0 || num_offsets < 1) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused_silu: bad sizes");
+  if (max_rows == 0 || inter == 0) return MAXFP8_OK;
+  if (inter % 128 != 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused_silu: the output width %lld must be a multiple of 128", (long long)inter);
+  if (in_row_stride < 2 * inter || out_row_stride < inter || (quantize && scales_ld < max_rows))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused_silu: strides smaller than the extents");
+  if (!out || !in || !row_offsets || (quantize && !out_scales)) MAXFP8_FAIL(MAXFP8_ERR_NULL, "fused_silu: null pointer");
+  if (!is_aligned(in, 16) || in_row_stride % 8 != 0 || !is_aligned(out, 16) || out_row_stride % (quantize ? 8 : 8) != 0)
+    MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "fused_silu: rows must be 16-byte aligned");
+  return fused_silu_dispatch(out, (float*)out_scales, in, row_offsets, num_offsets, max_rows, inter, in_row_stride,
+                             out_row_stride, scales_ld, quantize != 0, (hipStream_t)stream);
 }
 
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K) {

@@ -1,0 +1,215 @@
+// The MoE steps on either side of the grouped FP8 matmul:
+//
+//   * moe_create_indices: groups the (token, expert) assignments by expert -- a stable bucket
+//     sort of topk_ids (semantics: max/kernels/src/nn/moe.mojo:435-590).  The reference hands
+//     out expert slots in the order in which its blocks reach an atomic lock, so its
+//     expert_ids is some permutation of 0..E-1; here slot z is expert z and tokens keep their
+//     order inside a slot, which is one of the reference's possible results and the same on
+//     every run.  Three small launches (count, scan, scatter), no atomics, no scratch memory:
+//     the counts travel in expert_start_indices.
+//   * fused_silu / fused_silu_quantized: silu(gate) * up on the rows that row_offsets says
+//     are in use, written as the input dtype or quantised to e4m3fn with one scale per
+//     128 outputs, scales transposed (max/kernels/src/shmem/ep_comm.mojo:4409-4500, 4505-4624).
+//     Note the quantiser of this op: scale = max(amax, 1e-4) / 448 and out / scale (a division),
+//     not the min(amax, ub) / 448 and x * (1 / scale) of quantize_dynamic_scaled_fp8.
+#include "common.h"
+
+namespace maxfp8 {
+
+// ---- moe_create_indices -----------------------------------------------------------------------
+// block e counts the assignments to expert e; the count waits in expert_start_indices[e + 1]
+__global__ __launch_bounds__(256) void moe_count_kernel(uint32_t* __restrict__ expert_start_indices,
+                                                        const int32_t* __restrict__ topk_ids, int n) {
+  __shared__ int red[4];
+  const int e = blockIdx.x, tid = threadIdx.x;
+  int cnt = 0;
+  for (int i = tid; i < n; i += 256) cnt += topk_ids[i] == e;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) cnt += __shfl_xor(cnt, o, 64);
+  if ((tid & 63) == 0) red[tid >> 6] = cnt;
+  __syncthreads();
+  if (tid == 0) {
+    expert_start_indices[e + 1] = (uint32_t)(red[0] + red[1] + red[2] + red[3]);
+    if (e == 0) expert_start_indices[0] = 0;
+  }
+}
+
+// one block: counts -> start offsets (in place), expert_ids = identity, usage stats
+__global__ __launch_bounds__(1024) void moe_scan_kernel(uint32_t* __restrict__ expert_start_indices,
+                                                        int32_t* __restrict__ expert_ids,
+                                                        uint32_t* __restrict__ expert_usage_stats, int num_experts) {
+  __shared__ uint32_t wave_sum[16], wave_max_s[16];
+  __shared__ uint32_t carry;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) carry = 0;
+  uint32_t mx = 0;
+  __syncthreads();
+  for (int base = 0; base < num_experts; base += 1024) {
+    const int z = base + tid;
+    const uint32_t c = z < num_experts ? expert_start_indices[z + 1] : 0u;
+    mx = c > mx ? c : mx;
+    uint32_t incl = c;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const uint32_t up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    if (lane == 63) wave_sum[wave] = incl;
+    __syncthreads();
+    uint32_t before = carry;
+    for (int w = 0; w < wave; ++w) before += wave_sum[w];
+    if (z < num_experts) {
+      expert_start_indices[z + 1] = before + incl;
+      expert_ids[z] = z;
+    }
+    __syncthreads();
+    if (tid == 1023) carry = before + incl;
+    __syncthreads();
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint32_t other = __shfl_xor(mx, o, 64);
+    mx = other > mx ? other : mx;
+  }
+  if (lane == 0) wave_max_s[wave] = mx;
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t m = 0;
+    for (int w = 0; w < 16; ++w) m = wave_max_s[w] > m ? wave_max_s[w] : m;
+    expert_usage_stats[0] = m;                       // most tokens on one expert
+    expert_usage_stats[1] = (uint32_t)num_experts;   // every expert keeps a slot (moe.mojo:584-588)
+  }
+}
+
+// block e writes the positions of its assignments, in order, from expert_start_indices[e] on
+__global__ __launch_bounds__(256) void moe_scatter_kernel(uint32_t* __restrict__ token_expert_order,
+                                                          uint32_t* __restrict__ restore_token_order,
+                                                          const uint32_t* __restrict__ expert_start_indices,
+                                                          const int32_t* __restrict__ topk_ids, int n) {
+  __shared__ int wave_cnt[4];
+  const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  uint32_t base = expert_start_indices[e];
+  if (expert_start_indices[e + 1] == base) return;
+  for (int i0 = 0; i0 < n; i0 += 256) {
+    const int i = i0 + tid;
+    const bool hit = i < n && topk_ids[i] == e;
+    const unsigned long long mask = __ballot(hit);
+    const int before_in_wave = __popcll(mask & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_cnt[wave] = __popcll(mask);
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) before += wave_cnt[w];
+      total += wave_cnt[w];
+    }
+    if (hit) {
+      const uint32_t pos = base + (uint32_t)(before + before_in_wave);
+      token_expert_order[pos] = (uint32_t)i;
+      restore_token_order[i] = pos;
+    }
+    base += (uint32_t)total;
+    __syncthreads();
+  }
+}
+
+int moe_create_indices_dispatch(uint32_t* token_expert_order, uint32_t* expert_start_indices, uint32_t* restore_token_order,
+                                int32_t* expert_ids, uint32_t* expert_usage_stats, const int32_t* topk_ids, int64_t n,
+                                int64_t num_experts, hipStream_t stream) {
+  hipLaunchKernelGGL(moe_count_kernel, dim3((unsigned)num_experts), dim3(256), 0, stream, expert_start_indices, topk_ids, (int)n);
+  hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, stream, expert_start_indices, expert_ids, expert_usage_stats,
+                     (int)num_experts);
+  if (n > 0)
+    hipLaunchKernelGGL(moe_scatter_kernel, dim3((unsigned)num_experts), dim3(256), 0, stream, token_expert_order,
+                       restore_token_order, expert_start_indices, topk_ids, (int)n);
+  return launch_status("moe_create_indices");
+}
+
+// ---- fused SiLU(gate) * up --------------------------------------------------------------------
+// a / b from the hardware reciprocal and one correction step: the correctly rounded quotient
+// except for rare double roundings, at a third of the instructions of the IEEE sequence (the
+// kernels below are bound by these divisions, not by memory, when they use that sequence)
+__device__ __forceinline__ float fast_div(float a, float b, float rcp_b) {
+  const float q = a * rcp_b;
+  const float err = fmaf(-q, b, a);
+  return err == 0.0f ? q : fmaf(err, rcp_b, q);  // (keeps the sign of a zero quotient)
+}
+
+__device__ __forceinline__ float silu_mul(float gate, float up) {
+  // gate / (1 + exp(-gate)) * up, every step rounded to f32 (ep_comm.mojo:4494-4497)
+  const float d = 1.0f + expf(-gate);
+  // d = inf (gate < -88): gate / inf = -0; the correction step would produce NaN there
+  const float sig = d > 3.0e38f ? -0.0f : fast_div(gate, d, __builtin_amdgcn_rcpf(d));
+  return sig * up;
+}
+
+// 16 lanes own 128 consecutive outputs of one row (8 each): one 16-byte load of gate and of up
+// per lane; QUANT: amax over the 16 lanes by DPP, 8-byte packed fp8 store, lane 0 writes the scale.
+template <bool QUANT>
+__global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__ out, float* __restrict__ scales,
+                                                              const uint16_t* __restrict__ in,
+                                                              const uint32_t* __restrict__ row_offsets, int num_offsets,
+                                                              int inter, int64_t in_stride, int64_t out_stride,
+                                                              int64_t scales_ld) {
+  const uint32_t rows = row_offsets[num_offsets - 1];
+  const int groups = inter >> 7;
+  const int tid = threadIdx.x, sub = tid & 15;
+  const int64_t total = (int64_t)rows * groups;
+  for (int64_t item = (int64_t)blockIdx.x * 16 + (tid >> 4); item < total; item += (int64_t)gridDim.x * 16) {
+    const int64_t m = item / groups;
+    const int g = (int)(item - m * groups);
+    const uint16_t* src = in + m * in_stride + g * 128 + sub * 8;
+    const uint4 gv = *reinterpret_cast<const uint4*>(src);
+    const uint4 uv = *reinterpret_cast<const uint4*>(src + inter);
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[2 * j] = silu_mul(__uint_as_float(gw[j] << 16), __uint_as_float(uw[j] << 16));
+      f[2 * j + 1] = silu_mul(__uint_as_float(gw[j] & 0xffff0000u), __uint_as_float(uw[j] & 0xffff0000u));
+    }
+    if constexpr (!QUANT) {
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = f32_to_bf16_bits(f[2 * j]) | (f32_to_bf16_bits(f[2 * j + 1]) << 16);
+      *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(out) + m * out_stride + g * 128 + sub * 8) =
+          make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+      float amax = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(f[j]));
+      amax = row16_max(amax);
+      const float scale = fmaxf(amax, 1e-4f) / 448.0f;
+      const float rs = __builtin_amdgcn_rcpf(scale);
+      float q[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q[j] = clamp448(fast_div(f[j], scale, rs));
+      int lo = 0, hi = 0;
+      lo = cvt_pk_e4m3fn(q[0], q[1], lo, false);
+      lo = cvt_pk_e4m3fn(q[2], q[3], lo, true);
+      hi = cvt_pk_e4m3fn(q[4], q[5], hi, false);
+      hi = cvt_pk_e4m3fn(q[6], q[7], hi, true);
+      *reinterpret_cast<uint2*>(reinterpret_cast<uint8_t*>(out) + m * out_stride + g * 128 + sub * 8) =
+          make_uint2((uint32_t)lo, (uint32_t)hi);
+      if (sub == 0) scales[(int64_t)g * scales_ld + m] = scale;
+    }
+  }
+}
+
+int fused_silu_dispatch(void* out, float* scales, const void* in, const uint32_t* row_offsets, int64_t num_offsets,
+                        int64_t max_rows, int64_t inter, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
+                        bool quant, hipStream_t stream) {
+  // the number of rows in use is only known on the device: the grid is sized for max_rows and
+  // walks the items in strides
+  const int64_t items = max_rows * (inter / 128);
+  const unsigned blocks = (unsigned)(ceil_div(items, 16) < 8192 ? ceil_div(items, 16) : 8192);
+  if (quant)
+    hipLaunchKernelGGL(fused_silu_bf16_kernel<true>, dim3(blocks), dim3(256), 0, stream, out, scales, (const uint16_t*)in,
+                       row_offsets, (int)num_offsets, (int)inter, in_stride, out_stride, scales_ld);
+  else
+    hipLaunchKernelGGL(fused_silu_bf16_kernel<false>, dim3(blocks), dim3(256), 0, stream, out, scales, (const uint16_t*)in,
+                       row_offsets, (int)num_offsets, (int)inter, in_stride, out_stride, scales_ld);
+  return launch_status(quant ? "fused_silu_quantized" : "fused_silu");
+}
+
+}  // namespace maxfp8

@@ -57,6 +57,10 @@ def lib() -> ctypes.CDLL:
         L.orc_grouped_matmul.argtypes = [vp] * 7 + [i64] * 7 + [ci, ci, ci]
         L.orc_rms_norm_fused_quantize.restype = ci
         L.orc_rms_norm_fused_quantize.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, cf, cf, cf, ci]
+        L.orc_moe_create_indices.restype = ci
+        L.orc_moe_create_indices.argtypes = [vp] * 6 + [i64, i64]
+        L.orc_fused_silu.restype = ci
+        L.orc_fused_silu.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, ci, ci]
         L.orc_max_threads.restype = ci
         _lib = L
     return _lib
@@ -149,6 +153,37 @@ def rms_norm_fused_quantize(x: np.ndarray, gamma: np.ndarray, epsilon: float, we
     if rc:
         raise ValueError(f"oracle rms_norm_fused_quantize failed: {rc}")
     return q, sc
+
+
+def moe_create_indices(topk_ids: np.ndarray, num_experts: int):
+    """topk_ids: int32 [n].  Returns (token_expert_order, expert_start_indices, restore_token_order,
+    expert_ids, expert_usage_stats) in the canonical order (slot z = expert z, stable)."""
+    ids = np.ascontiguousarray(topk_ids, dtype=np.int32)
+    n = ids.shape[0]
+    order = np.zeros(n, dtype=np.uint32)
+    start = np.zeros(num_experts + 1, dtype=np.uint32)
+    restore = np.zeros(n, dtype=np.uint32)
+    eids = np.zeros(num_experts, dtype=np.int32)
+    stats = np.zeros(2, dtype=np.uint32)
+    lib().orc_moe_create_indices(_p(order), _p(start), _p(restore), _p(eids), _p(stats), _p(ids), n, num_experts)
+    return order, start, restore, eids, stats
+
+
+def fused_silu(x: np.ndarray, rows: int, *, quantize: bool = False, scales_ld: int | None = None, threads: int = 1):
+    """x: bf16 bits [max_rows, 2*I].  Rows >= `rows` are left at zero (scales at NaN).  Returns the bf16
+    bits [max_rows, I], or (e4m3fn bytes [max_rows, I], f32 scales [I/128, scales_ld]) when quantize."""
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    max_rows, two_i = x.shape
+    inter = two_i // 2
+    if not quantize:
+        out = np.zeros((max_rows, inter), dtype=np.uint16)
+        lib().orc_fused_silu(_p(out), None, _p(x), rows, inter, two_i, inter, 0, 0, threads)
+        return out
+    ld = max_rows if scales_ld is None else scales_ld
+    out = np.zeros((max_rows, inter), dtype=np.uint8)
+    sc = np.full((inter // 128, ld), np.nan, dtype=np.float32)
+    lib().orc_fused_silu(_p(out), _p(sc), _p(x), rows, inter, two_i, inter, ld, 1, threads)
+    return out, sc
 
 
 def matmul_blockwise(a: np.ndarray, b: np.ndarray, a_scales: np.ndarray, b_scales: np.ndarray,

@@ -244,6 +244,86 @@ int orc_rms_norm_fused_quantize(uint8_t* out, void* scales, const void* in, cons
   return 0;
 }
 
+/* ---- MoE plumbing on either side of the grouped matmul ------------------------------------ */
+
+/*
+ * moe_create_indices (max/kernels/src/nn/moe.mojo:435-590): a bucket sort of the assignments by
+ * expert.  The reference hands out slots in the order its blocks reach an atomic lock; the
+ * canonical result restated here gives slot z to expert z and keeps the assignments of a slot in
+ * increasing order.  What the reference's own test checks are the invariants
+ * (test_moe_indices.mojo:38-140): grouping, start indices against expert_ids, the restore
+ * permutation, stats[0] = largest count; stats[1] = number of slots (every block adds one,
+ * moe.mojo:584-588).
+ */
+int orc_moe_create_indices(uint32_t* token_expert_order, uint32_t* expert_start_indices,
+                           uint32_t* restore_token_order, int32_t* expert_ids, uint32_t* stats,
+                           const int32_t* topk_ids, int64_t n, int64_t num_experts) {
+  uint32_t mx = 0;
+  expert_start_indices[0] = 0;
+  uint32_t pos = 0;
+  for (int64_t e = 0; e < num_experts; ++e) {
+    uint32_t cnt = 0;
+    for (int64_t i = 0; i < n; ++i) {
+      if (topk_ids[i] == (int32_t)e) {
+        token_expert_order[pos] = (uint32_t)i;
+        restore_token_order[i] = pos;
+        ++pos;
+        ++cnt;
+      }
+    }
+    expert_start_indices[e + 1] = pos;
+    expert_ids[e] = (int32_t)e;
+    if (cnt > mx) mx = cnt;
+  }
+  stats[0] = mx;
+  stats[1] = (uint32_t)num_experts;
+  return 0;
+}
+
+/*
+ * fused_silu / fused_silu_quantized (max/kernels/src/shmem/ep_comm.mojo:4409-4500, 4505-4624):
+ *   v = (gate / (1 + exp(-gate))) * up                 in f32, gate = in[m,k], up = in[m,I+k]
+ *   plain:     out[m,k] = cast(v)
+ *   quantised: scale = max(amax_128(|v|), 1e-4) / 448;  out = e4m3fn(clamp(v / scale));
+ *              scales[k/128, m] = scale
+ * for rows m < rows.  PARITY UNPINNED in the last bit of exp(): the reference's GPU exp is not
+ * fixed by its source; libm's expf stands in.
+ */
+int orc_fused_silu(void* out, float* scales, const uint16_t* in, int64_t rows, int64_t inter,
+                   int64_t in_row_stride, int64_t out_row_stride, int64_t scales_ld, int quantize,
+                   int threads) {
+#ifdef _OPENMP
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+#endif
+  for (int64_t m = 0; m < rows; ++m) {
+    for (int64_t g0 = 0; g0 < inter; g0 += 128) {
+      float v[128];
+      const int64_t len = inter - g0 < 128 ? inter - g0 : 128;
+      float amax = 0.0f;
+      for (int64_t k = 0; k < len; ++k) {
+        const float gate = bf16_to_f32(in[m * in_row_stride + g0 + k]);
+        const float up = bf16_to_f32(in[m * in_row_stride + inter + g0 + k]);
+        const float sig = gate / (1.0f + expf(-gate));
+        v[k] = sig * up;
+        if (fabsf(v[k]) > amax) amax = fabsf(v[k]);
+      }
+      if (!quantize) {
+        for (int64_t k = 0; k < len; ++k) ((uint16_t*)out)[m * out_row_stride + g0 + k] = f32_to_bf16(v[k]);
+      } else {
+        const float scale = (amax > 1e-4f ? amax : 1e-4f) / 448.0f;
+        scales[(g0 / 128) * scales_ld + m] = scale;
+        for (int64_t k = 0; k < len; ++k) {
+          float q = v[k] / scale;
+          if (q > 448.0f) q = 448.0f;
+          if (q < -448.0f) q = -448.0f;
+          ((uint8_t*)out)[m * out_row_stride + g0 + k] = orc_f32_to_e4m3fn(q);
+        }
+      }
+    }
+  }
+  return 0;
+}
+
 /* ---- matmuls ------------------------------------------------------------ */
 
 static float g_lut[256];

@@ -1,0 +1,118 @@
+"""GPU parity of the MoE steps around the grouped matmul: moe_create_indices equal to the oracle
+(and so to numpy's stable sort) and meeting the invariants of the reference's test on its sizes;
+fused_silu within one rounding of the oracle (exp is not fixed to the last bit by the reference:
+the bounds are in the tests); and the whole MoE MLP chained on the device."""
+import numpy as np
+import pytest
+import torch
+
+import modular_amd as mx
+import oracle
+from modular_amd import synth
+from moe_checks import check_indices
+from util import fp8_bytes
+
+pytestmark = pytest.mark.gpu
+NT = oracle.default_threads()
+
+
+@pytest.mark.parametrize("n,num_experts", [(197, 256), (2500, 256), (11, 256), (1, 256), (20660, 256), (100000, 256),
+                                           (0, 8), (64, 3), (32768, 256), (5000, 1500)])
+@pytest.mark.parametrize("dtype", [torch.int32, torch.uint32])
+def test_create_indices(dev, n, num_experts, dtype):
+    rng = np.random.default_rng(n + num_experts)
+    ids = rng.integers(0, num_experts, n).astype(np.int32)
+    outs = mx.moe_create_indices(torch.from_numpy(ids).to(dev).view(dtype), num_experts)
+    torch.cuda.synchronize()
+    got = [o.cpu().view(torch.int32).numpy().view(np.uint32 if o.dtype == torch.uint32 else np.int32) for o in outs]
+    check_indices(ids, num_experts, *got)
+    want = oracle.moe_create_indices(ids, num_experts)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+
+
+def test_create_indices_config_routing_feeds_the_grouped_matmul(dev):
+    # BASELINE's MoE routing, then a grouped matmul on the gathered rows: same result as on the
+    # host-sorted routing
+    T, E, k, K, N = 512, 16, 4, 256, 384
+    gen = torch.Generator().manual_seed(1)
+    topk = torch.stack([torch.randperm(E, generator=gen)[:k] for _ in range(T)]).to(torch.int32)   # [T, k]
+    order, start, restore, eids, stats = mx.moe_create_indices(topk.reshape(-1).to(dev), E)
+    x = synth.random_fp8((T, K), 2)
+    rows = x.to(dev)[(order.to(torch.int64) // k)]          # assignment i belongs to token i // k
+    sa = synth.random_scales((K // 128, T * k), 3).to(dev)
+    w, ws = synth.random_fp8((E, N, K), 4).to(dev), synth.random_scales((E, N // 128, K // 128), 5).to(dev)
+    cfg = mx.blockwise_fp8_config()
+    y = mx.grouped_dynamic_scaled_fp8_matmul(rows, w, sa, ws, start, eids, stats.cpu(), cfg.input_scale, cfg.weight_scale,
+                                             out_type=torch.float32)
+    want = oracle.grouped_matmul(fp8_bytes(rows), fp8_bytes(w), sa.cpu().numpy(), ws.cpu().numpy(),
+                                 start.cpu().view(torch.int32).numpy().view(np.uint32), eids.cpu().numpy(),
+                                 int(stats[0]), int(stats[1]), threads=NT)
+    from util import F32_BUDGET, assert_rel
+    assert_rel(y.cpu().numpy(), want, 1e-2, "moe chain", F32_BUDGET)
+    # restore brings the rows back into token order
+    back = y[restore.to(torch.int64)]
+    assert torch.equal(back.reshape(T, k, N)[3, 2], y[int(restore[3 * k + 2])])
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("max_rows,rows,I", [(64, 64, 2048), (300, 257, 512), (16, 0, 256), (4096, 3000, 2048), (7, 7, 128)])
+def test_fused_silu(dev, max_rows, rows, I):
+    gen = torch.Generator().manual_seed(max_rows + I)
+    x = (torch.randn((max_rows, 2 * I), generator=gen) * 2.5).to(torch.bfloat16)
+    off = torch.tensor([0, rows // 3, rows], dtype=torch.int64).to(torch.uint32)
+    sentinel = 0x7FC1
+    out = mx.fused_silu(x.to(dev), off.to(dev))
+    want = oracle.fused_silu(_bits(x), rows, threads=NT)
+    torch.cuda.synchronize()
+    got = _bits(out.cpu())
+    # device expf vs libm expf: a result may differ by one bf16 step; nearly all are equal
+    a = torch.from_numpy(got[:rows].view(np.int16)).view(torch.bfloat16).float()
+    b = torch.from_numpy(want[:rows].view(np.int16)).view(torch.bfloat16).float()
+    assert float((got[:rows] != want[:rows]).mean()) <= 1e-3 if rows else True
+    assert bool(torch.all((a - b).abs() <= b.abs() * 2.0 ** -7 + 1e-30))
+
+
+@pytest.mark.parametrize("max_rows,rows,I", [(64, 64, 2048), (300, 257, 512), (4096, 3000, 2048), (5, 5, 128)])
+def test_fused_silu_quantized(dev, max_rows, rows, I):
+    gen = torch.Generator().manual_seed(max_rows + I + 1)
+    x = (torch.randn((max_rows, 2 * I), generator=gen) * 2.5).to(torch.bfloat16)
+    x[0, :128] = 0                                          # a group whose amax is under the 1e-4 floor
+    off = torch.tensor([0, rows], dtype=torch.int64).to(torch.uint32)
+    q, s = mx.fused_silu_quantized(x.to(dev), off.to(dev), mx.blockwise_fp8_config())
+    want_q, want_s = oracle.fused_silu(_bits(x), rows, quantize=True, threads=NT)
+    torch.cuda.synchronize()
+    assert tuple(q.shape) == (max_rows, I) and tuple(s.shape) == (I // 128, max_rows)
+    got_q, got_s = fp8_bytes(q)[:rows], s.cpu().numpy()[:, :rows]
+    assert got_s[0, 0] == np.float32(1e-4) / np.float32(448.0)
+    # scales within 2 ulp (the exp of the group's largest element), bytes equal or neighbours
+    assert np.allclose(got_s, want_s[:, :rows], rtol=2 * 2.0 ** -23, atol=0)
+    diff = got_q != want_q[:rows]
+    assert diff.mean() <= 2e-3
+    dec = oracle.e4m3fn_decode_table()
+    if diff.any():
+        a, b = dec[got_q[diff]], dec[want_q[:rows][diff]]
+        assert np.all(np.abs(a - b) <= np.maximum(np.abs(a), np.abs(b)) * 0.126 + 2.0 ** -9)
+
+
+def test_fused_silu_feeds_the_down_projection(dev):
+    # gate_up output -> fused_silu_quantized -> grouped down matmul == f32 evaluation within tolerance
+    E, rows_per, I, N = 4, 40, 256, 384
+    T = E * rows_per
+    gen = torch.Generator().manual_seed(5)
+    h = torch.randn((T, 2 * I), generator=gen).to(torch.bfloat16)
+    off = (torch.arange(E + 1, dtype=torch.int64) * rows_per).to(torch.uint32)
+    q, s = mx.fused_silu_quantized(h.to(dev), off.to(dev), mx.blockwise_fp8_config())
+    w = synth.weights_f32(E * N, I, seed=3).reshape(E, N, I)
+    wq, ws = synth.quantize_weight_block(w)
+    cfg = mx.blockwise_fp8_config()
+    stats = torch.tensor([rows_per, E], dtype=torch.int64).to(torch.uint32)
+    y = mx.grouped_dynamic_scaled_fp8_matmul(q, wq.to(dev), s, ws.to(dev), off.to(dev), torch.arange(E, dtype=torch.int32, device=dev),
+                                             stats, cfg.input_scale, cfg.weight_scale, out_type=torch.float32).cpu()
+    g, u = h[:, :I].float(), h[:, I:].float()
+    act = g / (1 + torch.exp(-g)) * u
+    ref = torch.cat([act[e * rows_per:(e + 1) * rows_per] @ w[e].T for e in range(E)])
+    assert float((y - ref).abs().max()) <= 0.08 * float(ref.abs().max())
