@@ -20,6 +20,10 @@
  *                            test_naive_blockwise_fp8_matmul.mojo:115-138
  *   orc_matmul_rowwise       max/kernels/src/linalg/fp8_quantization.mojo:1218-1259
  *   orc_grouped_matmul       max/kernels/src/linalg/fp8_quantization.mojo:1745-1865
+ *   orc_rms_norm_fused_...   max/kernels/src/nn/normalization.mojo:3996-4175, host procedure
+ *                            max/kernels/test/gpu/nn/test_rms_norm_fused_fp8.mojo:60-126
+ *   orc_moe_create_indices   max/kernels/src/nn/moe.mojo:435-590 (canonical slot order)
+ *   orc_fused_silu           max/kernels/src/shmem/ep_comm.mojo:4409-4500, 4505-4624
  *
  * Pinned by tests/test_oracle_*.py: exhaustive decode against the closed form and
  * the committed 256-entry table; encode over every bf16 value and 2^22 sampled
@@ -33,7 +37,10 @@
  *     max-reduction is not visible in its sources);
  *   - bf16 *scales* dtype: the quotient is formed in f32 and rounded once more to
  *     bf16 here; whether the reference divides in bf16 with a single rounding is
- *     not visible in its sources (its tests only use values where both agree).
+ *     not visible in its sources (its tests only use values where both agree);
+ *   - orc_rms_norm_fused_quantize beyond the reference test's own data: the order of the
+ *     sum of squares and the rsqrt are not fixed by the reference (see the function);
+ *   - orc_fused_silu in the last bit of exp() (see the function).
  */
 #include <math.h>
 #include <stdint.h>
