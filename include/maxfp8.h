@@ -177,6 +177,18 @@ int maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8(
     float scale_ub, void* stream);
 
 /*
+ * mo.quantize_static_scaled_float8  (wrapper: max/python/max/nn/kernels.py:6753-6801;
+ * registration: builtin_kernels/quantization.mojo:1268-1315; kernel:
+ * max/kernels/src/linalg/fp8_quantization.mojo:89-141)
+ *   out[m,k] = e4m3fn(clamp(f32(in[m,k]) * (1 / scale), -448, 448))
+ * with the per-tensor scale a host scalar.  (The op's scale_is_inverted parameter has no
+ * effect in the reference -- it always multiplies by 1 / scale -- and has none here.)
+ */
+int maxfp8_quantize_static_scaled_fp8(
+    void* out_fp8, const void* in, int64_t M, int64_t K,
+    int64_t in_row_stride, int64_t out_row_stride, int in_dtype, float scale, void* stream);
+
+/*
  * mo.moe.create.indices  (wrapper: max/python/max/nn/kernels.py:4980-5060; kernel:
  * max/kernels/src/nn/moe.mojo:435-720).  Groups the n = tokens * top_k expert assignments
  * topk_ids[i] (int32 / uint32, values in [0, num_experts)) by expert:

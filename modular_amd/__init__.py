@@ -6,7 +6,8 @@ through the C ABI of include/maxfp8.h; there is no CPU or PyTorch fallback.
 """
 from .quant_config import (InputScaleSpec, QuantConfig, QuantFormat, ScaleGranularity, ScaleOrigin,
                            WeightScaleSpec, blockwise_fp8_config, rowwise_fp8_config)
-from .kernels import (dynamic_scaled_matmul, grouped_dynamic_scaled_fp8_matmul,
+from .kernels import (dynamic_scaled_matmul, grouped_dynamic_scaled_fp8_matmul, matmul_static_scaled_float8,
+                      quantize_static_scaled_float8,
                       quantize_dynamic_scaled_float8, rms_norm_fused_quantize_dynamic_scaled_fp8)
 from .moe_kernels import fused_silu, fused_silu_quantized, moe_create_indices
 from .quant_ops import matmul_float8, quantized_matmul
@@ -18,4 +19,5 @@ __all__ = [
     "grouped_dynamic_scaled_fp8_matmul", "quantize_dynamic_scaled_float8", "matmul_float8",
     "quantized_matmul", "Linear", "rms_norm_fused_quantize_dynamic_scaled_fp8",
     "moe_create_indices", "fused_silu", "fused_silu_quantized",
+    "quantize_static_scaled_float8", "matmul_static_scaled_float8",
 ]

@@ -27,6 +27,7 @@ int quantize_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int6
                       float, hipStream_t);
 int rmsnorm_quantize_dispatch(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float,
                               float, float, hipStream_t);
+int quantize_static_dispatch(void*, const void*, int64_t, int64_t, int64_t, int64_t, int, float, hipStream_t);
 int moe_create_indices_dispatch(uint32_t*, uint32_t*, uint32_t*, int32_t*, uint32_t*, const int32_t*, int64_t, int64_t, hipStream_t);
 int fused_silu_dispatch(void*, float*, const void*, const uint32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool,
                         hipStream_t);
@@ -112,6 +113,17 @@ int maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_s
   return rmsnorm_quantize_dispatch(out_fp8, out_scales, in, gamma, rows, K, in_row_stride, out_row_stride, in_dtype,
                                    scales_dtype, round_to_dtype(epsilon, in_dtype), round_to_dtype(weight_offset, in_dtype),
                                    scale_ub, (hipStream_t)stream);
+}
+
+int maxfp8_quantize_static_scaled_fp8(void* out_fp8, const void* in, int64_t M, int64_t K, int64_t in_row_stride,
+                                      int64_t out_row_stride, int in_dtype, float scale, void* stream) {
+  if (in_dtype != MAXFP8_BF16 && in_dtype != MAXFP8_F16 && in_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize_static: expected input dtype to be float16, bfloat16, or float32 (got %d)", in_dtype);
+  if (M < 0 || K < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize_static: negative size");
+  if (M == 0 || K == 0) return MAXFP8_OK;
+  if (in_row_stride < K || out_row_stride < K) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize_static: row strides smaller than the row length");
+  if (!out_fp8 || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize_static: null pointer");
+  return quantize_static_dispatch(out_fp8, in, M, K, in_row_stride, out_row_stride, in_dtype, scale, (hipStream_t)stream);
 }
 
 int maxfp8_moe_create_indices(uint32_t* token_expert_order, uint32_t* expert_start_indices, uint32_t* restore_token_order,

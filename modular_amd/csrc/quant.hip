@@ -301,6 +301,44 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_generic_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Static per-tensor quantisation: out = e4m3fn(clamp(f32(x) * (1 / scale)))
+// (max/kernels/src/linalg/fp8_quantization.mojo:89-141; the op ignores scale_is_inverted and
+// always multiplies by 1 / scale, builtin_kernels/quantization.mojo:1292-1310).
+__global__ __launch_bounds__(256) void quant_static_bf16_kernel(uint8_t* __restrict__ out, const uint16_t* __restrict__ in,
+                                                                int64_t rows, int kvec, int64_t in_stride,
+                                                                int64_t out_stride, float recip) {
+  const int64_t total = rows * kvec;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / kvec;
+    const int c = (int)(i - r * kvec);
+    const uint4 v = reinterpret_cast<const uint4*>(in + r * in_stride)[c];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[2 * j] = __uint_as_float(w[j] << 16) * recip;
+      f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u) * recip;
+    }
+    int lo = 0, hi = 0;
+    lo = cvt_pk_e4m3fn(clamp448(f[0]), clamp448(f[1]), lo, false);
+    lo = cvt_pk_e4m3fn(clamp448(f[2]), clamp448(f[3]), lo, true);
+    hi = cvt_pk_e4m3fn(clamp448(f[4]), clamp448(f[5]), hi, false);
+    hi = cvt_pk_e4m3fn(clamp448(f[6]), clamp448(f[7]), hi, true);
+    reinterpret_cast<uint2*>(out + r * out_stride)[c] = make_uint2((uint32_t)lo, (uint32_t)hi);
+  }
+}
+
+__global__ __launch_bounds__(256) void quant_static_generic_kernel(uint8_t* __restrict__ out, const void* __restrict__ in,
+                                                                   int64_t rows, int64_t K, int64_t in_stride,
+                                                                   int64_t out_stride, int in_dtype, float recip) {
+  const int64_t total = rows * K;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / K, c = i - r * K;
+    out[r * out_stride + c] = encode_one(clamp448(load_elem(in, in_dtype, r * in_stride + c) * recip));
+  }
+}
+
+// ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void cast_f32_to_e4m3fn_kernel(uint8_t* out, const float* in, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
@@ -393,6 +431,22 @@ int rmsnorm_quantize_dispatch(void* out_fp8, void* out_scales, const void* in, c
   hipLaunchKernelGGL(rmsnorm_quant_generic_kernel, dim3((unsigned)rows), dim3(256), 0, stream, (uint8_t*)out_fp8, out_scales,
                      in, gamma, (int)K, in_row_stride, out_row_stride, in_dtype, scales_dtype, epsilon, weight_offset, scale_ub);
   return launch_status("rmsnorm_quant_generic");
+}
+
+int quantize_static_dispatch(void* out_fp8, const void* in, int64_t rows, int64_t K, int64_t in_row_stride,
+                             int64_t out_row_stride, int in_dtype, float scale, hipStream_t stream) {
+  const float recip = 1.0f / scale;
+  const bool fast = in_dtype == MAXFP8_BF16 && aligned16(in) && (in_row_stride % 8 == 0) && (K % 8 == 0) &&
+                    (reinterpret_cast<uintptr_t>(out_fp8) % 8 == 0) && (out_row_stride % 8 == 0);
+  const int64_t items = fast ? rows * (K / 8) : rows * K;
+  const unsigned blocks = (unsigned)(ceil_div(items, 256) < 16384 ? ceil_div(items, 256) : 16384);
+  if (fast)
+    hipLaunchKernelGGL(quant_static_bf16_kernel, dim3(blocks), dim3(256), 0, stream, (uint8_t*)out_fp8, (const uint16_t*)in,
+                       rows, (int)(K / 8), in_row_stride, out_row_stride, recip);
+  else
+    hipLaunchKernelGGL(quant_static_generic_kernel, dim3(blocks), dim3(256), 0, stream, (uint8_t*)out_fp8, in, rows, K,
+                       in_row_stride, out_row_stride, in_dtype, recip);
+  return launch_status("quantize_static");
 }
 
 int cast_f32_to_e4m3fn_dispatch(void* out, const float* in, int64_t n, hipStream_t stream) {

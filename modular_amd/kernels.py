@@ -13,7 +13,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from .quant_config import InputScaleSpec, WeightScaleSpec
+from .quant_config import InputScaleSpec, ScaleGranularity, ScaleOrigin, WeightScaleSpec
 
 _FP8 = torch.float8_e4m3fn
 _DT = {torch.bfloat16: _lib.BF16, torch.float16: _lib.F16, torch.float32: _lib.F32, _FP8: _lib.E4M3FN}
@@ -95,6 +95,63 @@ def quantize_dynamic_scaled_float8(
         group_size, a_scales_dim1, _DT[input.dtype], _DT[scales_type], float(scale_ub), _stream(input))
     _lib.check(st)
     return out, scales
+
+
+def _host_scalar(t: torch.Tensor, what: str) -> float:
+    if tuple(t.shape) not in ((), (1,)):
+        raise ValueError(f"expected {what} to be a scalar, but got shape of {list(t.shape)}")
+    if t.device.type != "cpu":
+        raise ValueError(f"expected {what} to be on CPU, but got {t.device}")
+    return float(t.reshape(()).to(torch.float32))
+
+
+def quantize_static_scaled_float8(x: torch.Tensor, scale: torch.Tensor, scale_is_inverted: bool = True,
+                                  out_type: torch.dtype = _FP8) -> torch.Tensor:
+    """Quantizes a rank-2 tensor to float8 with a static per-tensor scale held on the CPU:
+    clamp(x * (1 / scale)) (max/python/max/nn/kernels.py:6753-6801).  `scale_is_inverted` is accepted
+    and, as in the reference's kernel, has no effect."""
+    s = _host_scalar(scale, "scale")
+    if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise ValueError(f"expected input dtype to be float16, bfloat16, or float32, but got {x.dtype}")
+    if x.dim() != 2:
+        raise ValueError(f"expected input rank to be 2, but got {x.dim()}")
+    if out_type != _FP8:
+        raise ValueError("out_type must be float8_e4m3fn")
+    _require_gpu(x)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    M, K = x.shape
+    out = torch.empty((M, K), dtype=_FP8, device=x.device)
+    st = _lib.lib().maxfp8_quantize_static_scaled_fp8(out.data_ptr(), x.data_ptr(), M, K, x.stride(0) if M > 1 else K, K,
+                                                      _DT[x.dtype], s, _stream(x))
+    _lib.check(st)
+    return out
+
+
+def matmul_static_scaled_float8(input: torch.Tensor, weight: torch.Tensor, input_scale: torch.Tensor,
+                                weight_scale: torch.Tensor) -> torch.Tensor:
+    """input @ weight.T for float8 operands with per-tensor CPU scalar scales, bfloat16 out:
+    cast(acc * (input_scale * weight_scale)) (max/python/max/nn/kernels.py:8319-8405; epilogue
+    builtin_kernels/linalg.mojo:1790-1802)."""
+    a_s = _host_scalar(input_scale, "input_scale")
+    b_s = _host_scalar(weight_scale, "weight_scale")
+    if input.dtype != _FP8:
+        raise ValueError(f"expected input dtype to be float8_e4m3fn or float8_e4m3fnuz, but got {input.dtype}")
+    if weight.dtype != _FP8:
+        raise ValueError(f"expected weight dtype to be float8_e4m3fn or float8_e4m3fnuz, but got {weight.dtype}")
+    if input.dim() != 2:
+        raise ValueError(f"expected input rank to be 2, but got {input.dim()}")
+    if weight.dim() != 2:
+        raise ValueError(f"expected weight rank to be 2, but got {weight.dim()}")
+    if input.shape[1] != weight.shape[1]:
+        raise ValueError("K dimension does not match for matmul")
+    # the product of the two scales is formed first, in f32, and applied once
+    prod = torch.tensor([[a_s]], dtype=torch.float32) * torch.tensor([[b_s]], dtype=torch.float32)
+    one = torch.ones((1, 1), dtype=torch.float32)
+    in_spec = InputScaleSpec(ScaleGranularity.TENSOR, ScaleOrigin.STATIC, torch.float32)
+    w_spec = WeightScaleSpec(ScaleGranularity.TENSOR, torch.float32)
+    return dynamic_scaled_matmul(input, weight, prod.to(input.device), one.to(input.device), in_spec, w_spec,
+                                 out_type=torch.bfloat16)
 
 
 def rms_norm_fused_quantize_dynamic_scaled_fp8(

@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import torch
 
-from .quant_config import QuantConfig, ScaleGranularity
+from .quant_config import QuantConfig, ScaleGranularity, ScaleOrigin
 from .quant_ops import quantized_matmul
 
 
@@ -40,7 +40,10 @@ class Linear(torch.nn.Module):
                              .view(torch.float8_e4m3fn))
         shape = infer_weight_scale_shape(out_dim, in_dim, quant_config)
         self.register_buffer("weight_scale", torch.ones(shape, dtype=quant_config.weight_scale.dtype, device=device))
+        # static quantisation: the pre-computed input scale is a scalar kept on the CPU (linear.py:176-184)
         self.input_scale = None
+        if quant_config.input_scale.origin == ScaleOrigin.STATIC:
+            self.input_scale = torch.ones((), dtype=quant_config.input_scale.dtype)
         if has_bias:
             self.register_buffer("bias", torch.zeros((out_dim,), dtype=quant_config.bias_dtype or bias_dtype,
                                                      device=device))

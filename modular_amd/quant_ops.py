@@ -1,12 +1,13 @@
 """FP8 dispatch of a quantised linear, mirroring `quantized_matmul` /
-`_matmul_float8` (max/python/max/nn/quant_ops.py:516-592, 336-481) for the
-dynamic-scale branches this package executes on the MI355X.
+`_matmul_float8` (max/python/max/nn/quant_ops.py:516-592, 336-481): the static
+per-tensor branch and the dynamic tensor / per-row / block branches.
 """
 from __future__ import annotations
 
 import torch
 
-from .kernels import dynamic_scaled_matmul, quantize_dynamic_scaled_float8
+from .kernels import (dynamic_scaled_matmul, matmul_static_scaled_float8, quantize_dynamic_scaled_float8,
+                      quantize_static_scaled_float8)
 from .quant_config import InputScaleSpec, QuantConfig, ScaleGranularity, WeightScaleSpec
 
 
@@ -19,8 +20,17 @@ def matmul_float8(
 ) -> torch.Tensor:
     """x @ weight.T with float8 quantisation; x [M, K] bf16, weight [N, K] e4m3fn."""
     if input_scale is not None:
-        # static activation scales (quant_ops.py:384-417) are a different operator
-        raise NotImplementedError("static FP8 activation scales are outside the dynamic FP8 linear path")
+        # Static quantisation: the input scale was computed offline (quant_ops.py:384-417).
+        xq = quantize_static_scaled_float8(x, input_scale, out_type=weight.dtype)
+        if quant_config.weight_scale.is_tensor and weight_scale.dim() >= 2:
+            # fused QKV: per-projection weight scales broadcast to rowwise [N, 1]; the scalar
+            # input scale is broadcast to the per-token layout [1, M]
+            weight_scale = weight_scale.to(x.device)
+            a_scales = input_scale.reshape(1, 1).to(device=x.device, dtype=weight_scale.dtype).expand(1, xq.shape[0]).contiguous()
+            in_spec = InputScaleSpec(ScaleGranularity.COLWISE, quant_config.input_scale.origin, weight_scale.dtype)
+            w_spec = WeightScaleSpec(ScaleGranularity.ROWWISE, weight_scale.dtype)
+            return dynamic_scaled_matmul(xq, weight, a_scales, weight_scale, in_spec, w_spec, out_type=torch.bfloat16)
+        return matmul_static_scaled_float8(xq, weight, input_scale, weight_scale)
 
     if quant_config.input_scale.is_tensor and quant_config.weight_scale.is_tensor:
         # Dynamic tensor-wise FP8 is executed as per-token x per-channel with the

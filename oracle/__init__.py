@@ -57,6 +57,8 @@ def lib() -> ctypes.CDLL:
         L.orc_grouped_matmul.argtypes = [vp] * 7 + [i64] * 7 + [ci, ci, ci]
         L.orc_rms_norm_fused_quantize.restype = ci
         L.orc_rms_norm_fused_quantize.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, cf, cf, cf, ci]
+        L.orc_quantize_static.restype = ci
+        L.orc_quantize_static.argtypes = [vp, vp, i64, i64, ci, cf]
         L.orc_moe_create_indices.restype = ci
         L.orc_moe_create_indices.argtypes = [vp] * 6 + [i64, i64]
         L.orc_fused_silu.restype = ci
@@ -153,6 +155,14 @@ def rms_norm_fused_quantize(x: np.ndarray, gamma: np.ndarray, epsilon: float, we
     if rc:
         raise ValueError(f"oracle rms_norm_fused_quantize failed: {rc}")
     return q, sc
+
+
+def quantize_static(x: np.ndarray, scale: float, *, in_dtype: int = BF16) -> np.ndarray:
+    """x: [M, K] (uint16 bits for bf16/f16, float32 for f32) -> e4m3fn bytes of clamp(x * (1 / scale))."""
+    x = np.ascontiguousarray(x)
+    q = np.zeros(x.shape, dtype=np.uint8)
+    lib().orc_quantize_static(_p(q), _p(x), x.shape[0], x.shape[1], in_dtype, scale)
+    return q
 
 
 def moe_create_indices(topk_ids: np.ndarray, num_experts: int):

@@ -20,6 +20,7 @@
  *                            test_naive_blockwise_fp8_matmul.mojo:115-138
  *   orc_matmul_rowwise       max/kernels/src/linalg/fp8_quantization.mojo:1218-1259
  *   orc_grouped_matmul       max/kernels/src/linalg/fp8_quantization.mojo:1745-1865
+ *   orc_quantize_static      max/kernels/src/linalg/fp8_quantization.mojo:89-141
  *   orc_rms_norm_fused_...   max/kernels/src/nn/normalization.mojo:3996-4175, host procedure
  *                            max/kernels/test/gpu/nn/test_rms_norm_fused_fp8.mojo:60-126
  *   orc_moe_create_indices   max/kernels/src/nn/moe.mojo:435-590 (canonical slot order)
@@ -247,6 +248,19 @@ int orc_rms_norm_fused_quantize(uint8_t* out, void* scales, const void* in, cons
       if (v < -448.0f) v = -448.0f;
       out[r * out_row_stride + c] = orc_f32_to_e4m3fn(v);
     }
+  }
+  return 0;
+}
+
+/* Static per-tensor quantisation: out = e4m3fn(clamp(f32(x) * (1 / scale)))
+ * (max/kernels/src/linalg/fp8_quantization.mojo:89-141). */
+int orc_quantize_static(uint8_t* out, const void* in, int64_t M, int64_t K, int in_dtype, float scale) {
+  const float recip = 1.0f / scale;
+  for (int64_t i = 0; i < M * K; ++i) {
+    float v = load_in(in, in_dtype, i) * recip;
+    if (v > 448.0f) v = 448.0f;
+    if (v < -448.0f) v = -448.0f;
+    out[i] = orc_f32_to_e4m3fn(v);
   }
   return 0;
 }
