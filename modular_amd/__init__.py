@@ -12,6 +12,7 @@ from .kernels import (dynamic_scaled_matmul, grouped_dynamic_scaled_fp8_matmul, 
 from .moe_kernels import fused_silu, fused_silu_quantized, moe_create_indices
 from .quant_ops import matmul_float8, quantized_matmul
 from .linear import Linear
+from .weights_quant import parse_quant_config
 
 __all__ = [
     "InputScaleSpec", "QuantConfig", "QuantFormat", "ScaleGranularity", "ScaleOrigin", "WeightScaleSpec",
@@ -19,5 +20,5 @@ __all__ = [
     "grouped_dynamic_scaled_fp8_matmul", "quantize_dynamic_scaled_float8", "matmul_float8",
     "quantized_matmul", "Linear", "rms_norm_fused_quantize_dynamic_scaled_fp8",
     "moe_create_indices", "fused_silu", "fused_silu_quantized",
-    "quantize_static_scaled_float8", "matmul_static_scaled_float8",
+    "quantize_static_scaled_float8", "matmul_static_scaled_float8", "parse_quant_config",
 ]
