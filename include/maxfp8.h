@@ -1,11 +1,12 @@
 /*
  * maxfp8.h -- C ABI of the MI355X (gfx950) FP8 linear hot path.
  *
- * Three operators, named after the MAX custom ops they stand in for:
+ * The operators, named after the MAX custom ops they stand in for:
  *
  *   mo.quantize_dynamic_scaled_float8      -> maxfp8_quantize_dynamic_scaled_fp8
  *   mo.matmul_dynamic_scaled_fp8           -> maxfp8_matmul_dynamic_scaled_fp8
  *   mo.grouped.matmul.dynamic.scaled.fp8   -> maxfp8_grouped_matmul_dynamic_scaled_fp8
+ *   mo.batched.matmul.dynamic.scaled.fp8   -> maxfp8_batched_matmul_dynamic_scaled_fp8
  *
  * Conventions (the same as the reference's destination-passing custom-op ABI,
  * max/kernels/src/graph_compiler/extensibility/decorators.mojo:46-131):
@@ -91,6 +92,30 @@ int maxfp8_quantize_dynamic_scaled_fp8(
     int in_dtype, int scales_dtype, float scale_ub, void* stream);
 
 /*
+ * Batched dynamic activation quantisation: B independent [M, K] problems in one
+ * launch.  Replaces batched_quantize_dynamic_scaled_fp8
+ *   (max/kernels/src/linalg/fp8_quantization.mojo:779-954), which the MLA
+ * graph calls on a [row, batch, col] view of its activations
+ *   (max/kernels/src/nn/attention/gpu/mla_graph.mojo:1010-1033): hence the free
+ * batch and row strides of the input.
+ *
+ *   in          element (b, m, k) at in + b * in_batch_stride + m * in_row_stride + k
+ *   out_fp8     [B, M, K]: byte (b, m, k) at b * out_batch_stride + m * out_row_stride + k
+ *   out_scales  [B, K / group_size, scales_ld]: element (b, g, m) at
+ *               b * scales_batch_stride + g * scales_ld + m
+ *   B           at most 65535; B == 0 is a no-op (fp8_quantization.mojo:826-827)
+ * Everything else as in maxfp8_quantize_dynamic_scaled_fp8; each batch gets
+ * exactly that function's result.
+ */
+int maxfp8_batched_quantize_dynamic_scaled_fp8(
+    void* out_fp8, void* out_scales, const void* in,
+    int64_t B, int64_t M, int64_t K,
+    int64_t in_batch_stride, int64_t in_row_stride,
+    int64_t out_batch_stride, int64_t out_row_stride,
+    int64_t group_size, int64_t scales_batch_stride, int64_t scales_ld,
+    int in_dtype, int scales_dtype, float scale_ub, void* stream);
+
+/*
  * Scaled FP8 matmul, C = A . B^T with B stored [N, K] ("transpose_b").
  * Replaces MatmulDynamicScaledFloat8.execute
  *   (max/kernels/src/graph_compiler/builtin_kernels/linalg.mojo:1677-1720)
@@ -128,6 +153,38 @@ int maxfp8_matmul_dynamic_scaled_fp8(
     int64_t a_scales_ld, int64_t b_scales_ld,
     int c_dtype, int scales_dtype, int algo,
     void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Batched blockwise-scaled FP8 matmul: C[b] = A[b] . B[b]^T for b < B in one
+ * launch.  Replaces Struct_batched_matmul_dynamic_scaled_fp8.execute
+ *   (max/kernels/src/graph_compiler/builtin_kernels/linalg.mojo:1041-1090)
+ * -> batched_matmul_dynamic_scaled_fp8 (max/kernels/src/linalg/bmm.mojo:1561-1660;
+ * its portable form loops the 2-D blockwise kernel over the batch, bmm.mojo:1430-1558).
+ * Block scaling only, as in the reference (max/python/max/nn/kernels.py:6693-6724).
+ *
+ *   a         [B, M, K] e4m3fn: batch stride a_batch_stride, row stride lda (bytes)
+ *   b         [B, N, K] e4m3fn: batch stride b_batch_stride, row stride ldb (bytes)
+ *   c         [B, M, N] of c_dtype: batch stride c_batch_stride, row stride ldc (elements)
+ *   a_scales  [B, ceil(K/128), a_scales_ld] f32, batch stride a_scales_batch_stride
+ *   b_scales  [B, ceil(N/128), b_scales_ld] f32, batch stride b_scales_batch_stride
+ *   B         at most 65535; B == 0 is a no-op
+ * (gm, gn, gk), c_dtype, scales_dtype and algo as in
+ * maxfp8_matmul_dynamic_scaled_fp8; each batch gets that function's result up to
+ * the order of the f32 sums (the tile shape is chosen for the whole batch and K is
+ * never split).  The MFMA kernels additionally need batch strides
+ * of a and b that are multiples of 16; AUTO falls back to the naive kernel otherwise.
+ */
+int maxfp8_batched_matmul_dynamic_scaled_fp8(
+    void* c, const void* a, const void* b,
+    const void* a_scales, const void* b_scales,
+    int64_t B, int64_t M, int64_t N, int64_t K,
+    int64_t a_batch_stride, int64_t lda,
+    int64_t b_batch_stride, int64_t ldb,
+    int64_t c_batch_stride, int64_t ldc,
+    int64_t gm, int64_t gn, int64_t gk,
+    int64_t a_scales_batch_stride, int64_t a_scales_ld,
+    int64_t b_scales_batch_stride, int64_t b_scales_ld,
+    int c_dtype, int scales_dtype, int algo, void* stream);
 
 /* Bytes of workspace that lets AUTO use every kernel for this shape. */
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K);

@@ -24,8 +24,10 @@ EXPORTS = (
     "maxfp8_last_error",
     "maxfp8_version",
     "maxfp8_quantize_dynamic_scaled_fp8",
+    "maxfp8_batched_quantize_dynamic_scaled_fp8",
     "maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8",
     "maxfp8_matmul_dynamic_scaled_fp8",
+    "maxfp8_batched_matmul_dynamic_scaled_fp8",
     "maxfp8_matmul_workspace_bytes",
     "maxfp8_grouped_matmul_dynamic_scaled_fp8",
     "maxfp8_quantize_static_scaled_fp8",
@@ -60,11 +62,15 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_version.argtypes = []
     L.maxfp8_quantize_dynamic_scaled_fp8.restype = ci
     L.maxfp8_quantize_dynamic_scaled_fp8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, cf, vp]
+    L.maxfp8_batched_quantize_dynamic_scaled_fp8.restype = ci
+    L.maxfp8_batched_quantize_dynamic_scaled_fp8.argtypes = [vp, vp, vp] + [i64] * 10 + [ci, ci, cf, vp]
     L.maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8.restype = ci
     L.maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, cf, cf, cf, vp]
     L.maxfp8_matmul_dynamic_scaled_fp8.restype = ci
     L.maxfp8_matmul_dynamic_scaled_fp8.argtypes = ([vp] * 5 + [i64] * 6 + [ci, ci] + [i64] * 5 +
                                                   [ci, ci, ci, vp, ctypes.c_size_t, vp])
+    L.maxfp8_batched_matmul_dynamic_scaled_fp8.restype = ci
+    L.maxfp8_batched_matmul_dynamic_scaled_fp8.argtypes = [vp] * 5 + [i64] * 17 + [ci, ci, ci, vp]
     L.maxfp8_matmul_workspace_bytes.restype = ctypes.c_size_t
     L.maxfp8_matmul_workspace_bytes.argtypes = [i64, i64, i64]
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8.restype = ci

@@ -24,7 +24,7 @@ int launch_status(const char* what) {
 
 // kernels (defined in the other translation units)
 int quantize_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, int,
-                      float, hipStream_t);
+                      float, int64_t, int64_t, int64_t, int64_t, hipStream_t);
 int rmsnorm_quantize_dispatch(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float,
                               float, float, hipStream_t);
 int quantize_static_dispatch(void*, const void*, int64_t, int64_t, int64_t, int64_t, int, float, hipStream_t);
@@ -35,16 +35,16 @@ int cast_f32_to_e4m3fn_dispatch(void*, const float*, int64_t, hipStream_t);
 int cast_e4m3fn_to_f32_dispatch(float*, const void*, int64_t, hipStream_t);
 int copy_bytes_dispatch(void*, const void*, int64_t, hipStream_t);
 int naive_blockwise_dispatch(void*, const void*, const void*, const void*, const void*, int64_t, int64_t, int64_t,
-                             int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int,
-                             hipStream_t);
+                             int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, int64_t, int64_t,
+                             int64_t, int64_t, int64_t, int64_t, hipStream_t);
 int naive_rowwise_dispatch(void*, const void*, const void*, const void*, const void*, int64_t, int64_t, int64_t,
                            int64_t, int64_t, int64_t, int64_t, int64_t, int, int, hipStream_t);
 int naive_grouped_dispatch(void*, const void*, const void*, const void*, const void*, const uint32_t*,
                            const int32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int, hipStream_t);
-int gemm_tiled_dispatch(const GemmArgs&, bool, size_t, hipStream_t);
+int gemm_tiled_dispatch(const GemmArgs&, bool, size_t, int64_t, hipStream_t);
 size_t gemm_tiled_workspace_bytes(int64_t, int64_t, int64_t);
 int gemm_grouped_dispatch(const GemmArgs&, int64_t, int64_t, hipStream_t);
-int gemm_skinny_dispatch(const GemmArgs&, bool, hipStream_t);
+int gemm_skinny_dispatch(const GemmArgs&, bool, int64_t, hipStream_t);
 int gemm_skinny_max_m();
 
 // v rounded to bf16 / f16 and widened back: how an op parameter of the input's dtype arrives
@@ -93,7 +93,34 @@ int maxfp8_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const vo
                 (long long)in_row_stride, (long long)out_row_stride, (long long)scales_ld);
   if (!out_fp8 || !out_scales || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize: null pointer");
   return quantize_dispatch(out_fp8, out_scales, in, M, K, in_row_stride, out_row_stride, group_size, scales_ld,
-                           in_dtype, scales_dtype, scale_ub, (hipStream_t)stream);
+                           in_dtype, scales_dtype, scale_ub, 1, 0, 0, 0, (hipStream_t)stream);
+}
+
+int maxfp8_batched_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, int64_t B, int64_t M, int64_t K,
+                                               int64_t in_batch_stride, int64_t in_row_stride, int64_t out_batch_stride,
+                                               int64_t out_row_stride, int64_t group_size, int64_t scales_batch_stride,
+                                               int64_t scales_ld, int in_dtype, int scales_dtype, float scale_ub,
+                                               void* stream) {
+  if (B < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "batched quantize: negative batch");
+  if (B == 0) return MAXFP8_OK;  // fp8_quantization.mojo:826-827
+  if (B > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "batched quantize: batch %lld exceeds 65535", (long long)B);
+  if (in_dtype != MAXFP8_BF16 && in_dtype != MAXFP8_F16 && in_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize: input dtype %d is not bf16, f16 or f32", in_dtype);
+  if (scales_dtype != MAXFP8_F32 && scales_dtype != MAXFP8_BF16)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize: scales dtype should be bfloat16 or float32 (got %d)", scales_dtype);
+  if (M < 0 || K < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: negative size M=%lld K=%lld", (long long)M, (long long)K);
+  if (M == 0 || K == 0) return MAXFP8_OK;
+  if (group_size == -1) group_size = K;
+  if (group_size <= 0 || K % group_size != 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: group size %lld must divide K = %lld", (long long)group_size, (long long)K);
+  if (group_size % 4 != 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: group size must be multiple of simd size (4), got %lld", (long long)group_size);
+  if (in_row_stride < K || out_row_stride < K || scales_ld < M)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: strides smaller than the extents");
+  if (!out_fp8 || !out_scales || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize: null pointer");
+  return quantize_dispatch(out_fp8, out_scales, in, M, K, in_row_stride, out_row_stride, group_size, scales_ld, in_dtype,
+                           scales_dtype, scale_ub, B, in_batch_stride, out_batch_stride, scales_batch_stride,
+                           (hipStream_t)stream);
 }
 
 int maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, const void* gamma,
@@ -163,12 +190,16 @@ size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return gemm_tiled_workspace_bytes(M, N, K);  // split-K partial sums; 0 when no split would be used
 }
 
-int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
-                                     const void* b_scales, int64_t M, int64_t N, int64_t K, int64_t lda,
-                                     int64_t ldb, int64_t ldc, int input_granularity, int weight_granularity,
-                                     int64_t gm, int64_t gn, int64_t gk, int64_t a_scales_ld, int64_t b_scales_ld,
-                                     int c_dtype, int scales_dtype, int algo, void* workspace,
-                                     size_t workspace_bytes, void* stream) {
+}  // extern "C"
+
+namespace maxfp8 {
+struct BatchStrides { int64_t n, a, b, c, a_scales, b_scales; };  // n batches; steps in elements
+
+static int matmul_common(void* c, const void* a, const void* b, const void* a_scales, const void* b_scales, int64_t M,
+                         int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int input_granularity,
+                         int weight_granularity, int64_t gm, int64_t gn, int64_t gk, int64_t a_scales_ld,
+                         int64_t b_scales_ld, int c_dtype, int scales_dtype, int algo, void* workspace,
+                         size_t workspace_bytes, const BatchStrides& bt, void* stream) {
   if (c_dtype != MAXFP8_BF16 && c_dtype != MAXFP8_F32)
     MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "matmul: output dtype %d is not bf16 or f32", c_dtype);
   if (M < 0 || N < 0 || K < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: negative size");
@@ -196,7 +227,8 @@ int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, cons
   // Fast kernels: f32 scales, 16-byte aligned rows, K a multiple of 16, and for
   // block scaling the (1, 128, 128) granularity.
   const bool fast_layout = is_aligned(a, 16) && is_aligned(b, 16) && lda % 16 == 0 && ldb % 16 == 0 && K % 16 == 0 &&
-                           K > 0 && scales_dtype == MAXFP8_F32 && (!block || (gm == 1 && gn == 128 && gk == 128));
+                           K > 0 && scales_dtype == MAXFP8_F32 && (!block || (gm == 1 && gn == 128 && gk == 128)) &&
+                           (bt.n == 1 || (bt.a % 16 == 0 && bt.b % 16 == 0));
   if (algo == MAXFP8_ALGO_AUTO) {
     if (!fast_layout) algo = MAXFP8_ALGO_NAIVE;
     else if (M <= gemm_skinny_max_m()) algo = MAXFP8_ALGO_SKINNY;
@@ -205,7 +237,8 @@ int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, cons
   if (algo == MAXFP8_ALGO_NAIVE) {
     if (block)
       return naive_blockwise_dispatch(c, a, b, a_scales, b_scales, M, N, K, lda, ldb, ldc, gm, gn, gk, a_scales_ld,
-                                      b_scales_ld, c_dtype, st);
+                                      b_scales_ld, c_dtype, bt.n, bt.a, bt.b, bt.c, bt.a_scales, bt.b_scales, st);
+    if (bt.n != 1) MAXFP8_FAIL(MAXFP8_ERR_GRANULARITY, "batched matmul: only block scaling is supported");
     return naive_rowwise_dispatch(c, a, b, a_scales, b_scales, M, N, K, lda, ldb, ldc, tensor ? 0 : 1,
                                   tensor ? 0 : b_scales_ld, c_dtype, scales_dtype, st);
   }
@@ -230,10 +263,45 @@ int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, cons
   p.c_dtype = c_dtype;
   p.c_vec_ok = (ldc % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
   p.c_vec8_ok = (ldc % 8 == 0) && is_aligned(c, 16);
-  if (algo == MAXFP8_ALGO_SKINNY) return gemm_skinny_dispatch(p, block, st);
+  if (bt.n != 1) {  // every batch's C must keep the alignment the vector stores assume
+    p.c_vec_ok = p.c_vec_ok && bt.c % 4 == 0;
+    p.c_vec8_ok = p.c_vec8_ok && bt.c % 8 == 0;
+  }
+  p.a_batch = bt.a; p.b_batch = bt.b; p.c_batch = bt.c;
+  p.a_scales_batch = bt.a_scales; p.b_scales_batch = bt.b_scales;
+  if (algo == MAXFP8_ALGO_SKINNY) return gemm_skinny_dispatch(p, block, bt.n, st);
   if (workspace && !is_aligned(workspace, 16)) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "matmul: workspace must be 16-byte aligned");
   p.workspace = (float*)workspace;
-  return gemm_tiled_dispatch(p, block, workspace_bytes, st);
+  return gemm_tiled_dispatch(p, block, workspace_bytes, bt.n, st);
+}
+}  // namespace maxfp8
+
+extern "C" {
+
+int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
+                                     const void* b_scales, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                     int64_t ldb, int64_t ldc, int input_granularity, int weight_granularity,
+                                     int64_t gm, int64_t gn, int64_t gk, int64_t a_scales_ld, int64_t b_scales_ld,
+                                     int c_dtype, int scales_dtype, int algo, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+  const BatchStrides one = {1, 0, 0, 0, 0, 0};
+  return matmul_common(c, a, b, a_scales, b_scales, M, N, K, lda, ldb, ldc, input_granularity, weight_granularity, gm, gn,
+                       gk, a_scales_ld, b_scales_ld, c_dtype, scales_dtype, algo, workspace, workspace_bytes, one, stream);
+}
+
+int maxfp8_batched_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
+                                             const void* b_scales, int64_t B, int64_t M, int64_t N, int64_t K,
+                                             int64_t a_batch_stride, int64_t lda, int64_t b_batch_stride, int64_t ldb,
+                                             int64_t c_batch_stride, int64_t ldc, int64_t gm, int64_t gn, int64_t gk,
+                                             int64_t a_scales_batch_stride, int64_t a_scales_ld,
+                                             int64_t b_scales_batch_stride, int64_t b_scales_ld, int c_dtype,
+                                             int scales_dtype, int algo, void* stream) {
+  if (B < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "batched matmul: negative batch");
+  if (B == 0) return MAXFP8_OK;
+  if (B > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "batched matmul: batch %lld exceeds 65535", (long long)B);
+  const BatchStrides bt = {B, a_batch_stride, b_batch_stride, c_batch_stride, a_scales_batch_stride, b_scales_batch_stride};
+  return matmul_common(c, a, b, a_scales, b_scales, M, N, K, lda, ldb, ldc, MAXFP8_GRAN_BLOCK, MAXFP8_GRAN_BLOCK, gm, gn, gk,
+                       a_scales_ld, b_scales_ld, c_dtype, scales_dtype, algo, nullptr, 0, bt, stream);
 }
 
 int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,

@@ -25,9 +25,24 @@ struct GemmArgs {
   int big_rows, big_bm;      // slots with at least big_rows rows give their full big_bm-row tiles to the large-tile launch (0: none)
   int64_t b_expert_stride;   // bytes between experts in b
   int64_t bs_expert_stride;  // elements between experts in b_scales
+  // batched only: blockIdx.z (tiled) / blockIdx.y (skinny) steps the five base pointers, in elements
+  int64_t a_batch, b_batch, c_batch, a_scales_batch, b_scales_batch;
   // split-K / skinny only
   float* workspace;
   int splits;
 };
+
+#if defined(__HIPCC__)
+// the arguments of batch `b` of a batched matmul
+__device__ __forceinline__ GemmArgs batch_view(const GemmArgs& p, int64_t b) {
+  GemmArgs q = p;
+  q.a += b * p.a_batch;
+  q.b += b * p.b_batch;
+  q.c = reinterpret_cast<uint8_t*>(p.c) + b * p.c_batch * (p.c_dtype == 0 /* bf16 */ ? 2 : 4);
+  q.a_scales += b * p.a_scales_batch;
+  q.b_scales += b * p.b_scales_batch;
+  return q;
+}
+#endif
 
 }  // namespace maxfp8

@@ -63,7 +63,8 @@ struct SkinnyCfg {
 };
 
 template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
-__global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p) {
+__global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in) {
+  const GemmArgs p = gridDim.y == 1 ? p_in : batch_view(p_in, blockIdx.y);
   using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
   constexpr int WAVES = Cfg::WAVES, DEPTH = Cfg::DEPTH, SLOT = Cfg::SLOT, PER = Cfg::PER;
   static_assert((DEPTH - 1) * PER < 64, "vmcnt is a 6-bit counter");
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p) {
 }
 
 template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
-static int launch_skinny_r(const GemmArgs& p, hipStream_t stream) {
+static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream) {
   using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
   auto kern = gemm_skinny_kernel<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
   static bool attr_done = false;
@@ -265,7 +266,7 @@ static int launch_skinny_r(const GemmArgs& p, hipStream_t stream) {
     attr_done = true;
   }
   const int64_t blocks = ceil_div(p.N, 16 * NTW);
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NWAVES * 64), Cfg::SMEM, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, (unsigned)batch), dim3(NWAVES * 64), Cfg::SMEM, stream, p);
   return launch_status("gemm_skinny");
 }
 
@@ -276,32 +277,32 @@ static int launch_skinny_r(const GemmArgs& p, hipStream_t stream) {
 // (8 waves per block were tried for the small-N shapes and were slower.)
 // MAXFP8_SKINNY=<ntw>4<ringKB>, e.g. 1408 or 2416, forces a shape for tuning runs.
 template <int MT, bool BLOCKSCALE>
-static int pick_ntw(const GemmArgs& p, hipStream_t stream) {
+static int pick_ntw(const GemmArgs& p, int64_t batch, hipStream_t stream) {
   const char* e = getenv("MAXFP8_SKINNY");
   int sel = e ? atoi(e) : 0;
   if (!sel) sel = (p.N >= 16384 && MT <= 2) ? 2416 : 1408;
   switch (sel) {
-    case 1408: return launch_skinny_r<1, MT, BLOCKSCALE, 8, 4>(p, stream);
-    case 1416: return launch_skinny_r<1, MT, BLOCKSCALE, 16, 4>(p, stream);
-    case 2416: return launch_skinny_r<2, MT, BLOCKSCALE, 16, 4>(p, stream);
-    case 2408: return launch_skinny_r<2, MT, BLOCKSCALE, 8, 4>(p, stream);
+    case 1408: return launch_skinny_r<1, MT, BLOCKSCALE, 8, 4>(p, batch, stream);
+    case 1416: return launch_skinny_r<1, MT, BLOCKSCALE, 16, 4>(p, batch, stream);
+    case 2416: return launch_skinny_r<2, MT, BLOCKSCALE, 16, 4>(p, batch, stream);
+    case 2408: return launch_skinny_r<2, MT, BLOCKSCALE, 8, 4>(p, batch, stream);
     default: MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "skinny matmul: unknown shape selector %d", sel);
   }
 }
 
 int gemm_skinny_max_m() { return 64; }
 
-int gemm_skinny_dispatch(const GemmArgs& p, bool blockscale, hipStream_t stream) {
+int gemm_skinny_dispatch(const GemmArgs& p, bool blockscale, int64_t batch, hipStream_t stream) {
   if (p.M > 64) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "skinny matmul: M = %d exceeds 64", p.M);
   const int mt = (p.M + 15) / 16;
   if (blockscale) {
-    if (mt <= 1) return pick_ntw<1, true>(p, stream);
-    if (mt <= 2) return pick_ntw<2, true>(p, stream);
-    return pick_ntw<4, true>(p, stream);
+    if (mt <= 1) return pick_ntw<1, true>(p, batch, stream);
+    if (mt <= 2) return pick_ntw<2, true>(p, batch, stream);
+    return pick_ntw<4, true>(p, batch, stream);
   }
-  if (mt <= 1) return pick_ntw<1, false>(p, stream);
-  if (mt <= 2) return pick_ntw<2, false>(p, stream);
-  return pick_ntw<4, false>(p, stream);
+  if (mt <= 1) return pick_ntw<1, false>(p, batch, stream);
+  if (mt <= 2) return pick_ntw<2, false>(p, batch, stream);
+  return pick_ntw<4, false>(p, batch, stream);
 }
 
 }  // namespace maxfp8

@@ -372,7 +372,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
   const int in_group = pid - group * per_group;
   const int tm = first_m + in_group % gsize;
   const int tn = in_group / gsize;
-  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false>(p, smem, (int64_t)tm * BM, p.M, tn * BN, p.b, p.b_scales);
+  const GemmArgs q = gridDim.z == 1 ? p : batch_view(p, blockIdx.z);
+  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false>(q, smem, (int64_t)tm * BM, q.M, tn * BN, q.b, q.b_scales);
 }
 
 // ---- grouped (MoE) matmul ---------------------------------------------------------------------
@@ -592,12 +593,12 @@ static int pick_splits(int64_t tiles, int slots, int nslab) {
 }
 
 // cost of a shape (microseconds) = rounds of resident blocks * time of one tile
-static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can_split) {
+static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can_split, int64_t batch = 1) {
   int best = 0;
   float best_cost = 0.f;
   for (int i = 0; i < 3; ++i) {
     const TileShape& t = kShapes[i];
-    const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+    const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn) * batch;
     const int sp = can_split ? pick_splits(tiles, t.slots, nslab) : 1;
     float cost = (float)ceil_div(tiles * sp, t.slots) *
                  ((float)ceil_div(nslab, sp) * (blockscale ? t.t_slab_block : t.t_slab_row) + t.t_tile);
@@ -621,20 +622,20 @@ size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return worst * (size_t)M * (size_t)N * 4;
 }
 
-int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, hipStream_t stream) {
+int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, int64_t batch, hipStream_t stream) {
   GemmArgs p = p_in;
   const int nslab = (p.K + 127) / 128;
   int variant = tile_override();
-  if (!variant) variant = pick_shape(p.M, p.N, nslab, blockscale, p.workspace != nullptr);
+  if (!variant) variant = pick_shape(p.M, p.N, nslab, blockscale, p.workspace != nullptr && batch == 1, batch);
   const TileShape& t = kShapes[variant - 1];
   const int64_t tiles = ceil_div(p.M, t.bm) * ceil_div(p.N, t.bn);
   if (tiles >= ((int64_t)1 << 31)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "tiled matmul: too many tiles");
   p.splits = 1;
-  if (p.workspace) {
+  if (p.workspace && batch == 1) {
     const int sp = pick_splits(tiles, t.slots, (p.K + 127) / 128);
     if (sp > 1 && (size_t)sp * p.M * p.N * 4 <= workspace_bytes) p.splits = sp;
   }
-  const dim3 grid((unsigned)tiles, (unsigned)p.splits);
+  const dim3 grid((unsigned)tiles, (unsigned)p.splits, (unsigned)batch);
   const int rc = gemm_tiled_launch(p, blockscale, variant, grid, stream);
   if (rc != MAXFP8_OK || p.splits == 1) return rc;
   const int64_t quads = ceil_div((int64_t)p.M * p.N, 4);

@@ -41,7 +41,13 @@ __device__ __forceinline__ float blockwise_dot(const uint8_t* ar, const uint8_t*
 __global__ __launch_bounds__(256) void naive_blockwise_kernel(
     void* c, const uint8_t* a, const uint8_t* b, const float* a_scales, const float* b_scales, int64_t M,
     int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t gm, int64_t gn, int64_t gk,
-    int64_t a_scales_ld, int64_t b_scales_ld, int c_dtype) {
+    int64_t a_scales_ld, int64_t b_scales_ld, int c_dtype, int64_t a_batch, int64_t b_batch, int64_t c_batch,
+    int64_t as_batch, int64_t bs_batch) {
+  a += blockIdx.z * a_batch;
+  b += blockIdx.z * b_batch;
+  c = reinterpret_cast<uint8_t*>(c) + blockIdx.z * c_batch * (c_dtype == MAXFP8_BF16 ? 2 : 4);
+  a_scales += blockIdx.z * as_batch;
+  b_scales += blockIdx.z * bs_batch;
   const int64_t n = (int64_t)blockIdx.x * 16 + (threadIdx.x & 15);
   const int64_t m = (int64_t)blockIdx.y * 16 + (threadIdx.x >> 4);
   if (m >= M || n >= N) return;
@@ -89,12 +95,14 @@ __global__ __launch_bounds__(256) void naive_grouped_kernel(
 int naive_blockwise_dispatch(void* c, const void* a, const void* b, const void* a_scales, const void* b_scales,
                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t gm,
                              int64_t gn, int64_t gk, int64_t a_scales_ld, int64_t b_scales_ld, int c_dtype,
-                             hipStream_t stream) {
+                             int64_t batch, int64_t a_batch, int64_t b_batch, int64_t c_batch, int64_t as_batch,
+                             int64_t bs_batch, hipStream_t stream) {
   const int64_t gy = ceil_div(M, 16);
   if (gy > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "naive matmul: M = %lld too large (limit 1048560)", (long long)M);
-  hipLaunchKernelGGL(naive_blockwise_kernel, dim3((unsigned)ceil_div(N, 16), (unsigned)gy), dim3(256), 0, stream,
-                     c, (const uint8_t*)a, (const uint8_t*)b, (const float*)a_scales, (const float*)b_scales, M, N,
-                     K, lda, ldb, ldc, gm, gn, gk, a_scales_ld, b_scales_ld, c_dtype);
+  hipLaunchKernelGGL(naive_blockwise_kernel, dim3((unsigned)ceil_div(N, 16), (unsigned)gy, (unsigned)batch), dim3(256), 0,
+                     stream, c, (const uint8_t*)a, (const uint8_t*)b, (const float*)a_scales, (const float*)b_scales, M, N,
+                     K, lda, ldb, ldc, gm, gn, gk, a_scales_ld, b_scales_ld, c_dtype, a_batch, b_batch, c_batch, as_batch,
+                     bs_batch);
   return launch_status("naive_blockwise");
 }
 

@@ -23,12 +23,18 @@
 
 namespace maxfp8 {
 
+// Batched launches (blockIdx.y = batch) step the three base pointers by these element counts.
+struct BatchStep { int64_t in, out, scales; };
+
 // ---------------------------------------------------------------------------
 template <int U>
 __global__ __launch_bounds__(256) void quant_g128_bf16_kernel(
     uint8_t* __restrict__ out, float* __restrict__ scales, const uint16_t* __restrict__ in,
     int M, int ngroups, int nxb, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
-    float scale_ub) {
+    float scale_ub, BatchStep bs) {
+  in += blockIdx.y * bs.in;
+  out += blockIdx.y * bs.out;
+  scales += blockIdx.y * bs.scales;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int seg = lane >> 4, sl = lane & 15;
   const int rb = blockIdx.x / nxb, xb = blockIdx.x - rb * nxb;
@@ -83,7 +89,10 @@ __global__ __launch_bounds__(256) void quant_g128_bf16_kernel(
 template <int NV>
 __global__ __launch_bounds__(256) void quant_row_bf16_kernel(
     uint8_t* __restrict__ out, float* __restrict__ scales, const uint16_t* __restrict__ in,
-    int K, int64_t in_stride, int64_t out_stride, float scale_ub) {
+    int K, int64_t in_stride, int64_t out_stride, float scale_ub, BatchStep bs) {
+  in += blockIdx.y * bs.in;
+  out += blockIdx.y * bs.out;
+  scales += blockIdx.y * bs.scales;
   __shared__ float red[4];
   const int row = blockIdx.x, tid = threadIdx.x;
   const uint16_t* src = in + (int64_t)row * in_stride;
@@ -148,7 +157,10 @@ __device__ __forceinline__ uint8_t encode_one(float v) {
 __global__ __launch_bounds__(256) void quant_generic_kernel(
     uint8_t* __restrict__ out, void* __restrict__ scales, const void* __restrict__ in,
     int ngroups, int G, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
-    int in_dtype, int scales_dtype, float scale_ub) {
+    int in_dtype, int scales_dtype, float scale_ub, BatchStep bs) {
+  in = reinterpret_cast<const uint8_t*>(in) + blockIdx.y * bs.in * (in_dtype == MAXFP8_F32 ? 4 : 2);
+  out += blockIdx.y * bs.out;
+  scales = reinterpret_cast<uint8_t*>(scales) + blockIdx.y * bs.scales * (scales_dtype == MAXFP8_F32 ? 4 : 2);
   __shared__ float red[4];
   const int row = blockIdx.x / ngroups, g = blockIdx.x - row * ngroups;
   const int tid = threadIdx.x;
@@ -365,19 +377,22 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M, int64_t K,
                       int64_t in_row_stride, int64_t out_row_stride, int64_t G, int64_t scales_ld,
-                      int in_dtype, int scales_dtype, float scale_ub, hipStream_t stream) {
+                      int in_dtype, int scales_dtype, float scale_ub, int64_t batch, int64_t in_batch_stride,
+                      int64_t out_batch_stride, int64_t scales_batch_stride, hipStream_t stream) {
+  const BatchStep bs = {in_batch_stride, out_batch_stride, scales_batch_stride};
+  const unsigned nb = (unsigned)batch;
   const int64_t ngroups = K / G;
   const bool fast_types = in_dtype == MAXFP8_BF16 && scales_dtype == MAXFP8_F32;
   const bool vec_ok = aligned16(in) && (in_row_stride % 8 == 0) && (reinterpret_cast<uintptr_t>(out_fp8) % 8 == 0) &&
-                      (out_row_stride % 8 == 0);
+                      (out_row_stride % 8 == 0) && (in_batch_stride % 8 == 0) && (out_batch_stride % 8 == 0);
   if (fast_types && vec_ok && G == 128) {
     constexpr int U = 4;
     const int64_t nxb = ceil_div(ngroups, U);
     const int64_t blocks = ceil_div(M, 16) * nxb;
     if (blocks < (int64_t)1 << 31) {
-      hipLaunchKernelGGL(quant_g128_bf16_kernel<U>, dim3((unsigned)blocks), dim3(256), 0, stream,
+      hipLaunchKernelGGL(quant_g128_bf16_kernel<U>, dim3((unsigned)blocks, nb), dim3(256), 0, stream,
                          (uint8_t*)out_fp8, (float*)out_scales, (const uint16_t*)in, (int)M, (int)ngroups,
-                         (int)nxb, in_row_stride, out_row_stride, scales_ld, scale_ub);
+                         (int)nxb, in_row_stride, out_row_stride, scales_ld, scale_ub, bs);
       return launch_status("quant_g128_bf16");
     }
   }
@@ -388,8 +403,8 @@ int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M
     float* s = (float*)out_scales;
     const uint16_t* x = (const uint16_t*)in;
 #define LAUNCH_ROW(NV)                                                                            \
-  hipLaunchKernelGGL(quant_row_bf16_kernel<NV>, dim3((unsigned)M), dim3(256), 0, stream, o, s, x, \
-                     (int)K, in_row_stride, out_row_stride, scale_ub)
+  hipLaunchKernelGGL(quant_row_bf16_kernel<NV>, dim3((unsigned)M, nb), dim3(256), 0, stream, o, s, x, \
+                     (int)K, in_row_stride, out_row_stride, scale_ub, bs)
     if (nv <= 1) LAUNCH_ROW(1);
     else if (nv <= 2) LAUNCH_ROW(2);
     else if (nv <= 4) LAUNCH_ROW(4);
@@ -400,9 +415,9 @@ int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M
   }
   const int64_t blocks = M * ngroups;
   if (blocks >= (int64_t)1 << 31) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: M * K/group_size = %lld exceeds the grid limit", (long long)blocks);
-  hipLaunchKernelGGL(quant_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint8_t*)out_fp8,
+  hipLaunchKernelGGL(quant_generic_kernel, dim3((unsigned)blocks, nb), dim3(256), 0, stream, (uint8_t*)out_fp8,
                      out_scales, in, (int)ngroups, (int)G, in_row_stride, out_row_stride, scales_ld, in_dtype,
-                     scales_dtype, scale_ub);
+                     scales_dtype, scale_ub, bs);
   return launch_status("quant_generic");
 }
 

@@ -4,6 +4,7 @@ of the reference's graph-op wrappers:
   quantize_dynamic_scaled_float8      max/python/max/nn/kernels.py:6876-6957
   dynamic_scaled_matmul               max/python/max/nn/kernels.py:6960-7078
   grouped_dynamic_scaled_fp8_matmul   max/python/max/nn/kernels.py:6327-6487
+  batched_dynamic_scaled_fp8_matmul   max/python/max/nn/kernels.py:6642-6751
 
 They take torch tensors that live on the MI355X and call the HIP kernels through
 the C ABI on torch's current stream.  Nothing here computes on the CPU.
@@ -294,6 +295,123 @@ def dynamic_scaled_matmul(
         c.data_ptr(), a.data_ptr(), b.data_ptr(), a_scales.data_ptr(), b_scales.data_ptr(), M, N, K,
         lda, ldb, N, gin, gw, gm, gn, gk, a_ld, b_ld, _DT[out_type], _DT[a_scales.dtype], _ALGOS[algo],
         ws.data_ptr() if ws is not None else None, ws_bytes, _stream(a))
+    _lib.check(st)
+    return c
+
+
+def batched_quantize_dynamic_scaled_fp8(
+    input: torch.Tensor,
+    group_size_or_per_token: int = 128,
+    scale_ub: float = 1200.0,
+    scales_type: torch.dtype = torch.float32,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantize every [M, K] slice of `input` [B, M, K] in one launch.
+
+    The eager form of batched_quantize_dynamic_scaled_fp8
+    (max/kernels/src/linalg/fp8_quantization.mojo:779-954).  `input` may be any view
+    whose last axis is contiguous, e.g. the [row, batch, col] -> [batch, row, col]
+    transpose the MLA graph quantizes (mla_graph.mojo:1010-1033): it is read in place.
+    Returns (quantized [B, M, K] e4m3fn, scales [B, K / group, M_pad]); M_pad rounds
+    M up to 16 bytes of scales, the shape batched_dynamic_scaled_fp8_matmul expects.
+    """
+    if input.dim() != 3:
+        raise ValueError("input must be rank 3 tensor")
+    if scales_type not in (torch.float32, torch.bfloat16):
+        raise TypeError("scales dtype should be bfloat16 or float32")
+    if input.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError(f"input dtype {input.dtype} is not bfloat16, float16 or float32")
+    B, M, K = input.shape
+    group_size = K if group_size_or_per_token == -1 else group_size_or_per_token
+    if group_size <= 0 or K % group_size != 0:
+        raise ValueError(f"group size {group_size} must divide K = {K}")
+    _require_gpu(input)
+    if input.stride(2) != 1 and K > 1:
+        input = input.contiguous()
+    pad = 16 // torch.empty((), dtype=scales_type).element_size()
+    m_pad = -(-M // pad) * pad
+    out = torch.empty((B, M, K), dtype=_FP8, device=input.device)
+    scales = torch.empty((B, K // group_size, m_pad), dtype=scales_type, device=input.device)
+    st = _lib.lib().maxfp8_batched_quantize_dynamic_scaled_fp8(
+        out.data_ptr(), scales.data_ptr(), input.data_ptr(), B, M, K,
+        input.stride(0) if B > 1 else M * K, input.stride(1) if M > 1 else K, M * K, K,
+        group_size, (K // group_size) * m_pad, m_pad, _DT[input.dtype], _DT[scales_type], float(scale_ub),
+        _stream(input))
+    _lib.check(st)
+    return out, scales
+
+
+def batched_dynamic_scaled_fp8_matmul(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    input_scale_spec: InputScaleSpec,
+    weight_scale_spec: WeightScaleSpec,
+    out_type: torch.dtype = torch.bfloat16,
+    *,
+    algo: str = "auto",
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """C[i] = A[i] . B[i]^T with blockwise scaling factors; a [B, M, K], b [B, N, K],
+    a_scales [B, ceil(K/128), M_pad], b_scales [B, ceil(N/128), ceil(K/128)].
+    `out`, if given, is a [B, M, N] view with a contiguous last axis that receives the
+    result in place (e.g. the [M, B, N] buffer the MLA graph writes, transposed)."""
+    if a.dtype != b.dtype:
+        raise TypeError(f"a and b dtypes must match, but got {a.dtype}, {b.dtype}")
+    if a_scales.dtype != b_scales.dtype or a_scales.dtype != torch.float32:
+        raise TypeError(f"a_scales and b_scales dtypes must be float32, but got {a_scales.dtype}, {b_scales.dtype}")
+    if a.dim() != 3 or b.dim() != 3:
+        raise ValueError("A and B must be rank 3 tensors")
+    if a_scales.dim() != 3 or b_scales.dim() != 3:
+        raise ValueError("A_scales and B_scales must be rank 3 tensors")
+    if a.shape[0] != b.shape[0]:
+        raise ValueError("The batch dimension of b must match the batch dimension of a")
+    if a.shape[2] != b.shape[2]:
+        raise ValueError("A and B K dimension does not match")
+    if a.dtype != _FP8:
+        raise TypeError(f"a and b dtypes must be float8_e4m3fn, but got {a.dtype}, {b.dtype}")
+    if not (input_scale_spec.is_block and weight_scale_spec.is_block):
+        raise ValueError("unsupported FP8 scaling granularity")
+    if a_scales.shape[0] != b_scales.shape[0]:
+        raise ValueError("both a_scales and b_scales must have the same shape on the batch dimension")
+    if input_scale_spec.block_size is None or weight_scale_spec.block_size is None:
+        raise ValueError("both input scale_granularity and weight scale_granularity must be set for batched "
+                         "blockwise scaling")
+    if tuple(input_scale_spec.block_size) != (1, 128):
+        raise ValueError("batched blockwise scaling only supports (1,128) granularity for input")
+    if tuple(weight_scale_spec.block_size) != (128, 128):
+        raise ValueError("batched blockwise scaling only supports (128,128) granularity for weight")
+    if out_type not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"out_type {out_type} is not bfloat16 or float32")
+    B, M, K = a.shape
+    N = b.shape[1]
+    if a_scales.shape[0] != B or a_scales.shape[1] != -(-K // 128) or a_scales.shape[2] < M:
+        raise ValueError(f"a_scales shape {tuple(a_scales.shape)} does not cover a {tuple(a.shape)}")
+    if b_scales.shape[1] != -(-N // 128) or b_scales.shape[2] != -(-K // 128):
+        raise ValueError(f"b_scales shape {tuple(b_scales.shape)} does not cover b {tuple(b.shape)}")
+
+    _require_gpu(a, b, a_scales, b_scales)
+    a, b, a_scales, b_scales = (t if t.stride(2) == 1 or t.shape[2] == 1 else t.contiguous()
+                                for t in (a, b, a_scales, b_scales))
+    if out is None:
+        c = torch.empty((B, M, N), dtype=out_type, device=a.device)
+    else:
+        if tuple(out.shape) != (B, M, N) or out.dtype != out_type or (N > 1 and out.stride(2) != 1):
+            raise ValueError(f"out must be a [{B}, {M}, {N}] {out_type} view with a contiguous last axis")
+        _require_gpu(out)
+        c = out
+
+    def steps(t: torch.Tensor) -> tuple[int, int]:  # (batch, row) strides, well defined for extent-1 axes too
+        rows, cols = t.shape[1], t.shape[2]
+        row = t.stride(1) if rows > 1 else cols
+        return (t.stride(0) if t.shape[0] > 1 else rows * row), row
+
+    (a_bs, lda), (b_bs, ldb), (c_bs, ldc) = steps(a), steps(b), steps(c)
+    (as_bs, a_ld), (bs_bs, b_ld) = steps(a_scales), steps(b_scales)
+    st = _lib.lib().maxfp8_batched_matmul_dynamic_scaled_fp8(
+        c.data_ptr(), a.data_ptr(), b.data_ptr(), a_scales.data_ptr(), b_scales.data_ptr(), B, M, N, K,
+        a_bs, lda, b_bs, ldb, c_bs, ldc, 1, 128, 128, as_bs, a_ld, bs_bs, b_ld, _DT[out_type], _lib.F32,
+        _ALGOS[algo], _stream(a))
     _lib.check(st)
     return c
 
