@@ -246,6 +246,25 @@ int maxfp8_quantize_static_scaled_fp8(
     int64_t in_row_stride, int64_t out_row_stride, int in_dtype, float scale, void* stream);
 
 /*
+ * Dynamic per-tensor quantisation: one scale for the whole [M, K] tensor.
+ * Replaces QuantizeTensorDynamicScaledFloat8.execute
+ *   (max/kernels/src/graph_compiler/builtin_kernels/quantization.mojo:1318-1360)
+ * -> quantize_tensor_dynamic_scaled_fp8 (max/kernels/src/linalg/fp8_quantization.mojo:209-360).
+ *
+ *   out_scales  [1, M] of scales_dtype: EVERY element receives the tensor's scale
+ *               min(max |x|, scale_ub) / 448 (the reference guarantees it only for
+ *               element 0, which is what its callers read, quant_ops.py:451).  The
+ *               buffer doubles as the scratch of the row maxima during the call.
+ *   out_fp8     e4m3fn(clamp(x * (1 / scale))) with the guarded reciprocal of
+ *               maxfp8_quantize_dynamic_scaled_fp8
+ *   K           a multiple of 4 (the reference's smallest vector width)
+ */
+int maxfp8_quantize_tensor_dynamic_scaled_fp8(
+    void* out_fp8, void* out_scales, const void* in,
+    int64_t M, int64_t K, int64_t in_row_stride, int64_t out_row_stride,
+    int in_dtype, int scales_dtype, float scale_ub, void* stream);
+
+/*
  * mo.moe.create.indices  (wrapper: max/python/max/nn/kernels.py:4980-5060; kernel:
  * max/kernels/src/nn/moe.mojo:435-720).  Groups the n = tokens * top_k expert assignments
  * topk_ids[i] (int32 / uint32, values in [0, num_experts)) by expert:

@@ -8,7 +8,7 @@ from .quant_config import (InputScaleSpec, QuantConfig, QuantFormat, ScaleGranul
                            WeightScaleSpec, blockwise_fp8_config, rowwise_fp8_config)
 from .kernels import (batched_dynamic_scaled_fp8_matmul, batched_quantize_dynamic_scaled_fp8, dynamic_scaled_matmul,
                       grouped_dynamic_scaled_fp8_matmul, matmul_static_scaled_float8,
-                      quantize_static_scaled_float8,
+                      quantize_static_scaled_float8, quantize_tensor_dynamic_scaled_float8,
                       quantize_dynamic_scaled_float8, rms_norm_fused_quantize_dynamic_scaled_fp8)
 from .moe_kernels import fused_silu, fused_silu_quantized, moe_create_indices
 from .quant_ops import matmul_float8, quantized_matmul
@@ -23,4 +23,5 @@ __all__ = [
     "moe_create_indices", "fused_silu", "fused_silu_quantized",
     "quantize_static_scaled_float8", "matmul_static_scaled_float8", "parse_quant_config",
     "batched_dynamic_scaled_fp8_matmul", "batched_quantize_dynamic_scaled_fp8",
+    "quantize_tensor_dynamic_scaled_float8",
 ]

@@ -31,6 +31,7 @@ EXPORTS = (
     "maxfp8_matmul_workspace_bytes",
     "maxfp8_grouped_matmul_dynamic_scaled_fp8",
     "maxfp8_quantize_static_scaled_fp8",
+    "maxfp8_quantize_tensor_dynamic_scaled_fp8",
     "maxfp8_moe_create_indices",
     "maxfp8_fused_silu",
     "maxfp8_cast_f32_to_e4m3fn",
@@ -77,6 +78,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8.argtypes = [vp] * 7 + [i64] * 7 + [ci, ci, ci, vp]
     L.maxfp8_quantize_static_scaled_fp8.restype = ci
     L.maxfp8_quantize_static_scaled_fp8.argtypes = [vp, vp, i64, i64, i64, i64, ci, cf, vp]
+    L.maxfp8_quantize_tensor_dynamic_scaled_fp8.restype = ci
+    L.maxfp8_quantize_tensor_dynamic_scaled_fp8.argtypes = [vp, vp, vp, i64, i64, i64, i64, ci, ci, cf, vp]
     L.maxfp8_moe_create_indices.restype = ci
     L.maxfp8_moe_create_indices.argtypes = [vp] * 6 + [i64, i64, vp]
     L.maxfp8_fused_silu.restype = ci

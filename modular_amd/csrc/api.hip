@@ -28,6 +28,7 @@ int quantize_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int6
 int rmsnorm_quantize_dispatch(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float,
                               float, float, hipStream_t);
 int quantize_static_dispatch(void*, const void*, int64_t, int64_t, int64_t, int64_t, int, float, hipStream_t);
+int quantize_tensor_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float, hipStream_t);
 int moe_create_indices_dispatch(uint32_t*, uint32_t*, uint32_t*, int32_t*, uint32_t*, const int32_t*, int64_t, int64_t, hipStream_t);
 int fused_silu_dispatch(void*, float*, const void*, const uint32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool,
                         hipStream_t);
@@ -151,6 +152,23 @@ int maxfp8_quantize_static_scaled_fp8(void* out_fp8, const void* in, int64_t M, 
   if (in_row_stride < K || out_row_stride < K) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize_static: row strides smaller than the row length");
   if (!out_fp8 || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize_static: null pointer");
   return quantize_static_dispatch(out_fp8, in, M, K, in_row_stride, out_row_stride, in_dtype, scale, (hipStream_t)stream);
+}
+
+int maxfp8_quantize_tensor_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, int64_t M, int64_t K,
+                                              int64_t in_row_stride, int64_t out_row_stride, int in_dtype, int scales_dtype,
+                                              float scale_ub, void* stream) {
+  if (in_dtype != MAXFP8_BF16 && in_dtype != MAXFP8_F16 && in_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize_tensor: input dtype %d is not bf16, f16 or f32", in_dtype);
+  if (scales_dtype != MAXFP8_F32 && scales_dtype != MAXFP8_BF16)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize_tensor: scales dtype should be bfloat16 or float32 (got %d)", scales_dtype);
+  if (M < 0 || K < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize_tensor: negative size");
+  if (M == 0 || K == 0) return MAXFP8_OK;  // fp8_quantization.mojo:296-297
+  if (M >= ((int64_t)1 << 31)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize_tensor: M must fit 31 bits");
+  if (K % 4 != 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize_tensor: group size must be multiple of simd size (4), got %lld", (long long)K);
+  if (in_row_stride < K || out_row_stride < K) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize_tensor: row strides smaller than the row length");
+  if (!out_fp8 || !out_scales || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize_tensor: null pointer");
+  return quantize_tensor_dispatch(out_fp8, out_scales, in, M, K, in_row_stride, out_row_stride, in_dtype, scales_dtype,
+                                  scale_ub, (hipStream_t)stream);
 }
 
 int maxfp8_moe_create_indices(uint32_t* token_expert_order, uint32_t* expert_start_indices, uint32_t* restore_token_order,

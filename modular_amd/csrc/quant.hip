@@ -153,6 +153,16 @@ __device__ __forceinline__ uint8_t encode_one(float v) {
   return (uint8_t)(cvt_pk_e4m3fn(v, 0.0f, 0, false) & 0xff);
 }
 
+// 1 / scale as the dynamic quantisers use it: 0 for a zero scale or a reciprocal that overflows
+__device__ __forceinline__ float guarded_recip(float scale) {
+  float r = 0.0f;
+  if (scale != 0.0f) {
+    r = 1.0f / scale;
+    if (isinf(r) || isnan(r)) r = 0.0f;
+  }
+  return r;
+}
+
 // One block per (row, group); any group size, dtype and alignment.
 __global__ __launch_bounds__(256) void quant_generic_kernel(
     uint8_t* __restrict__ out, void* __restrict__ scales, const void* __restrict__ in,
@@ -318,7 +328,9 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_generic_kernel(
 // always multiplies by 1 / scale, builtin_kernels/quantization.mojo:1292-1310).
 __global__ __launch_bounds__(256) void quant_static_bf16_kernel(uint8_t* __restrict__ out, const uint16_t* __restrict__ in,
                                                                 int64_t rows, int kvec, int64_t in_stride,
-                                                                int64_t out_stride, float recip) {
+                                                                int64_t out_stride, float recip, const void* scale_ptr,
+                                                                int scales_dtype) {
+  if (scale_ptr) recip = guarded_recip(load_elem(scale_ptr, scales_dtype, 0));
   const int64_t total = rows * kvec;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t r = i / kvec;
@@ -342,11 +354,73 @@ __global__ __launch_bounds__(256) void quant_static_bf16_kernel(uint8_t* __restr
 
 __global__ __launch_bounds__(256) void quant_static_generic_kernel(uint8_t* __restrict__ out, const void* __restrict__ in,
                                                                    int64_t rows, int64_t K, int64_t in_stride,
-                                                                   int64_t out_stride, int in_dtype, float recip) {
+                                                                   int64_t out_stride, int in_dtype, float recip,
+                                                                   const void* scale_ptr, int scales_dtype) {
+  if (scale_ptr) recip = guarded_recip(load_elem(scale_ptr, scales_dtype, 0));
   const int64_t total = rows * K;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t r = i / K, c = i - r * K;
     out[r * out_stride + c] = encode_one(clamp448(load_elem(in, in_dtype, r * in_stride + c) * recip));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Dynamic per-tensor quantisation (max/kernels/src/linalg/fp8_quantization.mojo:209-360, 596-775):
+// one scale for the whole tensor, written to every scales[0, row].  Three launches, no scratch
+// memory: row amax -> scales[row] (as the scales dtype, like the reference's first kernel), one
+// block turns them into the tensor's scale in place, then the static-scale kernel quantises with
+// the scale it reads from scales[0].  (The reference's second kernel reads and overwrites the
+// per-row values in one launch, so what its later blocks see depends on block order; here every
+// row gets the scale of the true tensor maximum.)
+__global__ __launch_bounds__(256) void row_amax_kernel(void* __restrict__ scales, const void* __restrict__ in, int64_t K,
+                                                       int64_t in_stride, int in_dtype, int scales_dtype, int vec_bf16) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const int tid = threadIdx.x;
+  float amax = 0.0f;
+  if (vec_bf16) {
+    const uint4* src = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(in) + row * in_stride);
+    for (int64_t i = tid; i < (K >> 3); i += 256) {
+      const uint4 v = src[i];
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        amax = fmaxf(amax, fabsf(__uint_as_float(w[j] << 16)));
+        amax = fmaxf(amax, fabsf(__uint_as_float(w[j] & 0xffff0000u)));
+      }
+    }
+  } else {
+    for (int64_t i = tid; i < K; i += 256) amax = fmaxf(amax, fabsf(load_elem(in, in_dtype, row * in_stride + i)));
+  }
+  amax = wave_max(amax);
+  if ((tid & 63) == 0) red[tid >> 6] = amax;
+  __syncthreads();
+  if (tid == 0) {
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    if (scales_dtype == MAXFP8_BF16) reinterpret_cast<uint16_t*>(scales)[row] = (uint16_t)f32_to_bf16_bits(amax);
+    else reinterpret_cast<float*>(scales)[row] = amax;
+  }
+}
+
+__global__ __launch_bounds__(1024) void tensor_scale_kernel(void* __restrict__ scales, int64_t rows, int scales_dtype,
+                                                            float scale_ub) {
+  __shared__ float red[16];
+  const int tid = threadIdx.x;
+  float amax = 0.0f;
+  for (int64_t r = tid; r < rows; r += 1024) amax = fmaxf(amax, load_elem(scales, scales_dtype, r));
+  amax = wave_max(amax);
+  if ((tid & 63) == 0) red[tid >> 6] = amax;
+  __syncthreads();
+  amax = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) amax = fmaxf(amax, red[w]);
+  if (scales_dtype == MAXFP8_BF16) {
+    const float ub = bf16_bits_to_f32(f32_to_bf16_bits(scale_ub));
+    const uint16_t sb = (uint16_t)f32_to_bf16_bits(fminf(amax, ub) / 448.0f);
+    for (int64_t r = tid; r < rows; r += 1024) reinterpret_cast<uint16_t*>(scales)[r] = sb;
+  } else {
+    const float scale = fminf(amax, scale_ub) / 448.0f;
+    for (int64_t r = tid; r < rows; r += 1024) reinterpret_cast<float*>(scales)[r] = scale;
   }
 }
 
@@ -448,8 +522,10 @@ int rmsnorm_quantize_dispatch(void* out_fp8, void* out_scales, const void* in, c
   return launch_status("rmsnorm_quant_generic");
 }
 
-int quantize_static_dispatch(void* out_fp8, const void* in, int64_t rows, int64_t K, int64_t in_row_stride,
-                             int64_t out_row_stride, int in_dtype, float scale, hipStream_t stream) {
+// scale_ptr == nullptr: quantise with the host value `scale`; otherwise with element 0 of scale_ptr
+static int quantize_by_scale(void* out_fp8, const void* in, int64_t rows, int64_t K, int64_t in_row_stride,
+                             int64_t out_row_stride, int in_dtype, float scale, const void* scale_ptr, int scales_dtype,
+                             hipStream_t stream) {
   const float recip = 1.0f / scale;
   const bool fast = in_dtype == MAXFP8_BF16 && aligned16(in) && (in_row_stride % 8 == 0) && (K % 8 == 0) &&
                     (reinterpret_cast<uintptr_t>(out_fp8) % 8 == 0) && (out_row_stride % 8 == 0);
@@ -457,11 +533,25 @@ int quantize_static_dispatch(void* out_fp8, const void* in, int64_t rows, int64_
   const unsigned blocks = (unsigned)(ceil_div(items, 256) < 16384 ? ceil_div(items, 256) : 16384);
   if (fast)
     hipLaunchKernelGGL(quant_static_bf16_kernel, dim3(blocks), dim3(256), 0, stream, (uint8_t*)out_fp8, (const uint16_t*)in,
-                       rows, (int)(K / 8), in_row_stride, out_row_stride, recip);
+                       rows, (int)(K / 8), in_row_stride, out_row_stride, recip, scale_ptr, scales_dtype);
   else
     hipLaunchKernelGGL(quant_static_generic_kernel, dim3(blocks), dim3(256), 0, stream, (uint8_t*)out_fp8, in, rows, K,
-                       in_row_stride, out_row_stride, in_dtype, recip);
+                       in_row_stride, out_row_stride, in_dtype, recip, scale_ptr, scales_dtype);
   return launch_status("quantize_static");
+}
+
+int quantize_static_dispatch(void* out_fp8, const void* in, int64_t rows, int64_t K, int64_t in_row_stride,
+                             int64_t out_row_stride, int in_dtype, float scale, hipStream_t stream) {
+  return quantize_by_scale(out_fp8, in, rows, K, in_row_stride, out_row_stride, in_dtype, scale, nullptr, MAXFP8_F32, stream);
+}
+
+int quantize_tensor_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t rows, int64_t K, int64_t in_row_stride,
+                             int64_t out_row_stride, int in_dtype, int scales_dtype, float scale_ub, hipStream_t stream) {
+  const int vec = in_dtype == MAXFP8_BF16 && aligned16(in) && (in_row_stride % 8 == 0) && (K % 8 == 0);
+  hipLaunchKernelGGL(row_amax_kernel, dim3((unsigned)rows), dim3(256), 0, stream, out_scales, in, K, in_row_stride, in_dtype,
+                     scales_dtype, vec);
+  hipLaunchKernelGGL(tensor_scale_kernel, dim3(1), dim3(1024), 0, stream, out_scales, rows, scales_dtype, scale_ub);
+  return quantize_by_scale(out_fp8, in, rows, K, in_row_stride, out_row_stride, in_dtype, 1.0f, out_scales, scales_dtype, stream);
 }
 
 int cast_f32_to_e4m3fn_dispatch(void* out, const float* in, int64_t n, hipStream_t stream) {

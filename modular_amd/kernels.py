@@ -98,6 +98,44 @@ def quantize_dynamic_scaled_float8(
     return out, scales
 
 
+def quantize_tensor_dynamic_scaled_float8(
+    input: torch.Tensor,
+    input_scale_spec: InputScaleSpec,
+    weight_scale_spec: WeightScaleSpec,
+    scale_ub: float = 1200.0,
+    group_size_or_per_token: int = -1,
+    out_type: torch.dtype = _FP8,
+    scales_type: torch.dtype = torch.bfloat16,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantize `input` [M, K] to fp8 with one dynamic scale for the whole tensor
+    (max/python/max/nn/kernels.py:6804-6873).  Returns (quantized [M, K], scales [1, M]);
+    every element of scales holds the tensor's scale."""
+    if input.dim() != 2:
+        raise ValueError("input must be rank 2 tensor")
+    if out_type != _FP8:
+        raise ValueError("out_type must be float8_e4m3fn")
+    if not (input_scale_spec.is_tensor and weight_scale_spec.is_tensor):
+        raise ValueError("both input and weight must be tensor scaled for tensor scaling")
+    if group_size_or_per_token != -1:
+        raise ValueError("group_size_or_per_token should be -1 for dynamic tensor scaling so "
+                         "group_size == num_cols == input.shape[1]")
+    if scales_type not in (torch.float32, torch.bfloat16):
+        raise TypeError("scales dtype should be bfloat16 or float32")
+    if input.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError(f"input dtype {input.dtype} is not bfloat16, float16 or float32")
+    _require_gpu(input)
+    if input.stride(1) != 1:
+        input = input.contiguous()
+    M, K = input.shape
+    out = torch.empty((M, K), dtype=_FP8, device=input.device)
+    scales = torch.empty((1, M), dtype=scales_type, device=input.device)
+    st = _lib.lib().maxfp8_quantize_tensor_dynamic_scaled_fp8(
+        out.data_ptr(), scales.data_ptr(), input.data_ptr(), M, K, input.stride(0) if M > 1 else K, K,
+        _DT[input.dtype], _DT[scales_type], float(scale_ub), _stream(input))
+    _lib.check(st)
+    return out, scales
+
+
 def _host_scalar(t: torch.Tensor, what: str) -> float:
     if tuple(t.shape) not in ((), (1,)):
         raise ValueError(f"expected {what} to be a scalar, but got shape of {list(t.shape)}")

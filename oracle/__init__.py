@@ -165,6 +165,17 @@ def quantize_static(x: np.ndarray, scale: float, *, in_dtype: int = BF16) -> np.
     return q
 
 
+def quantize_tensor_dynamic(x: np.ndarray, *, in_dtype: int = BF16, scales_dtype: int = F32, scale_ub: float = 1200.0,
+                            threads: int = 1):
+    """Per-tensor dynamic quantisation (fp8_quantization.mojo:209-360, 596-775): the whole [M, K] tensor is
+    one group of quantize_dynamic_scaled_fp8.  Returns (q uint8 [M, K], scales [1, M], all equal)."""
+    x = np.ascontiguousarray(x)
+    M, K = x.shape
+    q, sc = quantize_dynamic_scaled_fp8(x.reshape(1, M * K), M * K, in_dtype=in_dtype, scales_dtype=scales_dtype,
+                                        scale_ub=scale_ub, threads=threads)
+    return q.reshape(M, K), np.repeat(sc[:1, :1], M, axis=1)
+
+
 def moe_create_indices(topk_ids: np.ndarray, num_experts: int):
     """topk_ids: int32 [n].  Returns (token_expert_order, expert_start_indices, restore_token_order,
     expert_ids, expert_usage_stats) in the canonical order (slot z = expert z, stable)."""

@@ -25,6 +25,10 @@
  *                            max/kernels/test/gpu/nn/test_rms_norm_fused_fp8.mojo:60-126
  *   orc_moe_create_indices   max/kernels/src/nn/moe.mojo:435-590 (canonical slot order)
  *   orc_fused_silu           max/kernels/src/shmem/ep_comm.mojo:4409-4500, 4505-4624
+ * Composed in oracle/__init__.py from the functions above, nothing new to pin: the batched
+ * quantiser and matmul (one 2-D call per batch, fp8_quantization.mojo:779-954, bmm.mojo:1430-1558)
+ * and the dynamic per-tensor quantiser (the whole tensor as one group,
+ * fp8_quantization.mojo:209-360; checked against the formula of the reference's own test).
  *
  * Pinned by tests/test_oracle_*.py: exhaustive decode against the closed form and
  * the committed 256-entry table; encode over every bf16 value and 2^22 sampled
