@@ -7,6 +7,7 @@
  *   mo.matmul_dynamic_scaled_fp8           -> maxfp8_matmul_dynamic_scaled_fp8
  *   mo.grouped.matmul.dynamic.scaled.fp8   -> maxfp8_grouped_matmul_dynamic_scaled_fp8
  *   mo.batched.matmul.dynamic.scaled.fp8   -> maxfp8_batched_matmul_dynamic_scaled_fp8
+ *   mo.fused_qkv_matmul.ragged.paged.scale -> maxfp8_fused_qkv_matmul_ragged_paged_scale
  *
  * Conventions (the same as the reference's destination-passing custom-op ABI,
  * max/kernels/src/graph_compiler/extensibility/decorators.mojo:46-131):
@@ -188,6 +189,50 @@ int maxfp8_batched_matmul_dynamic_scaled_fp8(
 
 /* Bytes of workspace that lets AUTO use every kernel for this shape. */
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Fused QKV projection with the K / V columns stored straight into a paged KV cache.
+ * Replaces Struct_fused_qkv_matmul_ragged_paged_scale (".bias" with a non-null bias)
+ *   (max/kernels/src/graph_compiler/builtin_kernels/attention.mojo:1043-1107)
+ * -> _fused_qkv_matmul_kv_cache_ragged_impl_scale (max/kernels/src/nn/kv_cache_ragged.mojo:1122-1307)
+ * and, with q_dim = 0 and N = kv_heads * head_dim, mo.k_matmul.ragged.paged.scale
+ *   (k_matmul_ragged_paged_scale, kv_cache_ragged.mojo:3025-3224).
+ *
+ *   input       [T, K] e4m3fn, contiguous; row t is token t of the ragged batch
+ *   wqkv        [N, K] e4m3fn, contiguous; N = q_dim + k_dim (K only, also the MLA layout)
+ *               or q_dim + 2 * k_dim (K then V), k_dim = num_kv_heads * head_dim
+ *   output      [T, q_dim] bf16, receives columns [0, q_dim) (may be NULL when q_dim == 0)
+ *   kv_blocks   [num_blocks, kv_dim, num_layers, page_size, num_kv_heads, head_dim] bf16,
+ *               kv_dim = 2 (K, V) or 1 (MLA); column q_dim + h * head_dim + d of row t goes to
+ *               kv_blocks[lookup_table[b, p / page_size], 0 (K) or 1 (V), layer_idx,
+ *                         p % page_size, h, d]
+ *               with b the sequence that owns row t (input_row_offsets[b] <= t <
+ *               input_row_offsets[b + 1]) and p = t - input_row_offsets[b] + cache_lengths[b]
+ *               (max/kernels/src/kv_cache/types.mojo:2274-2296).  A row whose page index is
+ *               outside the lookup table, or whose block index is >= num_blocks, stores nothing.
+ *   input_row_offsets [batch_size + 1], cache_lengths [batch_size], lookup_table [batch_size, lut_ld]: u32
+ *   bias        [N] bf16 or NULL
+ *   (gm, gn, gk)  the op's scales_granularity_mnk: (-1, -1, -1) per tensor (input_scale[0],
+ *               weight_scale[0]); (1, 1, -1) per token / per channel (input_scale [1, T],
+ *               weight_scale [N, 1] with element stride weight_scale_ld); otherwise block
+ *               scaling, of which (1, 128, 128) is built: input_scale [K/128, input_scale_ld],
+ *               weight_scale [N/128, weight_scale_ld].  scales_dtype must be MAXFP8_F32.
+ * Values take the reference's roundings: the f32 accumulator (block: with its scales applied) is
+ * rounded to bf16; per tensor / per channel that value is multiplied in bf16 by
+ * bf16(bf16(input_scale) * bf16(weight_scale)); the bias is added in bf16.
+ * The MFMA kernels need K % 16 == 0, 16-byte aligned buffers and q_dim, k_dim multiples of 8.
+ */
+int maxfp8_fused_qkv_matmul_ragged_paged_scale(
+    void* output, const void* input, const uint32_t* input_row_offsets,
+    const void* wqkv, const void* input_scale, const void* weight_scale,
+    void* kv_blocks, const uint32_t* cache_lengths, const uint32_t* lookup_table,
+    const void* bias,
+    int64_t T, int64_t N, int64_t K, int64_t q_dim, int64_t batch_size,
+    int64_t num_blocks, int64_t kv_dim, int64_t num_layers, int64_t layer_idx,
+    int64_t page_size, int64_t num_kv_heads, int64_t head_dim, int64_t lut_ld,
+    int64_t gm, int64_t gn, int64_t gk,
+    int64_t input_scale_ld, int64_t weight_scale_ld,
+    int scales_dtype, int algo, void* stream);
 
 /*
  * Grouped (MoE) blockwise-scaled FP8 matmul over token rows sorted by expert.

@@ -6,7 +6,9 @@ through the C ABI of include/maxfp8.h; there is no CPU or PyTorch fallback.
 """
 from .quant_config import (InputScaleSpec, QuantConfig, QuantFormat, ScaleGranularity, ScaleOrigin,
                            WeightScaleSpec, blockwise_fp8_config, rowwise_fp8_config)
-from .kernels import (batched_dynamic_scaled_fp8_matmul, batched_quantize_dynamic_scaled_fp8, dynamic_scaled_matmul,
+from .kv_cache import KVCacheParams, PagedCacheValues
+from .kernels import (fused_qkv_ragged_matmul_scaled_float8, matmul_k_cache_ragged_scaled_float8,
+                      batched_dynamic_scaled_fp8_matmul, batched_quantize_dynamic_scaled_fp8, dynamic_scaled_matmul,
                       grouped_dynamic_scaled_fp8_matmul, matmul_static_scaled_float8,
                       quantize_static_scaled_float8, quantize_tensor_dynamic_scaled_float8,
                       quantize_dynamic_scaled_float8, rms_norm_fused_quantize_dynamic_scaled_fp8)
@@ -23,5 +25,6 @@ __all__ = [
     "moe_create_indices", "fused_silu", "fused_silu_quantized",
     "quantize_static_scaled_float8", "matmul_static_scaled_float8", "parse_quant_config",
     "batched_dynamic_scaled_fp8_matmul", "batched_quantize_dynamic_scaled_fp8",
-    "quantize_tensor_dynamic_scaled_float8",
+    "quantize_tensor_dynamic_scaled_float8", "fused_qkv_ragged_matmul_scaled_float8",
+    "matmul_k_cache_ragged_scaled_float8", "KVCacheParams", "PagedCacheValues",
 ]

@@ -30,6 +30,7 @@ EXPORTS = (
     "maxfp8_batched_matmul_dynamic_scaled_fp8",
     "maxfp8_matmul_workspace_bytes",
     "maxfp8_grouped_matmul_dynamic_scaled_fp8",
+    "maxfp8_fused_qkv_matmul_ragged_paged_scale",
     "maxfp8_quantize_static_scaled_fp8",
     "maxfp8_quantize_tensor_dynamic_scaled_fp8",
     "maxfp8_moe_create_indices",
@@ -76,6 +77,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_matmul_workspace_bytes.argtypes = [i64, i64, i64]
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8.restype = ci
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8.argtypes = [vp] * 7 + [i64] * 7 + [ci, ci, ci, vp]
+    L.maxfp8_fused_qkv_matmul_ragged_paged_scale.restype = ci
+    L.maxfp8_fused_qkv_matmul_ragged_paged_scale.argtypes = [vp] * 10 + [i64] * 18 + [ci, ci, vp]
     L.maxfp8_quantize_static_scaled_fp8.restype = ci
     L.maxfp8_quantize_static_scaled_fp8.argtypes = [vp, vp, i64, i64, i64, i64, ci, cf, vp]
     L.maxfp8_quantize_tensor_dynamic_scaled_fp8.restype = ci

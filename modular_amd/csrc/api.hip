@@ -322,6 +322,85 @@ int maxfp8_batched_matmul_dynamic_scaled_fp8(void* c, const void* a, const void*
                        a_scales_ld, b_scales_ld, c_dtype, scales_dtype, algo, nullptr, 0, bt, stream);
 }
 
+int maxfp8_fused_qkv_matmul_ragged_paged_scale(void* output, const void* input, const uint32_t* input_row_offsets,
+                                               const void* wqkv, const void* input_scale, const void* weight_scale,
+                                               void* kv_blocks, const uint32_t* cache_lengths, const uint32_t* lookup_table,
+                                               const void* bias, int64_t T, int64_t N, int64_t K, int64_t q_dim,
+                                               int64_t batch_size, int64_t num_blocks, int64_t kv_dim, int64_t num_layers,
+                                               int64_t layer_idx, int64_t page_size, int64_t num_kv_heads, int64_t head_dim,
+                                               int64_t lut_ld, int64_t gm, int64_t gn, int64_t gk, int64_t input_scale_ld,
+                                               int64_t weight_scale_ld, int scales_dtype, int algo, void* stream) {
+  if (T < 0 || N < 0 || K < 0 || q_dim < 0 || batch_size < 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused qkv matmul: negative size");
+  if (batch_size == 0 || T == 0 || N == 0) return MAXFP8_OK;  // kv_cache_ragged.mojo:1193-1194
+  if (T >= ((int64_t)1 << 31) || N >= ((int64_t)1 << 31) || K >= ((int64_t)1 << 31) || batch_size >= ((int64_t)1 << 31))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused qkv matmul: sizes must fit 31 bits");
+  if (kv_dim != 1 && kv_dim != 2) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused qkv matmul: the cache holds 2 (K, V) or 1 (MLA) planes, got %lld", (long long)kv_dim);
+  if (num_blocks <= 0 || num_layers <= 0 || layer_idx < 0 || layer_idx >= num_layers || page_size <= 0 || num_kv_heads <= 0 ||
+      head_dim <= 0 || lut_ld <= 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused qkv matmul: bad cache geometry");
+  const int64_t k_dim = num_kv_heads * head_dim;
+  const int64_t rest = N - q_dim;
+  if (rest != k_dim && !(rest == 2 * k_dim && kv_dim == 2))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused qkv matmul: N = %lld is not q_dim %lld plus one or two times kv_heads * head_dim = %lld",
+                (long long)N, (long long)q_dim, (long long)k_dim);
+  if (!input || !wqkv || !input_scale || !weight_scale || !kv_blocks || !cache_lengths || !lookup_table || !input_row_offsets ||
+      (q_dim > 0 && !output))
+    MAXFP8_FAIL(MAXFP8_ERR_NULL, "fused qkv matmul: null pointer");
+  if (scales_dtype != MAXFP8_F32) MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "fused qkv matmul: scales must be float32");
+  const bool per_tensor = gm == -1 && gn == -1 && gk == -1;
+  const bool per_channel = gm == 1 && gn == 1 && gk == -1;
+  const bool block = !per_tensor && !per_channel;
+  if (block && !(gm == 1 && gn == 128 && gk == 128))
+    MAXFP8_FAIL(MAXFP8_ERR_GRANULARITY, "fused qkv matmul: block scaling needs the (1, 128, 128) granularity");
+  if (block && (input_scale_ld < T || weight_scale_ld < ceil_div(K, 128)))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused qkv matmul: scale leading dimensions too small");
+  // the MFMA kernels' layout, and 8-element chunks that stay inside one of Q / K / V and one cache row
+  if (!is_aligned(input, 16) || !is_aligned(wqkv, 16) || K % 16 != 0 || K <= 0)
+    MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "fused qkv matmul: needs 16-byte aligned rows and K %% 16 == 0");
+  if (q_dim % 8 != 0 || k_dim % 8 != 0 || !is_aligned(kv_blocks, 16) || (q_dim > 0 && !is_aligned(output, 16)))
+    MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "fused qkv matmul: q_dim and kv_heads * head_dim must be multiples of 8, buffers 16-byte aligned");
+
+  GemmArgs p;
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t*)input;
+  p.b = (const uint8_t*)wqkv;
+  p.c = output;
+  p.a_scales = (const float*)input_scale;
+  p.b_scales = (const float*)weight_scale;
+  p.M = (int)T; p.N = (int)N; p.K = (int)K;
+  p.lda = K; p.ldb = K; p.ldc = q_dim;
+  p.a_scales_ld = input_scale_ld;
+  p.b_scales_ld = weight_scale_ld;
+  p.a_scale_stride = per_tensor ? 0 : 1;
+  p.b_scale_stride = per_tensor ? 0 : weight_scale_ld;
+  p.c_dtype = MAXFP8_BF16;
+  p.c_vec_ok = 1;
+  p.c_vec8_ok = 1;
+  p.kv_on = 1;
+  const int64_t plane = page_size * k_dim;  // one (block, K|V, layer) plane
+  uint16_t* blocks = (uint16_t*)kv_blocks;
+  p.kv.k_base = blocks + layer_idx * plane;
+  p.kv.v_base = kv_dim == 2 ? blocks + (num_layers + layer_idx) * plane : nullptr;
+  p.kv.lookup_table = lookup_table;
+  p.kv.cache_lengths = cache_lengths;
+  p.kv.row_offsets = input_row_offsets;
+  p.kv.bias = (const uint16_t*)bias;
+  p.kv.block_stride = kv_dim * num_layers * plane;
+  p.kv.lut_ld = lut_ld;
+  p.kv.num_blocks = num_blocks;
+  p.kv.q_dim = (int)q_dim;
+  p.kv.k_dim = (int)k_dim;
+  p.kv.row_elems = (int)k_dim;
+  p.kv.page_size = (int)page_size;
+  p.kv.batch = (int)batch_size;
+  p.kv.bf16_scaling = block ? 0 : 1;
+  hipStream_t st = (hipStream_t)stream;
+  if (algo == MAXFP8_ALGO_AUTO) algo = T <= gemm_skinny_max_m() ? MAXFP8_ALGO_SKINNY : MAXFP8_ALGO_TILED;
+  if (algo == MAXFP8_ALGO_SKINNY) return gemm_skinny_dispatch(p, block, 1, st);
+  if (algo != MAXFP8_ALGO_TILED) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused qkv matmul: algo %d is not available", algo);
+  return gemm_tiled_dispatch(p, block, 0, 1, st);
+}
+
 int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
                                              const void* b_scales, const uint32_t* expert_start_indices,
                                              const int32_t* expert_ids, int64_t T, int64_t N, int64_t K,

@@ -41,6 +41,8 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return u >> 16;
 }
+// f rounded to bf16 (nearest even) and widened back
+__device__ __forceinline__ float bf16_round(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
 __device__ __forceinline__ float clamp448(float v) {
   // fminf/fmaxf return the non-NaN operand; inputs are never NaN on this path.

@@ -4,6 +4,27 @@
 
 namespace maxfp8 {
 
+// Where a fused QKV matmul puts its columns (max/kernels/src/nn/kv_cache_ragged.mojo:1122-1307):
+// columns [0, q_dim) go to C, [q_dim, q_dim + k_dim) to the K pages and the rest to the V pages
+// of a paged cache [num_blocks, 2, num_layers, page_size, kv_heads, head_dim] (bf16).  Row m is
+// token (m - row_offsets[b]) + cache_lengths[b] of sequence b, which lives in page
+// lookup_table[b, token / page_size] at slot token % page_size (max/kernels/src/kv_cache/types.mojo:2274-2296).
+struct KvStore {
+  uint16_t* k_base;               // element (block 0, K, layer, 0, 0, 0)
+  uint16_t* v_base;               // element (block 0, V, layer, 0, 0, 0)
+  const uint32_t* lookup_table;   // [batch, lut_ld]
+  const uint32_t* cache_lengths;  // [batch]
+  const uint32_t* row_offsets;    // [batch + 1]
+  const uint16_t* bias;           // [N] bf16 or null
+  int64_t block_stride;           // elements between consecutive blocks
+  int64_t lut_ld;
+  int64_t num_blocks;
+  int q_dim, k_dim;
+  int row_elems;                  // kv_heads * head_dim
+  int page_size, batch;
+  int bf16_scaling;               // per-tensor / per-channel flavour: scales are applied in bf16
+};
+
 struct GemmArgs {
   const uint8_t* a;        // [M, K] e4m3fn, row stride lda bytes
   const uint8_t* b;        // [N, K] e4m3fn (per expert when grouped), row stride ldb bytes
@@ -30,9 +51,36 @@ struct GemmArgs {
   // split-K / skinny only
   float* workspace;
   int splits;
+  // fused QKV only
+  int kv_on;
+  KvStore kv;
 };
 
 #if defined(__HIPCC__)
+// offset (elements from k_base / v_base) of the cache row that receives row m; -1 when the
+// lookup table has no page for it (nothing is stored then)
+__device__ __forceinline__ int64_t kv_row_offset(const KvStore& kv, int64_t m) {
+  int low = 0, high = kv.batch;
+  while (low + 1 < high) {  // the last sequence whose first row is <= m
+    const int mid = (low + high) >> 1;
+    if (m >= (int64_t)kv.row_offsets[mid]) low = mid;
+    else high = mid;
+  }
+  const uint32_t token = (uint32_t)(m - kv.row_offsets[low]) + kv.cache_lengths[low];
+  const uint32_t page = token / (uint32_t)kv.page_size, slot = token - page * (uint32_t)kv.page_size;
+  if ((int64_t)page >= kv.lut_ld) return -1;
+  const uint32_t block = kv.lookup_table[(int64_t)low * kv.lut_ld + page];
+  if ((int64_t)block >= kv.num_blocks) return -1;
+  return (int64_t)block * kv.block_stride + (int64_t)slot * kv.row_elems;
+}
+
+// destination of column n (and the columns after it up to the next multiple of 8) of row m
+__device__ __forceinline__ uint16_t* kv_dst(const KvStore& kv, void* c, int64_t ldc, int64_t m, int64_t row_off, int n) {
+  if (n < kv.q_dim) return reinterpret_cast<uint16_t*>(c) + m * ldc + n;
+  if (n < kv.q_dim + kv.k_dim) return kv.k_base + row_off + (n - kv.q_dim);
+  return kv.v_base + row_off + (n - kv.q_dim - kv.k_dim);
+}
+
 // the arguments of batch `b` of a batched matmul
 __device__ __forceinline__ GemmArgs batch_view(const GemmArgs& p, int64_t b) {
   GemmArgs q = p;

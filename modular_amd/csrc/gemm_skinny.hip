@@ -226,6 +226,35 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
       v[i] = sum;
     }
     if (m >= p.M || n >= p.N) continue;
+    if (p.kv_on) {
+      // fused QKV: the reference's bf16 roundings, then C or the row's K / V page (see tile_body)
+      const int64_t row_off = kv_row_offset(p.kv, m);
+      float a_s = 1.f;
+      if constexpr (!BLOCKSCALE) a_s = p.a_scales[(int64_t)m * p.a_scale_stride];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int nn = (n + i < p.N) ? n + i : p.N - 1;
+        float r = bf16_round(v[i]);
+        if constexpr (!BLOCKSCALE) {
+          const float sc = bf16_round(bf16_round(a_s) * bf16_round(p.b_scales[(int64_t)nn * p.b_scale_stride]));
+          r = bf16_round(r * sc);
+        }
+        if (p.kv.bias) r = bf16_round(r + bf16_bits_to_f32(p.kv.bias[nn]));
+        v[i] = r;
+      }
+      if (row_off < 0 && n >= p.kv.q_dim) continue;
+      uint16_t* dst = kv_dst(p.kv, p.c, p.ldc, m, row_off, n);
+      if (p.c_vec_ok && n + 3 < p.N) {
+        const uint32_t lo = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+        const uint32_t hi = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < p.N) dst[i] = (uint16_t)f32_to_bf16_bits(v[i]);
+      }
+      continue;
+    }
     if constexpr (!BLOCKSCALE) {
       const float a_s = p.a_scales[(int64_t)m * p.a_scale_stride];
 #pragma unroll

@@ -35,12 +35,23 @@
 // caps the wave tile at 128 x 64 with two waves per SIMD.
 #include <stdlib.h>
 
+#include <utility>
 #include "common.h"
 #include "gemm_args.h"
 
 namespace maxfp8 {
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// f(integral_constant<int, 0>{}) ... f(integral_constant<int, N - 1>{}): a loop whose index is a constant
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t t2_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
@@ -52,7 +63,7 @@ __device__ __forceinline__ uint32_t t2_clamp_u32(int64_t v) {
 // One BM x BN tile of C: rows [row_begin, row_end) (at most BM of them are used) by columns
 // [n0, n0 + BN) of the weight matrix at bptr / scales at bs_ptr.  Called by every thread of a
 // block of WAVES_M * WAVES_N waves with `smem` = the block's dynamic LDS.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED, bool KV = false>
 __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, const int64_t row_begin, const int64_t row_end,
                                           const int n0, const uint8_t* bptr, const float* bs_ptr) {
   constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -325,6 +336,65 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     }
     return;
   }
+  if constexpr (KV) {
+    // Fused QKV: bf16 only.  The value takes the reference's roundings -- the accumulator is
+    // rounded to bf16 first, per-tensor / per-channel scales are multiplied in bf16, the bias is
+    // added in bf16 (kv_cache_ragged.mojo:1210-1245) -- and goes to C or to the row's K / V page.
+    // Columns outside, rows inside: 8 weight scales and 8 bias values live at a time.
+    float a_s[TM];
+    int64_t row_off[TM];
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) {
+      int ml = wm * WM + mt * 16 + lm;
+      asm volatile("" : "+v"(ml));  // keeps the page lookups here, out of the registers of the main loop
+      a_s[mt] = 1.f;
+      row_off[mt] = -1;
+      if (ml < rows_here) {
+        if constexpr (!BLOCKSCALE) a_s[mt] = bf16_round(p.a_scales[(row_begin + ml) * p.a_scale_stride]);
+        row_off[mt] = kv_row_offset(p.kv, row_begin + ml);
+      }
+    }
+    static_for<TN / 2>([&](auto qc) {  // (a plain unrolled loop leaves acc indexed at run time here)
+      constexpr int q = decltype(qc)::value;
+      const int n = n0 + wn * WN + q * 32 + lq * 8;
+      if (n >= p.N) return;
+      float b_s[8], bias[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int nn = (n + i < p.N) ? n + i : p.N - 1;
+        b_s[i] = 1.f;
+        if constexpr (!BLOCKSCALE) b_s[i] = bf16_round(p.b_scales[(int64_t)nn * p.b_scale_stride]);
+        bias[i] = p.kv.bias ? bf16_bits_to_f32(p.kv.bias[nn]) : 0.f;
+      }
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        const int ml = wm * WM + mt * 16 + lm;
+        if (ml >= rows_here) continue;
+        if (row_off[mt] < 0 && n >= p.kv.q_dim) continue;
+        const v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
+        float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float r = bf16_round(v[i]);
+          if constexpr (!BLOCKSCALE) r = bf16_round(r * bf16_round(a_s[mt] * b_s[i]));
+          if (p.kv.bias) r = bf16_round(r + bias[i]);
+          v[i] = r;
+        }
+        uint16_t* dst = kv_dst(p.kv, p.c, p.ldc, row_begin + ml, row_off[mt], n);
+        if (p.c_vec8_ok && n + 7 < p.N) {
+          uint32_t w[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+          *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (n + i < p.N) dst[i] = (uint16_t)f32_to_bf16_bits(v[i]);
+        }
+      }
+    });
+    return;
+  }
 #pragma unroll
   for (int mt = 0; mt < TM; ++mt) {
     const int ml = wm * WM + mt * 16 + lm;
@@ -352,7 +422,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool KV = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   // ---- block -> tile: XCD de-interleave, then groups of GROUP_M row tiles share weight columns
@@ -373,7 +443,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
   const int tm = first_m + in_group % gsize;
   const int tn = in_group / gsize;
   const GemmArgs q = gridDim.z == 1 ? p : batch_view(p, blockIdx.z);
-  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false>(q, smem, (int64_t)tm * BM, q.M, tn * BN, q.b, q.b_scales);
+  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false, KV>(q, smem, (int64_t)tm * BM, q.M, tn * BN, q.b, q.b_scales);
 }
 
 // ---- grouped (MoE) matmul ---------------------------------------------------------------------
@@ -499,10 +569,10 @@ static int launch_with_lds(Kern kern, bool& attr_done, int smem, int threads, co
   return launch_status(name);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool KV = false>
 static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
   static bool attr_done = false;
-  return launch_with_lds(gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE>, attr_done,
+  return launch_with_lds(gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, KV>, attr_done,
                          tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
 
@@ -627,6 +697,7 @@ int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_
   const int nslab = (p.K + 127) / 128;
   int variant = tile_override();
   if (!variant) variant = pick_shape(p.M, p.N, nslab, blockscale, p.workspace != nullptr && batch == 1, batch);
+  if (p.kv_on && variant != 1) variant = 3;  // the fused QKV kernels exist in the 256 x 256 and 128 x 128 shapes
   const TileShape& t = kShapes[variant - 1];
   const int64_t tiles = ceil_div(p.M, t.bm) * ceil_div(p.N, t.bn);
   if (tiles >= ((int64_t)1 << 31)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "tiled matmul: too many tiles");
@@ -646,6 +717,14 @@ int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_
 }
 
 static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, dim3 grid, hipStream_t stream) {
+  if (p.kv_on) {  // fused QKV: the two larger shapes
+    if (blockscale) {
+      if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, true, true>(p, grid, stream, "gemm_qkv_block_256x256");
+      return launch_tiled<128, 128, 2, 2, 2, true, true>(p, grid, stream, "gemm_qkv_block_128x128");
+    }
+    if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false, true>(p, grid, stream, "gemm_qkv_row_256x256");
+    return launch_tiled<128, 128, 2, 2, 2, false, true>(p, grid, stream, "gemm_qkv_row_128x128");
+  }
   if (blockscale) {
     if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, true>(p, grid, stream, "gemm_tiled_block_256x256");
     if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, true>(p, grid, stream, "gemm_tiled_block_256x128");

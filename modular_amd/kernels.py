@@ -5,6 +5,8 @@ of the reference's graph-op wrappers:
   dynamic_scaled_matmul               max/python/max/nn/kernels.py:6960-7078
   grouped_dynamic_scaled_fp8_matmul   max/python/max/nn/kernels.py:6327-6487
   batched_dynamic_scaled_fp8_matmul   max/python/max/nn/kernels.py:6642-6751
+  fused_qkv_ragged_matmul_scaled_float8  max/python/max/nn/kernels.py:582-727
+  matmul_k_cache_ragged_scaled_float8    max/python/max/nn/kernels.py:1475-1539
 
 They take torch tensors that live on the MI355X and call the HIP kernels through
 the C ABI on torch's current stream.  Nothing here computes on the CPU.
@@ -14,7 +16,8 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from .quant_config import InputScaleSpec, ScaleGranularity, ScaleOrigin, WeightScaleSpec
+from .kv_cache import KVCacheParams, PagedCacheValues
+from .quant_config import InputScaleSpec, QuantConfig, ScaleGranularity, ScaleOrigin, WeightScaleSpec
 
 _FP8 = torch.float8_e4m3fn
 _DT = {torch.bfloat16: _lib.BF16, torch.float16: _lib.F16, torch.float32: _lib.F32, _FP8: _lib.E4M3FN}
@@ -452,6 +455,122 @@ def batched_dynamic_scaled_fp8_matmul(
         _ALGOS[algo], _stream(a))
     _lib.check(st)
     return c
+
+
+def _u32(t: torch.Tensor, what: str) -> torch.Tensor:
+    # torch has little support for uint32: int32 tensors with the same bits are accepted
+    if t.dtype not in (torch.uint32, torch.int32):
+        raise TypeError(f"expected {what} to have dtype uint32, but got {t.dtype}")
+    return t.contiguous()
+
+
+def _qkv_cache_matmul(kv_params: KVCacheParams, input: torch.Tensor, input_row_offsets: torch.Tensor,
+                      weight: torch.Tensor, input_scale: torch.Tensor, weight_scale: torch.Tensor,
+                      kv_collection: PagedCacheValues, layer_idx: int, q_dim: int,
+                      scales_granularity_mnk: tuple[int, int, int], bias: torch.Tensor | None,
+                      algo: str) -> torch.Tensor:
+    if input.dtype != weight.dtype:
+        raise ValueError(f"expected input and weight to have the same dtype, but got {input.dtype} and {weight.dtype}")
+    if input.dtype != _FP8:
+        raise TypeError(f"input and weight must be float8_e4m3fn, got {input.dtype}")
+    if input.dim() != 2:
+        raise ValueError(f"expected input to have rank 2, was {input.dim()}")
+    tensors = [weight, input_row_offsets, input_scale, weight_scale] + ([] if bias is None else [bias])
+    if not all(t.device == input.device for t in tensors):
+        raise ValueError(f"expected all tensors to be on the same device as input ({input.device})")
+    _require_gpu(input, kv_collection.kv_blocks, kv_collection.cache_lengths, kv_collection.lookup_table)
+    if kv_params.dtype != torch.bfloat16 or kv_collection.kv_blocks.dtype != torch.bfloat16:
+        raise TypeError("the paged cache must be bfloat16")
+    blocks = kv_collection.kv_blocks
+    if blocks.dim() != 6 or tuple(blocks.shape[1:]) != kv_params.blocks_shape(0)[1:] or not blocks.is_contiguous():
+        raise ValueError(f"kv_blocks must be a contiguous {kv_params.blocks_shape(-1)} tensor, got {tuple(blocks.shape)}")
+    row_offsets = _u32(input_row_offsets, "input_row_offsets")
+    cache_lengths = _u32(kv_collection.cache_lengths, "cache_lengths")
+    lut = _u32(kv_collection.lookup_table, "lookup_table")
+    batch = row_offsets.shape[0] - 1
+    if cache_lengths.shape[0] < batch or lut.dim() != 2 or lut.shape[0] < batch:
+        raise ValueError("cache_lengths / lookup_table hold fewer sequences than input_row_offsets")
+    if input_scale.dtype != torch.float32 or weight_scale.dtype != torch.float32:
+        raise TypeError("input_scale and weight_scale must be float32")
+    T, K = input.shape
+    N = weight.shape[0]
+    if weight.dim() != 2 or weight.shape[1] != K:
+        raise ValueError("weight must be [N, K] with the K of input")
+    input = input.contiguous()
+    weight = weight.contiguous()
+    input_scale = input_scale.contiguous()
+    weight_scale = weight_scale.contiguous()
+    if bias is not None:
+        if bias.dtype != torch.bfloat16 or bias.numel() != N:
+            raise ValueError("bias must be a bfloat16 vector of length N")
+        bias = bias.contiguous()
+    out = torch.empty((T, q_dim), dtype=torch.bfloat16, device=input.device)
+    in_ld = input_scale.shape[1] if input_scale.dim() == 2 else 1
+    w_ld = weight_scale.shape[1] if weight_scale.dim() == 2 else 1
+    st = _lib.lib().maxfp8_fused_qkv_matmul_ragged_paged_scale(
+        out.data_ptr() if q_dim else None, input.data_ptr(), row_offsets.data_ptr(), weight.data_ptr(),
+        input_scale.data_ptr(), weight_scale.data_ptr(), blocks.data_ptr(), cache_lengths.data_ptr(), lut.data_ptr(),
+        bias.data_ptr() if bias is not None else None, T, N, K, q_dim, batch, blocks.shape[0], kv_params.kv_dim,
+        kv_params.num_layers, int(layer_idx), kv_params.page_size, kv_params.n_kv_heads, kv_params.head_dim,
+        lut.shape[1], *scales_granularity_mnk, in_ld, w_ld, _lib.F32, _ALGOS[algo], _stream(input))
+    _lib.check(st)
+    return out
+
+
+def fused_qkv_ragged_matmul_scaled_float8(
+    kv_params: KVCacheParams,
+    input: torch.Tensor,
+    input_row_offsets: torch.Tensor,
+    wqkv: torch.Tensor,
+    kv_collection: PagedCacheValues,
+    layer_idx: int,
+    n_heads: int,
+    input_scale: torch.Tensor,
+    weight_scale: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    quant_config: QuantConfig | None = None,
+    _output_dim: int | None = None,
+    *,
+    algo: str = "auto",
+) -> torch.Tensor:
+    """Fused query, key and value projections of scaled float8 input and weights: returns
+    Q [total_seq_len, n_heads * head_dim] (bf16) and writes K and V into the paged cache
+    in place (max/python/max/nn/kernels.py:582-727)."""
+    if input_scale.dim() < 2 and input_scale.numel() == 1:
+        input_scale = input_scale.reshape(1, 1)
+    if weight_scale.dim() < 2 and weight_scale.numel() == 1:
+        weight_scale = weight_scale.reshape(1, 1)
+    if quant_config is not None:
+        mnk = quant_config.scales_granularity_mnk
+    elif tuple(input_scale.shape) == (1, 1) and tuple(weight_scale.shape) == (1, 1):
+        mnk = (-1, -1, -1)      # per-tensor quantization
+    elif input_scale.shape[0] == 1 and weight_scale.shape[1] == 1:
+        mnk = (1, 1, -1)        # per-channel quantization
+    else:
+        raise ValueError("Can not infer the quantization config from the input tensor shapes",
+                         "Please provide a quant_config")
+    output_dim = _output_dim if _output_dim is not None else n_heads * kv_params.head_dim
+    return _qkv_cache_matmul(kv_params, input, input_row_offsets, wqkv, input_scale, weight_scale, kv_collection,
+                             layer_idx, output_dim, tuple(mnk), bias, algo)
+
+
+def matmul_k_cache_ragged_scaled_float8(
+    kv_params: KVCacheParams,
+    hidden_states: torch.Tensor,
+    input_row_offsets: torch.Tensor,
+    weight: torch.Tensor,
+    input_scale: torch.Tensor,
+    weight_scale: torch.Tensor,
+    kv_collection: PagedCacheValues,
+    scales_granularity_mnk: tuple[int, int, int],
+    layer_idx: int,
+    *,
+    algo: str = "auto",
+) -> None:
+    """Block-scaled float8 matmul whose whole result is written to the key pages of the
+    cache (max/python/max/nn/kernels.py:1475-1539)."""
+    _qkv_cache_matmul(kv_params, hidden_states, input_row_offsets, weight, input_scale, weight_scale, kv_collection,
+                      layer_idx, 0, tuple(scales_granularity_mnk), None, algo)
 
 
 def grouped_dynamic_scaled_fp8_matmul(

@@ -176,6 +176,65 @@ def quantize_tensor_dynamic(x: np.ndarray, *, in_dtype: int = BF16, scales_dtype
     return q.reshape(M, K), np.repeat(sc[:1, :1], M, axis=1)
 
 
+def bf16_round(x: np.ndarray) -> np.ndarray:
+    """float32 array rounded to bf16 (nearest even; NaN kept) and widened back."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = np.where(nan, u | 0x400000, r)
+    return (r & 0xFFFFFFFF).astype(np.uint32).view(np.float32).reshape(np.shape(x))
+
+
+def bf16_bits_of(x: np.ndarray) -> np.ndarray:
+    """float32 array whose values are bf16-representable -> uint16 bit patterns."""
+    return (np.ascontiguousarray(x, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def fused_qkv_matmul(a: np.ndarray, w: np.ndarray, input_scale: np.ndarray, weight_scale: np.ndarray, gmnk,
+                     row_offsets: np.ndarray, cache_lengths: np.ndarray, lookup_table: np.ndarray,
+                     kv_blocks: np.ndarray, layer_idx: int, q_dim: int, *, bias: np.ndarray | None = None,
+                     threads: int = 1) -> np.ndarray:
+    """The fused QKV matmul of kv_cache_ragged.mojo:1122-1307 (and, with q_dim = 0, the K-cache
+    matmul of :3025-3224).  a [T, K], w [N, K] e4m3fn bytes; kv_blocks uint16 (bf16 bits)
+    [blocks, kv_dim, layers, page, heads, head_dim], UPDATED IN PLACE; bias uint16 [N] or None.
+    Returns the Q part, uint16 [T, q_dim].  Rounding steps as in the reference's epilogue: the matmul
+    result arrives as bf16; per tensor (-1,-1,-1) / per channel (1,1,-1) it is multiplied in bf16 by
+    the bf16 product of the two bf16-rounded scales; the bias is added in bf16."""
+    T, K = a.shape
+    N = w.shape[0]
+    gmnk = tuple(gmnk)
+    if gmnk in ((-1, -1, -1), (1, 1, -1)):
+        raw = matmul_rowwise(a, w, np.ones((1, 1), np.float32), np.ones((1, 1), np.float32), tensor_scales=True,
+                             threads=threads)
+        sa = bf16_round(np.asarray(input_scale, dtype=np.float32).reshape(-1))
+        sb = bf16_round(np.asarray(weight_scale, dtype=np.float32).reshape(-1))
+        if gmnk[0] == -1:
+            sc = np.full((T, N), bf16_round(sa[:1] * sb[:1])[0], dtype=np.float32)
+        else:
+            sc = bf16_round(sa[:T, None] * sb[None, :N])
+        val = bf16_round(bf16_round(raw) * sc)
+    else:
+        bits = matmul_blockwise(a, w, input_scale, weight_scale, gmnk=gmnk, c_dtype=BF16, threads=threads)
+        val = (bits.astype(np.uint32) << 16).view(np.float32)
+    if bias is not None:
+        val = bf16_round(val + (np.asarray(bias, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)[None, :])
+    out_bits = bf16_bits_of(val)
+    heads, head_dim = kv_blocks.shape[4], kv_blocks.shape[5]
+    page = kv_blocks.shape[3]
+    k_dim = heads * head_dim
+    has_v = N - q_dim == 2 * k_dim
+    assert N - q_dim == k_dim or (has_v and kv_blocks.shape[1] == 2)
+    ro = np.asarray(row_offsets, dtype=np.int64)
+    for t in range(T):
+        b = int(np.searchsorted(ro, t, side="right")) - 1   # the last sequence whose first row is <= t
+        tok = t - int(ro[b]) + int(cache_lengths[b])
+        blk = int(lookup_table[b, tok // page])
+        kv_blocks[blk, 0, layer_idx, tok % page] = out_bits[t, q_dim:q_dim + k_dim].reshape(heads, head_dim)
+        if has_v:
+            kv_blocks[blk, 1, layer_idx, tok % page] = out_bits[t, q_dim + k_dim:].reshape(heads, head_dim)
+    return np.ascontiguousarray(out_bits[:, :q_dim])
+
+
 def moe_create_indices(topk_ids: np.ndarray, num_experts: int):
     """topk_ids: int32 [n].  Returns (token_expert_order, expert_start_indices, restore_token_order,
     expert_ids, expert_usage_stats) in the canonical order (slot z = expert z, stable)."""
