@@ -6,9 +6,11 @@ from __future__ import annotations
 
 import torch
 
-from .kernels import (dynamic_scaled_matmul, matmul_static_scaled_float8, quantize_dynamic_scaled_float8,
-                      quantize_static_scaled_float8)
-from .quant_config import InputScaleSpec, QuantConfig, ScaleGranularity, WeightScaleSpec
+from .kernels import (dynamic_scaled_matmul, fused_qkv_ragged_matmul_scaled_float8, matmul_static_scaled_float8,
+                      quantize_dynamic_scaled_float8, quantize_static_scaled_float8,
+                      quantize_tensor_dynamic_scaled_float8)
+from .kv_cache import KVCacheParams, PagedCacheValues
+from .quant_config import InputScaleSpec, QuantConfig, QuantFormat, ScaleGranularity, WeightScaleSpec
 
 
 def matmul_float8(
@@ -69,3 +71,44 @@ def quantized_matmul(
     if weight.dtype != torch.float8_e4m3fn:
         raise TypeError(f"weight dtype {weight.dtype} is not float8_e4m3fn")
     return matmul_float8(x, weight, weight_scale, input_scale, quant_config)
+
+
+def quantized_fused_qkv_matmul(
+    kv_params: KVCacheParams,
+    x: torch.Tensor,
+    wqkv: torch.Tensor,
+    kv_collection: PagedCacheValues,
+    layer_idx: int,
+    input_row_offsets: torch.Tensor,
+    n_heads: int,
+    quant_config: QuantConfig,
+    weight_scale: torch.Tensor,
+    input_scale: torch.Tensor | None = None,
+    bias: torch.Tensor | None = None,
+    _output_dim: int | None = None,
+) -> torch.Tensor:
+    """Entry point of the quantised fused QKV projection (quant_ops.py:594-760), FP8 formats:
+    quantise x the way the config says, then one matmul that returns Q and stores K and V in the
+    paged cache.  (Scales in bfloat16 are widened to float32 for the kernel, which is exact.)"""
+    if quant_config.format not in (QuantFormat.COMPRESSED_TENSORS_FP8, QuantFormat.FBGEMM_FP8, QuantFormat.BLOCKSCALED_FP8):
+        raise NotImplementedError(f"{quant_config.format} is not an FP8 format of this package")
+    common = dict(input_row_offsets=input_row_offsets, wqkv=wqkv, kv_collection=kv_collection, layer_idx=layer_idx,
+                  n_heads=n_heads, bias=bias, _output_dim=_output_dim)
+    if quant_config.is_static:
+        assert input_scale is not None
+        xq = quantize_static_scaled_float8(x, input_scale.cpu())
+        x_scales = input_scale
+    elif quant_config.input_scale.is_tensor and quant_config.weight_scale.is_tensor:
+        # dynamic per-tensor input scale against the rowwise [N, 1] scales of the fused weight: the
+        # kernel infers per-channel scaling from the [1, M] / [N, 1] shapes (quant_ops.py:707-738)
+        xq, x_scales = quantize_tensor_dynamic_scaled_float8(x, quant_config.input_scale, quant_config.weight_scale,
+                                                             out_type=wqkv.dtype, scales_type=weight_scale.dtype)
+        return fused_qkv_ragged_matmul_scaled_float8(kv_params, input=xq, input_scale=x_scales.to(x.device).float(),
+                                                     weight_scale=weight_scale.to(x.device).float(), quant_config=None,
+                                                     **common)
+    else:
+        xq, x_scales = quantize_dynamic_scaled_float8(x, quant_config.input_scale, quant_config.weight_scale,
+                                                      scales_type=weight_scale.dtype, out_type=wqkv.dtype)
+    return fused_qkv_ragged_matmul_scaled_float8(kv_params, input=xq, input_scale=x_scales.to(x.device).float(),
+                                                 weight_scale=weight_scale.to(x.device).float(), quant_config=quant_config,
+                                                 **common)

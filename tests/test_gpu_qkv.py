@@ -163,3 +163,64 @@ def test_errors(dev):
     # no sequences: nothing happens
     out = mx.fused_qkv_ragged_matmul_scaled_float8(params, a[:0].to(dev), ro[:1], w.to(dev), coll, 0, 3, sa.to(dev)[:, :0], sb.to(dev))
     assert out.shape == (0, 48)
+
+
+@pytest.mark.parametrize("flavour", ["block", "rowwise", "tensor_dynamic", "static"])
+def test_quantized_fused_qkv_matmul_equals_its_parts(dev, flavour):
+    # the dispatcher = the quantiser of the config + the fused matmul; compared with the unfused linear
+    # (quantized_matmul) whose K / V columns are read back from the cache
+    from modular_amd.quant_config import InputScaleSpec, QuantConfig, QuantFormat, ScaleGranularity, ScaleOrigin, WeightScaleSpec
+    Hq, H, D, K, page = 4, 2, 64, 512, 16
+    prompt, cached = [40, 3, 90], [5, 0, 17]
+    T, q_dim, k_dim = sum(prompt), Hq * D, H * D
+    N = q_dim + 2 * k_dim
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn((T, K), generator=g) * 2).to(torch.bfloat16).to(dev)
+    w = (torch.randn((N, K), generator=g) * 0.05)
+    input_scale = None
+    if flavour == "block":
+        cfg = mx.blockwise_fp8_config()
+        ws = torch.rand((-(-N // 128), K // 128), generator=g) * 0.01 + 0.001
+        wq = (w / ws.repeat_interleave(128, 0)[:N].repeat_interleave(128, 1)).clamp(-448, 448).to(torch.float8_e4m3fn)
+    elif flavour == "rowwise":
+        cfg = mx.rowwise_fp8_config()
+        ws = w.abs().amax(dim=1, keepdim=True) / 448
+        wq = (w / ws).to(torch.float8_e4m3fn)
+    else:
+        origin = ScaleOrigin.STATIC if flavour == "static" else ScaleOrigin.DYNAMIC
+        cfg = QuantConfig(InputScaleSpec(ScaleGranularity.TENSOR, origin, torch.float32),
+                          WeightScaleSpec(ScaleGranularity.TENSOR, torch.float32), format=QuantFormat.COMPRESSED_TENSORS_FP8)
+        if flavour == "static":
+            ws = (w.abs().amax() / 448).reshape(1)
+            wq = (w / ws).to(torch.float8_e4m3fn)
+            input_scale = torch.tensor([0.03])
+        else:
+            ws = w.abs().amax(dim=1, keepdim=True) / 448      # fused QKV weights carry rowwise [N, 1] scales
+            wq = (w / ws).to(torch.float8_e4m3fn)
+    ro, cl, lut = make_cache_case(prompt, cached, page, 16, 1)
+    params = KVCacheParams(torch.bfloat16, H, D, 1, page)
+    blocks = torch.zeros(params.blocks_shape(16), dtype=torch.bfloat16, device=dev)
+    coll = PagedCacheValues(blocks, as_i32(cl).to(dev), as_i32(lut).to(dev))
+    q = mx.quantized_fused_qkv_matmul(params, x, wq.to(dev), coll, 0, as_i32(ro).to(dev), Hq, cfg, ws.to(dev), input_scale=input_scale)
+    if flavour == "tensor_dynamic":
+        # the unfused linear quantises per token there; build the per-tensor reference from the pieces
+        xq, xs = mx.quantize_tensor_dynamic_scaled_float8(x, cfg.input_scale, cfg.weight_scale, scales_type=torch.float32)
+        row = mx.rowwise_fp8_config()
+        full = mx.dynamic_scaled_matmul(xq, wq.to(dev), xs, ws.to(dev), row.input_scale, row.weight_scale)
+    else:
+        full = mx.quantized_matmul(x, wq.to(dev), ws.to(dev) if flavour != "static" else ws, input_scale=input_scale, quant_config=cfg)
+    torch.cuda.synchronize()
+    full_np = full.float().cpu().numpy()
+    # the unfused linear applies f32 scales once; the fused epilogue rounds both scales, their product and the
+    # value to bf16 (the reference's epilogue): five roundings of 2^-9 .. 2^-8 each
+    tol = TOL if flavour == "block" else 2.0 ** -5
+    zero = np.zeros(N)
+    check_vals(bf16_bits(q), bf16_bits(full[:, :q_dim].contiguous()), zero[:q_dim], tol, "Q")
+    got_blocks = bf16_bits(blocks)
+    for b in range(len(prompt)):
+        rows = slice(int(ro[b]), int(ro[b + 1]))
+        for plane in range(2):
+            got = logical_rows(got_blocks, plane, 0, lut, b, cached[b], prompt[b], page)
+            lo = q_dim + plane * k_dim
+            want = bf16_bits(full[rows, lo:lo + k_dim].contiguous())
+            check_vals(got, want, zero[:k_dim], tol, f"sequence {b} plane {plane}")
