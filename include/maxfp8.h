@@ -348,6 +348,12 @@ int maxfp8_fused_silu(
  */
 int maxfp8_cast_f32_to_e4m3fn(void* out_fp8, const float* in, int64_t n, void* stream);
 
+/*
+ * Elementwise f32 -> bf16 (round to nearest even) with the hardware convert the
+ * matmul epilogues use, exposed so it can be checked against the software rounding.
+ */
+int maxfp8_cast_f32_to_bf16(void* out_bf16, const float* in, int64_t n, void* stream);
+
 /* Elementwise e4m3fn -> f32 (mojo/stdlib/std/builtin/simd.mojo:3690-3749). */
 int maxfp8_cast_e4m3fn_to_f32(float* out, const void* in_fp8, int64_t n, void* stream);
 

@@ -37,6 +37,7 @@ EXPORTS = (
     "maxfp8_fused_silu",
     "maxfp8_cast_f32_to_e4m3fn",
     "maxfp8_cast_e4m3fn_to_f32",
+    "maxfp8_cast_f32_to_bf16",
     "maxfp8_copy_bytes",
 )
 
@@ -89,6 +90,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_fused_silu.argtypes = [vp] * 4 + [i64] * 6 + [ci, ci, vp]
     L.maxfp8_cast_f32_to_e4m3fn.restype = ci
     L.maxfp8_cast_f32_to_e4m3fn.argtypes = [vp, vp, i64, vp]
+    L.maxfp8_cast_f32_to_bf16.restype = ci
+    L.maxfp8_cast_f32_to_bf16.argtypes = [vp, vp, i64, vp]
     L.maxfp8_cast_e4m3fn_to_f32.restype = ci
     L.maxfp8_cast_e4m3fn_to_f32.argtypes = [vp, vp, i64, vp]
     L.maxfp8_copy_bytes.restype = ci

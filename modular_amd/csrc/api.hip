@@ -34,6 +34,7 @@ int fused_silu_dispatch(void*, float*, const void*, const uint32_t*, int64_t, in
                         hipStream_t);
 int cast_f32_to_e4m3fn_dispatch(void*, const float*, int64_t, hipStream_t);
 int cast_e4m3fn_to_f32_dispatch(float*, const void*, int64_t, hipStream_t);
+int cast_f32_to_bf16_dispatch(void*, const float*, int64_t, hipStream_t);
 int copy_bytes_dispatch(void*, const void*, int64_t, hipStream_t);
 int naive_blockwise_dispatch(void*, const void*, const void*, const void*, const void*, int64_t, int64_t, int64_t,
                              int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, int64_t, int64_t,
@@ -465,6 +466,12 @@ int maxfp8_cast_e4m3fn_to_f32(float* out, const void* in_fp8, int64_t n, void* s
   if (n <= 0) return MAXFP8_OK;
   if (!out || !in_fp8) MAXFP8_FAIL(MAXFP8_ERR_NULL, "cast: null pointer");
   return cast_e4m3fn_to_f32_dispatch(out, in_fp8, n, (hipStream_t)stream);
+}
+
+int maxfp8_cast_f32_to_bf16(void* out_bf16, const float* in, int64_t n, void* stream) {
+  if (n <= 0) return MAXFP8_OK;
+  if (!out_bf16 || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "cast: null pointer");
+  return cast_f32_to_bf16_dispatch(out_bf16, in, n, (hipStream_t)stream);
 }
 
 int maxfp8_copy_bytes(void* dst, const void* src, int64_t n, void* stream) {

@@ -41,6 +41,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return u >> 16;
 }
+// two f32 -> two bf16 (a in the low half) with the hardware convert of gfx950, v_cvt_pk_bf16_f32:
+// round to nearest even like f32_to_bf16_bits, one instruction instead of a dozen
+typedef float v2f_t __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  const v2f_t f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, v2bf_t));
+}
 // f rounded to bf16 (nearest even) and widened back
 __device__ __forceinline__ float bf16_round(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 

@@ -57,21 +57,55 @@ struct GemmArgs {
 };
 
 #if defined(__HIPCC__)
-// offset (elements from k_base / v_base) of the cache row that receives row m; -1 when the
-// lookup table has no page for it (nothing is stored then)
-__device__ __forceinline__ int64_t kv_row_offset(const KvStore& kv, int64_t m) {
-  int low = 0, high = kv.batch;
-  while (low + 1 < high) {  // the last sequence whose first row is <= m
-    const int mid = (low + high) >> 1;
-    if (m >= (int64_t)kv.row_offsets[mid]) low = mid;
-    else high = mid;
+// offsets (elements from k_base / v_base) of the cache rows that receive rows m[0..R); -1 for a
+// row that is not live or that the lookup table has no page for (nothing is stored then).  The R
+// binary searches run in lockstep with a trip count that only depends on the batch size, so
+// their dependent loads overlap instead of queueing up behind each other.
+template <int R>
+__device__ __forceinline__ void kv_row_offsets(const KvStore& kv, const int64_t (&m)[R], const bool (&live)[R], int64_t (&off)[R]) {
+  int low[R], high[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) { low[r] = 0; high[r] = kv.batch; }
+  const int steps = kv.batch > 1 ? 32 - __builtin_clz((unsigned)(kv.batch - 1)) : 0;
+  for (int s = 0; s < steps; ++s) {
+    uint32_t first[R];
+    int mid[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      mid[r] = (low[r] + high[r]) >> 1;  // == low[r] once the search has narrowed to one sequence
+      first[r] = live[r] ? kv.row_offsets[mid[r]] : 0u;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (m[r] >= (int64_t)first[r]) low[r] = mid[r];  // the last sequence whose first row is <= m
+      else high[r] = mid[r];
+    }
   }
-  const uint32_t token = (uint32_t)(m - kv.row_offsets[low]) + kv.cache_lengths[low];
-  const uint32_t page = token / (uint32_t)kv.page_size, slot = token - page * (uint32_t)kv.page_size;
-  if ((int64_t)page >= kv.lut_ld) return -1;
-  const uint32_t block = kv.lookup_table[(int64_t)low * kv.lut_ld + page];
-  if ((int64_t)block >= kv.num_blocks) return -1;
-  return (int64_t)block * kv.block_stride + (int64_t)slot * kv.row_elems;
+  uint32_t token[R], page[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    token[r] = live[r] ? (uint32_t)(m[r] - kv.row_offsets[low[r]]) + kv.cache_lengths[low[r]] : 0u;
+    page[r] = token[r] / (uint32_t)kv.page_size;
+  }
+  uint32_t block[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const bool ok = live[r] && (int64_t)page[r] < kv.lut_ld;
+    block[r] = ok ? kv.lookup_table[(int64_t)low[r] * kv.lut_ld + page[r]] : 0xffffffffu;
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t slot = token[r] - page[r] * (uint32_t)kv.page_size;
+    off[r] = (int64_t)block[r] < kv.num_blocks ? (int64_t)block[r] * kv.block_stride + (int64_t)slot * kv.row_elems : -1;
+  }
+}
+
+__device__ __forceinline__ int64_t kv_row_offset(const KvStore& kv, int64_t m) {
+  const int64_t mm[1] = {m};
+  const bool live[1] = {true};
+  int64_t off[1];
+  kv_row_offsets<1>(kv, mm, live, off);
+  return off[0];
 }
 
 // destination of column n (and the columns after it up to the next multiple of 8) of row m

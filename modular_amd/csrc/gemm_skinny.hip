@@ -245,8 +245,8 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
       if (row_off < 0 && n >= p.kv.q_dim) continue;
       uint16_t* dst = kv_dst(p.kv, p.c, p.ldc, m, row_off, n);
       if (p.c_vec_ok && n + 3 < p.N) {
-        const uint32_t lo = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-        const uint32_t hi = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+        const uint32_t lo = pack_bf16x2(v[0], v[1]);
+        const uint32_t hi = pack_bf16x2(v[2], v[3]);
         *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
       } else {
 #pragma unroll
@@ -267,8 +267,8 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
     if (p.c_dtype == MAXFP8_BF16) {
       uint16_t* dst = reinterpret_cast<uint16_t*>(p.c) + (int64_t)m * p.ldc + n;
       if (p.c_vec_ok && n + 3 < p.N) {
-        const uint32_t lo = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-        const uint32_t hi = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+        const uint32_t lo = pack_bf16x2(v[0], v[1]);
+        const uint32_t hi = pack_bf16x2(v[2], v[3]);
         *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
       } else {
 #pragma unroll

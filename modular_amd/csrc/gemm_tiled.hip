@@ -96,7 +96,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
       if (p.c_vec8_ok && n + 7 < p.N) {
         uint32_t w[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
         *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
       } else {
 #pragma unroll
@@ -342,18 +342,19 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     // added in bf16 (kv_cache_ragged.mojo:1210-1245) -- and goes to C or to the row's K / V page.
     // Columns outside, rows inside: 8 weight scales and 8 bias values live at a time.
     float a_s[TM];
-    int64_t row_off[TM];
+    int64_t row_off[TM], rows[TM];
+    bool live[TM];
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) {
       int ml = wm * WM + mt * 16 + lm;
       asm volatile("" : "+v"(ml));  // keeps the page lookups here, out of the registers of the main loop
+      live[mt] = ml < rows_here;
+      rows[mt] = row_begin + ml;
       a_s[mt] = 1.f;
-      row_off[mt] = -1;
-      if (ml < rows_here) {
-        if constexpr (!BLOCKSCALE) a_s[mt] = bf16_round(p.a_scales[(row_begin + ml) * p.a_scale_stride]);
-        row_off[mt] = kv_row_offset(p.kv, row_begin + ml);
-      }
+      if constexpr (!BLOCKSCALE)
+        if (live[mt]) a_s[mt] = bf16_round(p.a_scales[rows[mt] * p.a_scale_stride]);
     }
+    kv_row_offsets<TM>(p.kv, rows, live, row_off);
     static_for<TN / 2>([&](auto qc) {  // (a plain unrolled loop leaves acc indexed at run time here)
       constexpr int q = decltype(qc)::value;
       const int n = n0 + wn * WN + q * 32 + lq * 8;
@@ -372,24 +373,27 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
         if (ml >= rows_here) continue;
         if (row_off[mt] < 0 && n >= p.kv.q_dim) continue;
         const v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
-        float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        uint32_t w[4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          float r = bf16_round(v[i]);
-          if constexpr (!BLOCKSCALE) r = bf16_round(r * bf16_round(a_s[mt] * b_s[i]));
-          if (p.kv.bias) r = bf16_round(r + bias[i]);
-          v[i] = r;
+        for (int i = 0; i < 4; ++i) {
+          w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+          if constexpr (!BLOCKSCALE) {
+            const float s0 = a_s[mt] * b_s[2 * i], s1 = a_s[mt] * b_s[2 * i + 1];
+            const uint32_t sc = pack_bf16x2(s0, s1);
+            w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) * __uint_as_float(sc << 16),
+                               __uint_as_float(w[i] & 0xffff0000u) * __uint_as_float(sc & 0xffff0000u));
+          }
+          if (p.kv.bias)
+            w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) + bias[2 * i], __uint_as_float(w[i] & 0xffff0000u) + bias[2 * i + 1]);
         }
         uint16_t* dst = kv_dst(p.kv, p.c, p.ldc, row_begin + ml, row_off[mt], n);
         if (p.c_vec8_ok && n + 7 < p.N) {
-          uint32_t w[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
           *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
         } else {
 #pragma unroll
           for (int i = 0; i < 8; ++i)
-            if (n + i < p.N) dst[i] = (uint16_t)f32_to_bf16_bits(v[i]);
+            if (n + i < p.N) dst[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
         }
       }
     });
@@ -692,12 +696,75 @@ size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return worst * (size_t)M * (size_t)N * 4;
 }
 
+// cost (microseconds) of an unsplit M x N region in tiles of shape t
+static float region_cost(int64_t M, int64_t N, int nslab, const TileShape& t, bool blockscale) {
+  const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+  return (float)ceil_div(tiles, t.slots) * ((float)nslab * (blockscale ? t.t_slab_block : t.t_slab_row) + t.t_tile);
+}
+
+// A matmul whose tiles fill the chip a whole number of times plus a small rest wastes most of its
+// last round.  Such a problem is cut in two along N or M: a first region that the main shape
+// covers in full rounds, and a rest that runs as a second launch in whatever shape fills the
+// chip best (e.g. Llama-8B gate_up, M = 2048: 896 tiles of 256 x 256 are 3.5 rounds; 768 of
+// them plus 256 tiles of 256 x 128 are 3 rounds and one short one).  The cost model decides.
+struct TwoRegionPlan { int axis; int64_t cut; int v1, v2; float cost; };  // axis 0: none, 1: N, 2: M
+static TwoRegionPlan pick_two_regions(int64_t M, int64_t N, int nslab, bool blockscale, float single_cost) {
+  constexpr float kSecondLaunch = 4.0f;  // the second launch starts when the first has drained
+  TwoRegionPlan best = {0, 0, 0, 0, single_cost - 4.0f};  // must beat the single launch by a margin
+  for (int i = 0; i < 3; ++i) {
+    for (int j = 0; j < 3; ++j) {
+      const TileShape &a = kShapes[i], &b = kShapes[j];
+      for (int64_t c = 1; c < ceil_div(N, a.bn); ++c) {
+        const float t = region_cost(M, c * a.bn, nslab, a, blockscale) + region_cost(M, N - c * a.bn, nslab, b, blockscale) + kSecondLaunch;
+        if (t < best.cost) best = {1, c * a.bn, i + 1, j + 1, t};
+      }
+      for (int64_t c = 1; c < ceil_div(M, a.bm); ++c) {
+        const float t = region_cost(c * a.bm, N, nslab, a, blockscale) + region_cost(M - c * a.bm, N, nslab, b, blockscale) + kSecondLaunch;
+        if (t < best.cost) best = {2, c * a.bm, i + 1, j + 1, t};
+      }
+    }
+  }
+  return best;
+}
+
 int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, int64_t batch, hipStream_t stream) {
   GemmArgs p = p_in;
   const int nslab = (p.K + 127) / 128;
   int variant = tile_override();
+  const bool free_choice = variant == 0;
   if (!variant) variant = pick_shape(p.M, p.N, nslab, blockscale, p.workspace != nullptr && batch == 1, batch);
   if (p.kv_on && variant != 1) variant = 3;  // the fused QKV kernels exist in the 256 x 256 and 128 x 128 shapes
+  if (free_choice && batch == 1 && !p.kv_on && !getenv("MAXFP8_ONE_REGION")) {
+    const TileShape& t1 = kShapes[variant - 1];
+    const int64_t tiles1 = ceil_div(p.M, t1.bm) * ceil_div(p.N, t1.bn);
+    const bool would_split_k = p.workspace && pick_splits(tiles1, t1.slots, nslab) > 1;
+    const TwoRegionPlan plan = would_split_k ? TwoRegionPlan{0, 0, 0, 0, 0.f}
+                                             : pick_two_regions(p.M, p.N, nslab, blockscale, region_cost(p.M, p.N, nslab, t1, blockscale));
+    if (plan.axis) {
+      GemmArgs r1 = p, r2 = p;
+      r1.splits = r2.splits = 1;
+      const int64_t esz = p.c_dtype == MAXFP8_BF16 ? 2 : 4;
+      if (plan.axis == 1) {  // columns [0, cut) and [cut, N): weight rows, their scales, C columns
+        r1.N = (int)plan.cut;
+        r2.N = p.N - (int)plan.cut;
+        r2.b = p.b + plan.cut * p.ldb;
+        r2.c = reinterpret_cast<uint8_t*>(p.c) + plan.cut * esz;
+        r2.b_scales = blockscale ? p.b_scales + (plan.cut / 128) * p.b_scales_ld : p.b_scales + plan.cut * p.b_scale_stride;
+      } else {               // rows [0, cut) and [cut, M): activation rows, their scales, C rows
+        r1.M = (int)plan.cut;
+        r2.M = p.M - (int)plan.cut;
+        r2.a = p.a + plan.cut * p.lda;
+        r2.c = reinterpret_cast<uint8_t*>(p.c) + plan.cut * p.ldc * esz;
+        r2.a_scales = blockscale ? p.a_scales + plan.cut : p.a_scales + plan.cut * p.a_scale_stride;
+      }
+      const TileShape &ta = kShapes[plan.v1 - 1], &tb = kShapes[plan.v2 - 1];
+      const dim3 g1((unsigned)(ceil_div(r1.M, ta.bm) * ceil_div(r1.N, ta.bn)), 1, 1);
+      const dim3 g2((unsigned)(ceil_div(r2.M, tb.bm) * ceil_div(r2.N, tb.bn)), 1, 1);
+      const int rc = gemm_tiled_launch(r1, blockscale, plan.v1, g1, stream);
+      if (rc != MAXFP8_OK) return rc;
+      return gemm_tiled_launch(r2, blockscale, plan.v2, g2, stream);
+    }
+  }
   const TileShape& t = kShapes[variant - 1];
   const int64_t tiles = ceil_div(p.M, t.bm) * ceil_div(p.N, t.bn);
   if (tiles >= ((int64_t)1 << 31)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "tiled matmul: too many tiles");

@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__
     if constexpr (!QUANT) {
       uint32_t w[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) w[j] = f32_to_bf16_bits(f[2 * j]) | (f32_to_bf16_bits(f[2 * j + 1]) << 16);
+      for (int j = 0; j < 4; ++j) w[j] = pack_bf16x2(f[2 * j], f[2 * j + 1]);
       *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(out) + m * out_stride + g * 128 + sub * 8) =
           make_uint4(w[0], w[1], w[2], w[3]);
     } else {

@@ -431,6 +431,17 @@ __global__ __launch_bounds__(256) void cast_f32_to_e4m3fn_kernel(uint8_t* out, c
   for (; i < n; i += stride) out[i] = encode_one(clamp448(in[i]));
 }
 
+// pairs of f32 -> bf16 through pack_bf16x2, the convert the matmul epilogues use
+__global__ __launch_bounds__(256) void cast_f32_to_bf16_kernel(uint16_t* out, const float* in, int64_t n) {
+  int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  const int64_t stride = (int64_t)gridDim.x * 512;
+  for (; i < n; i += stride) {
+    const uint32_t w = pack_bf16x2(in[i], i + 1 < n ? in[i + 1] : 0.f);
+    out[i] = (uint16_t)w;
+    if (i + 1 < n) out[i + 1] = (uint16_t)(w >> 16);
+  }
+}
+
 __global__ __launch_bounds__(256) void cast_e4m3fn_to_f32_kernel(float* out, const uint8_t* in, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
@@ -558,6 +569,13 @@ int cast_f32_to_e4m3fn_dispatch(void* out, const float* in, int64_t n, hipStream
   const unsigned blocks = (unsigned)(ceil_div(n, 256) < 65536 ? ceil_div(n, 256) : 65536);
   hipLaunchKernelGGL(cast_f32_to_e4m3fn_kernel, dim3(blocks), dim3(256), 0, stream, (uint8_t*)out, in, n);
   return launch_status("cast_f32_to_e4m3fn");
+}
+
+int cast_f32_to_bf16_dispatch(void* out, const float* in, int64_t n, hipStream_t stream) {
+  const int64_t pairs = ceil_div(n, 2);
+  const unsigned blocks = (unsigned)(ceil_div(pairs, 256) < 65536 ? ceil_div(pairs, 256) : 65536);
+  hipLaunchKernelGGL(cast_f32_to_bf16_kernel, dim3(blocks), dim3(256), 0, stream, (uint16_t*)out, in, n);
+  return launch_status("cast_f32_to_bf16");
 }
 
 int cast_e4m3fn_to_f32_dispatch(float* out, const void* in, int64_t n, hipStream_t stream) {

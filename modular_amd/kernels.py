@@ -667,6 +667,14 @@ def cast_f32_to_e4m3fn(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def cast_f32_to_bf16(x: torch.Tensor) -> torch.Tensor:
+    _require_gpu(x)
+    x = x.contiguous().to(torch.float32)
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    _lib.check(_lib.lib().maxfp8_cast_f32_to_bf16(out.data_ptr(), x.data_ptr(), x.numel(), _stream(x)))
+    return out
+
+
 def cast_e4m3fn_to_f32(x: torch.Tensor) -> torch.Tensor:
     _require_gpu(x)
     x = x.contiguous()

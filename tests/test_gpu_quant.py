@@ -180,3 +180,19 @@ def test_moe_size_properties(dev):
     assert bool(torch.all(mag[amax > 0] == 0x7E))
     # idempotence of the byte pattern: dequantise * scale, requantise with the same scales -> same bytes
     assert not bool(torch.any((q.view(torch.uint8) & 0x7F) == 0x7F))
+
+
+def test_hardware_bf16_convert_is_round_to_nearest_even(dev):
+    # every bf16 value with the three low-half patterns that decide the rounding (just below a tie,
+    # the tie, just above), plus random bit patterns; NaNs only have to stay NaNs
+    hi = np.arange(65536, dtype=np.uint32) << 16
+    cases = np.concatenate([hi | lo for lo in (0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF)])
+    rnd = np.random.default_rng(0).integers(0, 2 ** 32, size=1 << 22, dtype=np.uint64).astype(np.uint32)
+    x = np.concatenate([cases, rnd]).view(np.float32)
+    if x.size % 2:
+        x = x[:-1]
+    got = bf16_bits(kernels.cast_f32_to_bf16(torch.from_numpy(x).to(dev)))
+    want = oracle.bf16_bits_of(oracle.bf16_round(x))
+    nan = np.isnan(x)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.all((got[nan] & 0x7F80) == 0x7F80) and np.all((got[nan] & 0x007F) != 0)

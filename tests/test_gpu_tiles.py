@@ -161,3 +161,30 @@ def test_grouped_small_tiles_exact(dev):
             want[r0:r1] += part * np.exp2(ea[j, r0:r1])[:, None] * np.exp2(eb[e][np.arange(N) // 128, j])[None, :]
     c = run_grouped(a, b, sa, sb, off, ids, max(counts), len(counts), dev, algo="tiled")
     assert np.array_equal(f32_np(c).astype(np.float64), want)
+
+
+# Problems whose 256 x 256 tiles make a whole number of rounds plus a small rest run as two
+# launches (a cut along N or along M, the rest in another tile shape): both sides of the cut
+# are checked on sampled rows by the naive kernel, which is the oracle bit for bit.
+@pytest.mark.parametrize("M,K,N,kind", [
+    (2048, 4096, 28672, "block"),    # Llama-3.1-8B gate_up: 3.5 rounds -> cut along N
+    (2040, 4096, 28600, "block"),    # the same with ragged edges on both axes
+    (28672, 4096, 2048, "block"),    # the transposed problem -> cut along M
+    (28600, 4096, 2040, "row"),
+    (2048, 4096, 28672, "row"),
+])
+def test_two_region_launch(dev, M, K, N, kind):
+    cfg = BLK if kind == "block" else ROW
+    x = synth.activations(M, K, seed=0, outlier_frac=0.0 if kind == "row" else 0.01, device=dev)
+    wf = synth.weights_f32(N, K, seed=1, device=dev)
+    w, sb = synth.quantize_weight_block(wf) if kind == "block" else synth.quantize_weight_rowwise(wf)
+    q, sa = mx.quantize_dynamic_scaled_float8(x, cfg.input_scale, cfg.weight_scale, scales_type=torch.float32)
+    c = mx.dynamic_scaled_matmul(q, w, sa, sb, cfg.input_scale, cfg.weight_scale)
+    rows = torch.unique(torch.cat([torch.arange(0, M, max(1, M // 29), device=dev), torch.tensor([M - 1], device=dev)]))
+    ref = mx.dynamic_scaled_matmul(q[rows].contiguous(), w, sa[:, rows].contiguous(), sb, cfg.input_scale,
+                                   cfg.weight_scale, out_type=torch.float32, algo="naive")
+    torch.cuda.synchronize()
+    assert_rel(f32_np(c[rows]), f32_np(ref), TOL, f"two regions {M}x{N}x{K} {kind}")
+    # and the f32 output path, against the same reference
+    c32 = mx.dynamic_scaled_matmul(q, w, sa, sb, cfg.input_scale, cfg.weight_scale, out_type=torch.float32)
+    assert_rel(f32_np(c32[rows]), f32_np(ref), TOL, f"two regions f32 {M}x{N}x{K} {kind}", abs_budget=F32_BUDGET)
