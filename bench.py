@@ -273,6 +273,13 @@ def result_line(name, steps, warmup, with_cpu=True):
     roof["algorithmic_bytes"] = mm_bytes
     roof["kernel"] = {"grouped": "gemm_grouped_kernel", "row": "gemm_skinny_kernel", "rmsq": "rmsnorm_quant_row_bf16_kernel"}.get(
         kind, "gemm_skinny_kernel" if M <= 64 else "gemm_tiled_kernel")
+    # the matmul can be more than one launch (two regions in different tile shapes; the grouped matmul's
+    # large-tile launch and the rest): kernel_ms_* is the time of all of them, one after the other
+    if kind == "grouped":
+        roof["launches"] = "gemm_grouped_large_kernel (full 256-row tiles of experts with >= 1024 rows) + gemm_grouped_kernel (the rest)"
+    elif kind in ("block", "row") and M > 64:
+        from modular_amd import _lib
+        roof["launches"] = _lib.matmul_describe(M, N, K, kind == "block", True)
     roof["kernel_ms_avg"], roof["kernel_ms_median"], roof["kernel_ms_min"] = mm_avg, mm_med, mm_min
     out = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,

@@ -187,6 +187,14 @@ int maxfp8_batched_matmul_dynamic_scaled_fp8(
     int64_t b_scales_batch_stride, int64_t b_scales_ld,
     int c_dtype, int scales_dtype, int algo, void* stream);
 
+/*
+ * Diagnostic: which launches MAXFP8_ALGO_AUTO makes for a fast-layout M x N x K matmul, as text
+ * ("256x256 x768 + columns from 24576: 256x128 x256", "256x128 x112, K split 4", "skinny").
+ * Returns the length snprintf would have written.  No counterpart in the reference.
+ */
+int maxfp8_matmul_describe(int64_t M, int64_t N, int64_t K, int block_scaling, int with_workspace,
+                           char* buf, size_t len);
+
 /* Bytes of workspace that lets AUTO use every kernel for this shape. */
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K);
 

@@ -29,6 +29,7 @@ EXPORTS = (
     "maxfp8_matmul_dynamic_scaled_fp8",
     "maxfp8_batched_matmul_dynamic_scaled_fp8",
     "maxfp8_matmul_workspace_bytes",
+    "maxfp8_matmul_describe",
     "maxfp8_grouped_matmul_dynamic_scaled_fp8",
     "maxfp8_fused_qkv_matmul_ragged_paged_scale",
     "maxfp8_quantize_static_scaled_fp8",
@@ -74,6 +75,8 @@ def lib() -> ctypes.CDLL:
                                                   [ci, ci, ci, vp, ctypes.c_size_t, vp])
     L.maxfp8_batched_matmul_dynamic_scaled_fp8.restype = ci
     L.maxfp8_batched_matmul_dynamic_scaled_fp8.argtypes = [vp] * 5 + [i64] * 17 + [ci, ci, ci, vp]
+    L.maxfp8_matmul_describe.restype = ci
+    L.maxfp8_matmul_describe.argtypes = [i64, i64, i64, ci, ci, ctypes.c_char_p, ctypes.c_size_t]
     L.maxfp8_matmul_workspace_bytes.restype = ctypes.c_size_t
     L.maxfp8_matmul_workspace_bytes.argtypes = [i64, i64, i64]
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8.restype = ci
@@ -115,3 +118,10 @@ def check(status: int) -> None:
     if status in (ERR_SHAPE, ERR_ALIGN, ERR_GRANULARITY, ERR_NULL, ERR_WORKSPACE):
         raise ValueError(msg)
     raise RuntimeError(msg)
+
+
+def matmul_describe(M: int, N: int, K: int, block_scaling: bool = True, with_workspace: bool = True) -> str:
+    """The launches MAXFP8_ALGO_AUTO makes for a fast-layout matmul, as text (diagnostic)."""
+    buf = ctypes.create_string_buffer(256)
+    lib().maxfp8_matmul_describe(M, N, K, int(block_scaling), int(with_workspace), buf, 256)
+    return buf.value.decode()

@@ -45,6 +45,7 @@ int naive_grouped_dispatch(void*, const void*, const void*, const void*, const v
                            const int32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int, hipStream_t);
 int gemm_tiled_dispatch(const GemmArgs&, bool, size_t, int64_t, hipStream_t);
 size_t gemm_tiled_workspace_bytes(int64_t, int64_t, int64_t);
+int gemm_tiled_describe(int64_t, int64_t, int64_t, bool, bool, char*, size_t);
 int gemm_grouped_dispatch(const GemmArgs&, int64_t, int64_t, hipStream_t);
 int gemm_skinny_dispatch(const GemmArgs&, bool, int64_t, hipStream_t);
 int gemm_skinny_max_m();
@@ -296,6 +297,13 @@ static int matmul_common(void* c, const void* a, const void* b, const void* a_sc
 }  // namespace maxfp8
 
 extern "C" {
+
+int maxfp8_matmul_describe(int64_t M, int64_t N, int64_t K, int block_scaling, int with_workspace, char* buf, size_t len) {
+  if (!buf || len == 0) return 0;
+  if (M <= 0 || N <= 0 || K <= 0) return snprintf(buf, len, "nothing to do");
+  if (M <= gemm_skinny_max_m()) return snprintf(buf, len, "skinny");
+  return gemm_tiled_describe(M, N, K, block_scaling != 0, with_workspace != 0, buf, len);
+}
 
 int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
                                      const void* b_scales, int64_t M, int64_t N, int64_t K, int64_t lda,

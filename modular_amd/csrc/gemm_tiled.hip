@@ -727,52 +727,77 @@ static TwoRegionPlan pick_two_regions(int64_t M, int64_t N, int nslab, bool bloc
   return best;
 }
 
+// What a tiled matmul will launch: one shape (possibly with K split), or two regions.
+struct TiledPlan { int variant; int splits; TwoRegionPlan two; };
+static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, size_t workspace_bytes,
+                           int64_t batch, bool kv_on) {
+  TiledPlan plan = {0, 1, {0, 0, 0, 0, 0.f}};
+  const int nslab = (int)ceil_div(K, 128);
+  plan.variant = tile_override();
+  const bool free_choice = plan.variant == 0;
+  if (!plan.variant) plan.variant = pick_shape(M, N, nslab, blockscale, has_workspace && batch == 1, batch);
+  if (kv_on && plan.variant != 1) plan.variant = 3;  // the fused QKV kernels exist in the 256 x 256 and 128 x 128 shapes
+  const TileShape& t = kShapes[plan.variant - 1];
+  const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+  if (has_workspace && batch == 1 && !kv_on) {
+    const int sp = pick_splits(tiles, t.slots, nslab);
+    if (sp > 1 && (size_t)sp * M * N * 4 <= workspace_bytes) plan.splits = sp;
+  }
+  if (free_choice && batch == 1 && !kv_on && plan.splits == 1 && !getenv("MAXFP8_ONE_REGION"))
+    plan.two = pick_two_regions(M, N, nslab, blockscale, region_cost(M, N, nslab, t, blockscale));
+  return plan;
+}
+
+// "256x256 x896" / "256x256 x448, K split 2" / "256x256 x768 + columns from 24576: 256x128 x256"
+int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, char* buf, size_t len) {
+  const TiledPlan plan = make_plan(M, N, K, blockscale, has_workspace, has_workspace ? gemm_tiled_workspace_bytes(M, N, K) : 0, 1, false);
+  auto count = [](int64_t m, int64_t n, const TileShape& t) { return (long long)(ceil_div(m, t.bm) * ceil_div(n, t.bn)); };
+  if (plan.two.axis) {
+    const TileShape &a = kShapes[plan.two.v1 - 1], &b = kShapes[plan.two.v2 - 1];
+    const bool cols = plan.two.axis == 1;
+    const int64_t m1 = cols ? M : plan.two.cut, n1 = cols ? plan.two.cut : N;
+    const int64_t m2 = cols ? M : M - plan.two.cut, n2 = cols ? N - plan.two.cut : N;
+    return snprintf(buf, len, "%dx%d x%lld + %s from %lld: %dx%d x%lld", a.bm, a.bn, count(m1, n1, a), cols ? "columns" : "rows",
+                    (long long)plan.two.cut, b.bm, b.bn, count(m2, n2, b));
+  }
+  const TileShape& t = kShapes[plan.variant - 1];
+  if (plan.splits > 1) return snprintf(buf, len, "%dx%d x%lld, K split %d", t.bm, t.bn, count(M, N, t), plan.splits);
+  return snprintf(buf, len, "%dx%d x%lld", t.bm, t.bn, count(M, N, t));
+}
+
 int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, int64_t batch, hipStream_t stream) {
   GemmArgs p = p_in;
-  const int nslab = (p.K + 127) / 128;
-  int variant = tile_override();
-  const bool free_choice = variant == 0;
-  if (!variant) variant = pick_shape(p.M, p.N, nslab, blockscale, p.workspace != nullptr && batch == 1, batch);
-  if (p.kv_on && variant != 1) variant = 3;  // the fused QKV kernels exist in the 256 x 256 and 128 x 128 shapes
-  if (free_choice && batch == 1 && !p.kv_on && !getenv("MAXFP8_ONE_REGION")) {
-    const TileShape& t1 = kShapes[variant - 1];
-    const int64_t tiles1 = ceil_div(p.M, t1.bm) * ceil_div(p.N, t1.bn);
-    const bool would_split_k = p.workspace && pick_splits(tiles1, t1.slots, nslab) > 1;
-    const TwoRegionPlan plan = would_split_k ? TwoRegionPlan{0, 0, 0, 0, 0.f}
-                                             : pick_two_regions(p.M, p.N, nslab, blockscale, region_cost(p.M, p.N, nslab, t1, blockscale));
-    if (plan.axis) {
-      GemmArgs r1 = p, r2 = p;
-      r1.splits = r2.splits = 1;
-      const int64_t esz = p.c_dtype == MAXFP8_BF16 ? 2 : 4;
-      if (plan.axis == 1) {  // columns [0, cut) and [cut, N): weight rows, their scales, C columns
-        r1.N = (int)plan.cut;
-        r2.N = p.N - (int)plan.cut;
-        r2.b = p.b + plan.cut * p.ldb;
-        r2.c = reinterpret_cast<uint8_t*>(p.c) + plan.cut * esz;
-        r2.b_scales = blockscale ? p.b_scales + (plan.cut / 128) * p.b_scales_ld : p.b_scales + plan.cut * p.b_scale_stride;
-      } else {               // rows [0, cut) and [cut, M): activation rows, their scales, C rows
-        r1.M = (int)plan.cut;
-        r2.M = p.M - (int)plan.cut;
-        r2.a = p.a + plan.cut * p.lda;
-        r2.c = reinterpret_cast<uint8_t*>(p.c) + plan.cut * p.ldc * esz;
-        r2.a_scales = blockscale ? p.a_scales + plan.cut : p.a_scales + plan.cut * p.a_scale_stride;
-      }
-      const TileShape &ta = kShapes[plan.v1 - 1], &tb = kShapes[plan.v2 - 1];
-      const dim3 g1((unsigned)(ceil_div(r1.M, ta.bm) * ceil_div(r1.N, ta.bn)), 1, 1);
-      const dim3 g2((unsigned)(ceil_div(r2.M, tb.bm) * ceil_div(r2.N, tb.bn)), 1, 1);
-      const int rc = gemm_tiled_launch(r1, blockscale, plan.v1, g1, stream);
-      if (rc != MAXFP8_OK) return rc;
-      return gemm_tiled_launch(r2, blockscale, plan.v2, g2, stream);
+  const TiledPlan plan = make_plan(p.M, p.N, p.K, blockscale, p.workspace != nullptr, workspace_bytes, batch, p.kv_on != 0);
+  if (plan.two.axis) {
+    const TwoRegionPlan& two = plan.two;
+    GemmArgs r1 = p, r2 = p;
+    r1.splits = r2.splits = 1;
+    const int64_t esz = p.c_dtype == MAXFP8_BF16 ? 2 : 4;
+    if (two.axis == 1) {  // columns [0, cut) and [cut, N): weight rows, their scales, C columns
+      r1.N = (int)two.cut;
+      r2.N = p.N - (int)two.cut;
+      r2.b = p.b + two.cut * p.ldb;
+      r2.c = reinterpret_cast<uint8_t*>(p.c) + two.cut * esz;
+      r2.b_scales = blockscale ? p.b_scales + (two.cut / 128) * p.b_scales_ld : p.b_scales + two.cut * p.b_scale_stride;
+    } else {              // rows [0, cut) and [cut, M): activation rows, their scales, C rows
+      r1.M = (int)two.cut;
+      r2.M = p.M - (int)two.cut;
+      r2.a = p.a + two.cut * p.lda;
+      r2.c = reinterpret_cast<uint8_t*>(p.c) + two.cut * p.ldc * esz;
+      r2.a_scales = blockscale ? p.a_scales + two.cut : p.a_scales + two.cut * p.a_scale_stride;
     }
+    const TileShape &ta = kShapes[two.v1 - 1], &tb = kShapes[two.v2 - 1];
+    const dim3 g1((unsigned)(ceil_div(r1.M, ta.bm) * ceil_div(r1.N, ta.bn)), 1, 1);
+    const dim3 g2((unsigned)(ceil_div(r2.M, tb.bm) * ceil_div(r2.N, tb.bn)), 1, 1);
+    const int rc = gemm_tiled_launch(r1, blockscale, two.v1, g1, stream);
+    if (rc != MAXFP8_OK) return rc;
+    return gemm_tiled_launch(r2, blockscale, two.v2, g2, stream);
   }
+  const int variant = plan.variant;
   const TileShape& t = kShapes[variant - 1];
   const int64_t tiles = ceil_div(p.M, t.bm) * ceil_div(p.N, t.bn);
   if (tiles >= ((int64_t)1 << 31)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "tiled matmul: too many tiles");
-  p.splits = 1;
-  if (p.workspace && batch == 1) {
-    const int sp = pick_splits(tiles, t.slots, (p.K + 127) / 128);
-    if (sp > 1 && (size_t)sp * p.M * p.N * 4 <= workspace_bytes) p.splits = sp;
-  }
+  p.splits = plan.splits;
   const dim3 grid((unsigned)tiles, (unsigned)p.splits, (unsigned)batch);
   const int rc = gemm_tiled_launch(p, blockscale, variant, grid, stream);
   if (rc != MAXFP8_OK || p.splits == 1) return rc;

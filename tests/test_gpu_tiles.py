@@ -174,6 +174,7 @@ def test_grouped_small_tiles_exact(dev):
     (2048, 4096, 28672, "row"),
 ])
 def test_two_region_launch(dev, M, K, N, kind):
+    assert " + " in _lib.matmul_describe(M, N, K, kind == "block"), "this shape is meant to run as two launches"
     cfg = BLK if kind == "block" else ROW
     x = synth.activations(M, K, seed=0, outlier_frac=0.0 if kind == "row" else 0.01, device=dev)
     wf = synth.weights_f32(N, K, seed=1, device=dev)

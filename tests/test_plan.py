@@ -1,0 +1,35 @@
+"""Host logic that chooses the launches of a tiled matmul (no GPU needed): one tile shape,
+a K split when the caller brings a workspace, or two regions when the last round of the
+main shape would leave most of the chip idle."""
+import re
+
+from modular_amd import _lib
+
+
+def parse(text):
+    parts = [re.match(r"(\d+)x(\d+) x(\d+)", p.strip()) for p in re.split(r"\+ (?:columns|rows) from \d+:", text)]
+    return [(int(m.group(1)), int(m.group(2)), int(m.group(3))) for m in parts]
+
+
+def test_single_shapes_and_k_split():
+    assert _lib.matmul_describe(2048, 6144, 4096) == "256x256 x192"
+    assert _lib.matmul_describe(8, 4096, 4096) == "skinny"
+    with_ws, without = _lib.matmul_describe(256, 7168, 16384), _lib.matmul_describe(256, 7168, 16384, True, False)
+    assert "K split" in with_ws and "K split" not in without
+    assert _lib.matmul_describe(0, 10, 10) == "nothing to do"
+
+
+def test_two_regions_cover_the_problem_once():
+    for (M, N, K) in [(2048, 28672, 4096), (28672, 2048, 4096), (2040, 28600, 4096)]:
+        text = _lib.matmul_describe(M, N, K)
+        assert " + " in text, text
+        cut = int(re.search(r"from (\d+)", text).group(1))
+        (bm1, bn1, n1), (bm2, bn2, n2) = parse(text)
+        ceil = lambda a, b: -(-a // b)
+        if "columns" in text:
+            assert cut % bn1 == 0 and 0 < cut < N
+            assert n1 == ceil(M, bm1) * (cut // bn1) and n2 == ceil(M, bm2) * ceil(N - cut, bn2)
+        else:
+            assert cut % bm1 == 0 and 0 < cut < M
+            assert n1 == (cut // bm1) * ceil(N, bn1) and n2 == ceil(M - cut, bm2) * ceil(N, bn2)
+        assert n1 % 256 == 0, "the first region runs in whole rounds of the 256 CUs"
