@@ -399,6 +399,53 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     });
     return;
   }
+  // bf16 tiles with all their columns go through LDS, so that a store instruction writes whole
+  // 128-byte lines (8 lanes per row of the wave's WM x WN part) instead of 64-byte halves: each
+  // wave owns WM * WN * 2 bytes of the stage memory, written with the 16-byte chunk index XORed
+  // with the row (conflict-free in both directions).
+  constexpr int CH = WN * 2 / 16;  // 16-byte chunks per row of a wave's part
+  constexpr bool LDS_STORE = !GROUPED && CH == 8 && NWAVES * WM * WN * 2 <= NS * STAGE_BYTES;
+  if constexpr (LDS_STORE) {
+    if (p.c_dtype == MAXFP8_BF16 && p.c_vec8_ok && n0 + BN <= p.N) {
+      __syncthreads();  // every wave has finished reading the stages
+      uint8_t* wbuf = smem + wave * (WM * WN * 2);
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        const int r = mt * 16 + lm;
+        float a_s = 1.f;
+        if constexpr (!BLOCKSCALE) {
+          const int64_t mm = row_begin + wm * WM + r;
+          a_s = p.a_scales[(mm < p.M ? mm : p.M - 1) * p.a_scale_stride];
+        }
+#pragma unroll
+        for (int q = 0; q < TN / 2; ++q) {
+          v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
+          if constexpr (!BLOCKSCALE) {
+            const int n = n0 + wn * WN + q * 32 + lq * 8;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
+              lo[i] = t_lo * p.b_scales[(int64_t)(n + i) * p.b_scale_stride];
+              hi[i] = t_hi * p.b_scales[(int64_t)(n + 4 + i) * p.b_scale_stride];
+            }
+          }
+          const int chunk = (q * 4 + lq) ^ (r & 7);
+          *reinterpret_cast<uint4*>(wbuf + r * (WN * 2) + chunk * 16) =
+              make_uint4(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3]));
+        }
+      }
+      // (a wave reads back only what it wrote itself: no barrier, the compiler orders the LDS accesses)
+      const int rr = lane >> 3, cc = lane & 7;
+      uint16_t* cbase = reinterpret_cast<uint16_t*>(p.c) + (row_begin + wm * WM) * p.ldc + n0 + wn * WN + cc * 8;
+#pragma unroll
+      for (int i = 0; i < WM / 8; ++i) {
+        const int r = i * 8 + rr;
+        const uint4 v = *reinterpret_cast<const uint4*>(wbuf + r * (WN * 2) + ((cc ^ (r & 7)) * 16));
+        if (wm * WM + r < rows_here) *reinterpret_cast<uint4*>(cbase + (int64_t)r * p.ldc) = v;
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int mt = 0; mt < TM; ++mt) {
     const int ml = wm * WM + mt * 16 + lm;
