@@ -268,6 +268,24 @@ int maxfp8_grouped_matmul_dynamic_scaled_fp8(
     int64_t a_scales_ld, int c_dtype, int scales_dtype, int algo, void* stream);
 
 /*
+ * Grouped (MoE) FP8 matmul with per-token activation scales and per-output-channel weight
+ * scales.  Replaces mo.grouped.matmul.rowwise.dynamic.scaled.fp8
+ *   (wrapper max/python/max/nn/kernels.py:6490-6640)
+ * -> grouped_matmul_rowwise_dynamic_scaled_fp8 (max/kernels/src/linalg/grouped_matmul.mojo:1440-1713):
+ *   C[t, n] = (sum_k A[t, k] B[expert_ids[z], n, k]) * a_scales[t] * b_scales[expert_ids[z], n]
+ * for the rows t of slot z; slots with expert id -1 give zeros.
+ *   a [T, K], b [num_experts, N, K] e4m3fn contiguous; a_scales [T, 1], b_scales [num_experts, N, 1] f32;
+ *   expert_start_indices, expert_ids, max_num_tokens_per_expert, num_active_experts as in
+ *   maxfp8_grouped_matmul_dynamic_scaled_fp8.  Needs K % 16 == 0 and 16-byte aligned a, b.
+ */
+int maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8(
+    void* c, const void* a, const void* b, const void* a_scales, const void* b_scales,
+    const uint32_t* expert_start_indices, const int32_t* expert_ids,
+    int64_t T, int64_t N, int64_t K, int64_t num_experts,
+    int64_t max_num_tokens_per_expert, int64_t num_active_experts,
+    int c_dtype, int scales_dtype, void* stream);
+
+/*
  * mo.composite.rms_norm_fused_quantize_dynamic_scaled_fp8
  *   (op registration: max/kernels/src/graph_compiler/builtin_kernels/quantization.mojo:112-237;
  *    kernel: max/kernels/src/nn/normalization.mojo:3996-4175)

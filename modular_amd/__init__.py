@@ -7,7 +7,7 @@ through the C ABI of include/maxfp8.h; there is no CPU or PyTorch fallback.
 from .quant_config import (InputScaleSpec, QuantConfig, QuantFormat, ScaleGranularity, ScaleOrigin,
                            WeightScaleSpec, blockwise_fp8_config, rowwise_fp8_config)
 from .kv_cache import KVCacheParams, PagedCacheValues
-from .kernels import (fused_qkv_ragged_matmul_scaled_float8, matmul_k_cache_ragged_scaled_float8,
+from .kernels import (grouped_matmul_rowwise_dynamic_scaled_fp8, fused_qkv_ragged_matmul_scaled_float8, matmul_k_cache_ragged_scaled_float8,
                       batched_dynamic_scaled_fp8_matmul, batched_quantize_dynamic_scaled_fp8, dynamic_scaled_matmul,
                       grouped_dynamic_scaled_fp8_matmul, matmul_static_scaled_float8,
                       quantize_static_scaled_float8, quantize_tensor_dynamic_scaled_float8,
@@ -26,5 +26,5 @@ __all__ = [
     "quantize_static_scaled_float8", "matmul_static_scaled_float8", "parse_quant_config",
     "batched_dynamic_scaled_fp8_matmul", "batched_quantize_dynamic_scaled_fp8",
     "quantize_tensor_dynamic_scaled_float8", "fused_qkv_ragged_matmul_scaled_float8",
-    "matmul_k_cache_ragged_scaled_float8", "KVCacheParams", "PagedCacheValues", "quantized_fused_qkv_matmul",
+    "matmul_k_cache_ragged_scaled_float8", "KVCacheParams", "PagedCacheValues", "quantized_fused_qkv_matmul", "grouped_matmul_rowwise_dynamic_scaled_fp8",
 ]

@@ -31,6 +31,7 @@ EXPORTS = (
     "maxfp8_matmul_workspace_bytes",
     "maxfp8_matmul_describe",
     "maxfp8_grouped_matmul_dynamic_scaled_fp8",
+    "maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8",
     "maxfp8_fused_qkv_matmul_ragged_paged_scale",
     "maxfp8_quantize_static_scaled_fp8",
     "maxfp8_quantize_tensor_dynamic_scaled_fp8",
@@ -81,6 +82,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_matmul_workspace_bytes.argtypes = [i64, i64, i64]
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8.restype = ci
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8.argtypes = [vp] * 7 + [i64] * 7 + [ci, ci, ci, vp]
+    L.maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8.restype = ci
+    L.maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8.argtypes = [vp] * 7 + [i64] * 6 + [ci, ci, vp]
     L.maxfp8_fused_qkv_matmul_ragged_paged_scale.restype = ci
     L.maxfp8_fused_qkv_matmul_ragged_paged_scale.argtypes = [vp] * 10 + [i64] * 18 + [ci, ci, vp]
     L.maxfp8_quantize_static_scaled_fp8.restype = ci

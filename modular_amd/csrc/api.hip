@@ -46,7 +46,7 @@ int naive_grouped_dispatch(void*, const void*, const void*, const void*, const v
 int gemm_tiled_dispatch(const GemmArgs&, bool, size_t, int64_t, hipStream_t);
 size_t gemm_tiled_workspace_bytes(int64_t, int64_t, int64_t);
 int gemm_tiled_describe(int64_t, int64_t, int64_t, bool, bool, char*, size_t);
-int gemm_grouped_dispatch(const GemmArgs&, int64_t, int64_t, hipStream_t);
+int gemm_grouped_dispatch(const GemmArgs&, bool, int64_t, int64_t, hipStream_t);
 int gemm_skinny_dispatch(const GemmArgs&, bool, int64_t, hipStream_t);
 int gemm_skinny_max_m();
 
@@ -461,7 +461,51 @@ int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void*
   p.num_active = (int)num_active_experts;
   p.b_expert_stride = N * K;
   p.bs_expert_stride = ceil_div(N, 128) * ceil_div(K, 128);
-  return gemm_grouped_dispatch(p, T, max_num_tokens_per_expert, st);
+  return gemm_grouped_dispatch(p, true, T, max_num_tokens_per_expert, st);
+}
+
+int maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
+                                                     const void* b_scales, const uint32_t* expert_start_indices,
+                                                     const int32_t* expert_ids, int64_t T, int64_t N, int64_t K,
+                                                     int64_t num_experts, int64_t max_num_tokens_per_expert,
+                                                     int64_t num_active_experts, int c_dtype, int scales_dtype, void* stream) {
+  if (c_dtype != MAXFP8_BF16 && c_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "grouped rowwise matmul: output dtype %d is not bf16 or f32", c_dtype);
+  if (scales_dtype != MAXFP8_F32)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "grouped rowwise matmul: A and B scales must be float32 for rowwise/per-token granularity");
+  if (T < 0 || N < 0 || K < 0 || num_experts < 0 || max_num_tokens_per_expert < 0 || num_active_experts < 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped rowwise matmul: negative size");
+  // grouped_matmul.mojo:1675-1676
+  if (max_num_tokens_per_expert == 0 || num_active_experts == 0 || T == 0 || N == 0) return MAXFP8_OK;
+  if (num_active_experts > num_experts)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped rowwise matmul: %lld active slots but expert_ids holds %lld",
+                (long long)num_active_experts, (long long)num_experts);
+  if (T >= ((int64_t)1 << 31) || N >= ((int64_t)1 << 31) || K >= ((int64_t)1 << 31))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped rowwise matmul: sizes must fit 31 bits");
+  if (!c || !a || !b || !a_scales || !b_scales || !expert_start_indices || !expert_ids)
+    MAXFP8_FAIL(MAXFP8_ERR_NULL, "grouped rowwise matmul: null pointer");
+  if (!(is_aligned(a, 16) && is_aligned(b, 16) && K % 16 == 0 && K > 0))
+    MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "grouped rowwise matmul: needs 16-byte aligned rows and K %% 16 == 0");
+  GemmArgs p;
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t*)a;
+  p.b = (const uint8_t*)b;
+  p.c = c;
+  p.a_scales = (const float*)a_scales;  // [T, 1]
+  p.b_scales = (const float*)b_scales;  // [E, N, 1]
+  p.M = (int)T; p.N = (int)N; p.K = (int)K;
+  p.lda = K; p.ldb = K; p.ldc = N;
+  p.a_scale_stride = 1;
+  p.b_scale_stride = 1;
+  p.c_dtype = c_dtype;
+  p.c_vec_ok = (N % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
+  p.c_vec8_ok = (N % 8 == 0) && is_aligned(c, 16);
+  p.offsets = expert_start_indices;
+  p.expert_ids = expert_ids;
+  p.num_active = (int)num_active_experts;
+  p.b_expert_stride = N * K;
+  p.bs_expert_stride = N;
+  return gemm_grouped_dispatch(p, false, T, max_num_tokens_per_expert, (hipStream_t)stream);
 }
 
 int maxfp8_cast_f32_to_e4m3fn(void* out_fp8, const float* in, int64_t n, void* stream) {

@@ -464,8 +464,8 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
           const int n_lo = (n + i < p.N) ? n + i : p.N - 1;
           const int n_hi = (n + 4 + i < p.N) ? n + 4 + i : p.N - 1;
           const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
-          lo[i] = t_lo * p.b_scales[(int64_t)n_lo * p.b_scale_stride];
-          hi[i] = t_hi * p.b_scales[(int64_t)n_hi * p.b_scale_stride];
+          lo[i] = t_lo * bs_ptr[(int64_t)n_lo * p.b_scale_stride];  // (bs_ptr: this expert's scales when grouped)
+          hi[i] = t_hi * bs_ptr[(int64_t)n_hi * p.b_scale_stride];
         }
       }
       store8(m, n, lo, hi);
@@ -556,7 +556,7 @@ __device__ __forceinline__ int grouped_head_rows(const GemmArgs& p, int rows) {
 // The rows the large-tile launch leaves: BM-row tiles, and one SBM-row tile with one more LDS stage
 // for what is at most small_rows (<= SBM) rows (such tiles only stream weights, so what they need is bytes in
 // flight).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS, bool BLOCKSCALE = true>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_grouped_kernel(GemmArgs p) {
   static_assert(WAVES_M * WAVES_N == SWAVES_M * SWAVES_N, "both tile kinds run on the same block");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -580,12 +580,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
   }
   const uint8_t* bptr = p.b + (int64_t)e * p.b_expert_stride;
   const float* bs_ptr = p.b_scales + (int64_t)e * p.bs_expert_stride;
-  if (small) tile_body<SBM, BN, SWAVES_M, SWAVES_N, SNS, true, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
-  else tile_body<BM, BN, WAVES_M, WAVES_N, NS, true, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+  if (small) tile_body<SBM, BN, SWAVES_M, SWAVES_N, SNS, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+  else tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
 }
 
 // The full BM-row tiles (BM == big_bm) of the slots with at least big_rows rows.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE = true>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -599,8 +599,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_k
     grouped_zero_tile<NWAVES * 64>(p, row_begin, BM, n0, BN);
     return;
   }
-  tile_body<BM, BN, WAVES_M, WAVES_N, NS, true, true>(p, smem, row_begin, row_begin + BM, n0, p.b + (int64_t)e * p.b_expert_stride,
-                                                       p.b_scales + (int64_t)e * p.bs_expert_stride);
+  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, true>(p, smem, row_begin, row_begin + BM, n0, p.b + (int64_t)e * p.b_expert_stride,
+                                                             p.b_scales + (int64_t)e * p.bs_expert_stride);
 }
 
 template <int BM, int BN, int NS, bool BLOCKSCALE>
@@ -627,19 +627,19 @@ static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const 
                          tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS, bool BLOCKSCALE = true>
 static int launch_grouped(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
   static bool attr_done = false;
-  constexpr int big = tile_lds_bytes<BM, BN, NS, true>(), small = tile_lds_bytes<SBM, BN, SNS, true>();
-  return launch_with_lds(gemm_grouped_kernel<BM, BN, WAVES_M, WAVES_N, NS, SBM, SWAVES_M, SWAVES_N, SNS>, attr_done,
+  constexpr int big = tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), small = tile_lds_bytes<SBM, BN, SNS, BLOCKSCALE>();
+  return launch_with_lds(gemm_grouped_kernel<BM, BN, WAVES_M, WAVES_N, NS, SBM, SWAVES_M, SWAVES_N, SNS, BLOCKSCALE>, attr_done,
                          big > small ? big : small, WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE = true>
 static int launch_grouped_large(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
   static bool attr_done = false;
-  return launch_with_lds(gemm_grouped_large_kernel<BM, BN, WAVES_M, WAVES_N, NS>, attr_done, tile_lds_bytes<BM, BN, NS, true>(),
-                         WAVES_M * WAVES_N * 64, p, grid, stream, name);
+  return launch_with_lds(gemm_grouped_large_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE>, attr_done,
+                         tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
 
 // Sums the split-K partial results in split order (deterministic), applies the row / tensor
@@ -875,7 +875,7 @@ static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, di
   return launch_tiled<128, 128, 2, 2, 2, false>(p, grid, stream, "gemm_tiled_row_128x128");
 }
 
-int gemm_grouped_dispatch(const GemmArgs& p_in, int64_t T, int64_t max_tokens, hipStream_t stream) {
+int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int64_t max_tokens, hipStream_t stream) {
   GemmArgs p = p_in;
   // Slots with at least 1024 rows (the caller's bound on the largest slot says whether there can
   // be any) hand their full 256-row tiles to a launch with 256 x 256 tiles; everything else --
@@ -888,16 +888,22 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, int64_t T, int64_t max_tokens, h
   p.small_rows = tune == 3 ? 0 : (big ? 64 : 32);
   p.big_rows = 0;
   p.big_bm = 256;
-  if (!big && tune != 4 && max_tokens >= 1024 && T / 256 <= 65535) {
-    p.big_rows = 1024;
+  const int big_rows = getenv("MAXFP8_BIG_ROWS") ? atoi(getenv("MAXFP8_BIG_ROWS")) : 1024;
+  if (!big && tune != 4 && max_tokens >= big_rows && T / 256 <= 65535) {
+    p.big_rows = big_rows;
     const dim3 lgrid((unsigned)ceil_div(p.N, 256), (unsigned)(T / 256));
-    const int rc = launch_grouped_large<256, 256, 2, 4, 2>(p, lgrid, stream, "gemm_grouped_block_256x256");
+    const int rc = blockscale ? launch_grouped_large<256, 256, 2, 4, 2>(p, lgrid, stream, "gemm_grouped_block_256x256")
+                              : launch_grouped_large<256, 256, 2, 4, 2, false>(p, lgrid, stream, "gemm_grouped_row_256x256");
     if (rc != MAXFP8_OK) return rc;
   }
   // a slot owns one small tile or ceil(rows / BM) tiles: their sum is <= T / BM + num_active
   const int64_t m_tiles = T / bm + p.num_active;
   if (m_tiles > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: %lld row tiles exceed the launch limit", (long long)m_tiles);
   const dim3 grid((unsigned)ceil_div(p.N, 128), (unsigned)m_tiles);
+  if (!blockscale) {
+    if (big) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped rowwise matmul: the 256 x 128 shape is not built");
+    return launch_grouped<128, 128, 2, 2, 2, 32, 1, 4, 3, false>(p, grid, stream, "gemm_grouped_row_128x128");
+  }
   if (big) return launch_grouped<256, 128, 4, 2, 3, 64, 2, 4, 3>(p, grid, stream, "gemm_grouped_block_256x128");
   return launch_grouped<128, 128, 2, 2, 2, 32, 1, 4, 3>(p, grid, stream, "gemm_grouped_block_128x128");
 }

@@ -7,6 +7,7 @@ of the reference's graph-op wrappers:
   batched_dynamic_scaled_fp8_matmul   max/python/max/nn/kernels.py:6642-6751
   fused_qkv_ragged_matmul_scaled_float8  max/python/max/nn/kernels.py:582-727
   matmul_k_cache_ragged_scaled_float8    max/python/max/nn/kernels.py:1475-1539
+  grouped_matmul_rowwise_dynamic_scaled_fp8  max/python/max/nn/kernels.py:6490-6640
 
 They take torch tensors that live on the MI355X and call the HIP kernels through
 the C ABI on torch's current stream.  Nothing here computes on the CPU.
@@ -653,6 +654,70 @@ def grouped_dynamic_scaled_fp8_matmul(
         c.data_ptr(), hidden_states.data_ptr(), weight.data_ptr(), a_scales.data_ptr(), b_scales.data_ptr(),
         expert_start_indices.data_ptr(), expert_ids.data_ptr(), T, N, K, E, max_tokens, num_active, a_ld,
         _DT[out_type], _DT[a_scales.dtype], _ALGOS[algo], _stream(hidden_states))
+    _lib.check(st)
+    return c
+
+
+def grouped_matmul_rowwise_dynamic_scaled_fp8(
+    hidden_states: torch.Tensor,
+    weight: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    expert_start_indices: torch.Tensor,
+    expert_ids: torch.Tensor,
+    expert_usage_stats_host: torch.Tensor,
+    out_type: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    """Grouped (ragged MoE) FP8 matmul with per-token activation scales [total_tokens, 1] and
+    per-output-channel weight scales [num_experts, N, 1]:
+    out[t, n] = (sum_k a[t, k] * b[expert_ids[g], n, k]) * a_scale[t] * b_scale[expert_ids[g], n]."""
+    if hidden_states.dim() != 2:
+        raise ValueError(f"expected hidden_states of rank 2 but got {hidden_states.dim()}")
+    if weight.dim() != 3:
+        raise ValueError(f"expected weight of rank 3 but got {weight.dim()}")
+    if weight.shape[2] != hidden_states.shape[1] or weight.shape[0] != expert_ids.shape[0]:
+        raise ValueError(f"expected weight of shape [num_experts, N, {hidden_states.shape[1]}] with num_experts = "
+                         f"{expert_ids.shape[0]} but got {tuple(weight.shape)}")
+    if (hidden_states.dtype != weight.dtype) or (hidden_states.dtype != _FP8):
+        raise TypeError(
+            f"hidden_states and weight dtypes must be float8_e4m3fn, but got {hidden_states.dtype}, {weight.dtype}")
+    if a_scales.dim() != 2 or b_scales.dim() != 3:
+        raise ValueError(
+            f"expected a_scales of rank 2 and b_scales of rank 3 but got {a_scales.dim()} and {b_scales.dim()}")
+    if a_scales.dtype != torch.float32 or b_scales.dtype != torch.float32:
+        raise TypeError("a_scales and b_scales dtypes must both be float32 for rowwise / per-token granularity, "
+                        f"but got {a_scales.dtype}, {b_scales.dtype}")
+    T, K = hidden_states.shape
+    E, N, _ = weight.shape
+    if a_scales.shape[1] != 1 or a_scales.shape[0] < T:
+        raise ValueError(f"expected per-token a_scales of shape [total_tokens, 1] but got {tuple(a_scales.shape)}")
+    if tuple(b_scales.shape) != (E, N, 1):
+        raise ValueError("expected per-channel b_scales of shape [num_experts, N, 1] matching weight [num_experts, N, K], "
+                         f"but got b_scales {tuple(b_scales.shape)} and weight {tuple(weight.shape)}")
+    if expert_ids.dtype != torch.int32:
+        raise TypeError(f"expert_ids dtype must be int32, but got {expert_ids.dtype}")
+    if expert_ids.dim() != 1:
+        raise ValueError(f"expected expert_ids of rank 1 but got {expert_ids.dim()}")
+    if expert_start_indices.dtype != torch.uint32:
+        raise TypeError(f"expert_start_indices dtype must be uint32, but got {expert_start_indices.dtype}")
+    if expert_start_indices.dim() != 1:
+        raise ValueError(f"expected expert_start_indices of rank 1 but got {expert_start_indices.dim()}")
+    if out_type not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"out_type {out_type} is not bfloat16 or float32")
+    stats = expert_usage_stats_host
+    if stats.is_cuda:
+        raise ValueError("expert_usage_stats_host must live on the CPU")
+    max_tokens, num_active = int(stats[0]), int(stats[1])
+    if expert_start_indices.shape[0] < num_active + 1:
+        raise ValueError("expert_start_indices is shorter than num_active_experts + 1")
+    _require_gpu(hidden_states, weight, a_scales, b_scales, expert_start_indices, expert_ids)
+    hidden_states, weight = hidden_states.contiguous(), weight.contiguous()
+    a_scales, b_scales = a_scales.contiguous(), b_scales.contiguous()
+    c = torch.empty((T, N), dtype=out_type, device=hidden_states.device)
+    st = _lib.lib().maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8(
+        c.data_ptr(), hidden_states.data_ptr(), weight.data_ptr(), a_scales.data_ptr(), b_scales.data_ptr(),
+        expert_start_indices.data_ptr(), expert_ids.data_ptr(), T, N, K, E, max_tokens, num_active,
+        _DT[out_type], _lib.F32, _stream(hidden_states))
     _lib.check(st)
     return c
 

@@ -176,6 +176,28 @@ def quantize_tensor_dynamic(x: np.ndarray, *, in_dtype: int = BF16, scales_dtype
     return q.reshape(M, K), np.repeat(sc[:1, :1], M, axis=1)
 
 
+def grouped_matmul_rowwise(a: np.ndarray, b: np.ndarray, a_scales: np.ndarray, b_scales: np.ndarray,
+                           offsets: np.ndarray, expert_ids: np.ndarray, num_active: int, *, c_dtype: int = F32,
+                           threads: int = 1, fill: float = np.nan) -> np.ndarray:
+    """grouped_matmul_rowwise_scaled_fp8_kernel (max/kernels/src/linalg/grouped_matmul.mojo:1440-1541): slot z
+    multiplies its rows by expert expert_ids[z] with matmul_rowwise's arithmetic; expert -1 gives zeros; rows
+    past the last active slot keep `fill`.  a [T, K], b [E, N, K] bytes; a_scales [T, 1], b_scales [E, N, 1]."""
+    T = a.shape[0]
+    E, N, _ = b.shape
+    c = np.full((T, N), fill, dtype=np.float32) if c_dtype == F32 else np.full((T, N), 0xFFFF, dtype=np.uint16)
+    for z in range(num_active):
+        lo, hi = int(offsets[z]), int(offsets[z + 1])
+        if hi <= lo:
+            continue
+        e = int(expert_ids[z])
+        if e < 0:
+            c[lo:hi] = 0
+            continue
+        c[lo:hi] = matmul_rowwise(a[lo:hi], b[e], np.asarray(a_scales, np.float32).reshape(1, -1)[:, lo:hi],
+                                  np.asarray(b_scales, np.float32)[e].reshape(-1, 1), c_dtype=c_dtype, threads=threads)
+    return c
+
+
 def bf16_round(x: np.ndarray) -> np.ndarray:
     """float32 array rounded to bf16 (nearest even; NaN kept) and widened back."""
     u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)

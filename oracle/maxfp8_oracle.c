@@ -29,6 +29,7 @@
  * quantiser and matmul (one 2-D call per batch, fp8_quantization.mojo:779-954, bmm.mojo:1430-1558)
  * and the dynamic per-tensor quantiser (the whole tensor as one group,
  * fp8_quantization.mojo:209-360; checked against the formula of the reference's own test).
+ * oracle.grouped_matmul_rowwise (max/kernels/src/linalg/grouped_matmul.mojo:1440-1541): orc_matmul_rowwise per slot.
  * oracle.fused_qkv_matmul (max/kernels/src/nn/kv_cache_ragged.mojo:1122-1307, page arithmetic of
  * max/kernels/src/kv_cache/types.mojo:2274-2296) is numpy around the matmuls above; pinned by exact
  * integer cases read back through an independent gather and by a float64 matmul.  Parity unpinned:
