@@ -309,6 +309,9 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     }
     buf = buf + 1 == NS ? 0 : buf + 1;
   }
+  // the copies issued for slabs past the end only write zeros, but they write them into LDS: they
+  // must have landed before the stage memory is reused below or handed to the next block
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue -----------------------------------------------------------------------------
   if (partial_out) {
