@@ -288,15 +288,18 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
       if (!SKIP_ROWS || mt < mt_live) {
         v8i af_next = af;
         if (mt + 1 < TM) af_next = read_frag(sa + a_frag_base + (mt + 1) * 2048);
+        if constexpr (BLOCKSCALE) {
+          // the group's MFMAs first, then their promotions: the first product is ready when the last one issues
+          const v4f zero = {0.f, 0.f, 0.f, 0.f};
+          v4f part[TN];
 #pragma unroll
-        for (int nt = 0; nt < TN; ++nt) {
-          if constexpr (BLOCKSCALE) {
-            const v4f zero = {0.f, 0.f, 0.f, 0.f};
-            const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
-            acc[mt][nt] += part * s_cur[mt];
-          } else {
+          for (int nt = 0; nt < TN; ++nt) part[nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+          for (int nt = 0; nt < TN; ++nt) acc[mt][nt] += part[nt] * s_cur[mt];
+        } else {
+#pragma unroll
+          for (int nt = 0; nt < TN; ++nt)
             acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
-          }
         }
         af = af_next;
       }
@@ -344,6 +347,80 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     // rounded to bf16 first, per-tensor / per-channel scales are multiplied in bf16, the bias is
     // added in bf16 (kv_cache_ragged.mojo:1210-1245) -- and goes to C or to the row's K / V page.
     // Columns outside, rows inside: 8 weight scales and 8 bias values live at a time.
+    //
+    // Tiles with all their columns: the finished bf16 values are staged in the wave's 16 KB of stage
+    // memory (as the plain epilogue does) and each row's cache offset is looked up ONCE per wave and
+    // parked in LDS after the staging area (KV kernels are launched with that much more LDS), so
+    // that a store instruction writes 8 rows x one whole 128-byte line to C or to the rows' pages.
+    if constexpr (WN == 64 && WM % 64 == 0) {
+      if (p.c_vec8_ok && n0 + BN <= p.N) {
+        __syncthreads();  // every wave has finished reading the stages
+        uint8_t* wbuf = smem + wave * (WM * WN * 2);
+        int64_t* otab = reinterpret_cast<int64_t*>(smem + NWAVES * (WM * WN * 2) + wave * (WM * 8));
+        {
+          constexpr int R = WM / 64;
+          int64_t rows[R], off[R];
+          bool live[R];
+#pragma unroll
+          for (int j = 0; j < R; ++j) {
+            int r = j * 64 + lane;
+            asm volatile("" : "+v"(r));  // keeps the page lookups here, out of the registers of the main loop
+            rows[j] = row_begin + wm * WM + r;
+            live[j] = wm * WM + r < rows_here;
+          }
+          kv_row_offsets<R>(p.kv, rows, live, off);
+#pragma unroll
+          for (int j = 0; j < R; ++j) otab[j * 64 + lane] = off[j];
+        }
+        static_for<TN / 2>([&](auto qc) {
+          constexpr int q = decltype(qc)::value;
+          const int n = n0 + wn * WN + q * 32 + lq * 8;
+          float b_s[8], bias[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            b_s[i] = 1.f;
+            if constexpr (!BLOCKSCALE) b_s[i] = bf16_round(p.b_scales[(int64_t)(n + i) * p.b_scale_stride]);
+            bias[i] = p.kv.bias ? bf16_bits_to_f32(p.kv.bias[n + i]) : 0.f;
+          }
+#pragma unroll
+          for (int mt = 0; mt < TM; ++mt) {
+            const int r = mt * 16 + lm;
+            float a_s = 1.f;
+            if constexpr (!BLOCKSCALE) {
+              const int64_t mm = row_begin + wm * WM + r;
+              a_s = bf16_round(p.a_scales[(mm < p.M ? mm : p.M - 1) * p.a_scale_stride]);
+            }
+            const v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
+            const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+              if constexpr (!BLOCKSCALE) {
+                const uint32_t sc = pack_bf16x2(a_s * b_s[2 * i], a_s * b_s[2 * i + 1]);
+                w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) * __uint_as_float(sc << 16),
+                                   __uint_as_float(w[i] & 0xffff0000u) * __uint_as_float(sc & 0xffff0000u));
+              }
+              if (p.kv.bias)
+                w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) + bias[2 * i], __uint_as_float(w[i] & 0xffff0000u) + bias[2 * i + 1]);
+            }
+            *reinterpret_cast<uint4*>(wbuf + r * (WN * 2) + (((q * 4 + lq) ^ (r & 7)) * 16)) = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+        });
+        // (a wave reads back only what it wrote itself; LDS operations of a wave execute in order)
+        const int rr = lane >> 3, cc = lane & 7;
+        const int n = n0 + wn * WN + cc * 8;
+#pragma unroll
+        for (int i = 0; i < WM / 8; ++i) {
+          const int r = i * 8 + rr;
+          const uint4 v = *reinterpret_cast<const uint4*>(wbuf + r * (WN * 2) + ((cc ^ (r & 7)) * 16));
+          const int64_t off = otab[r];
+          if (wm * WM + r < rows_here && !(off < 0 && n >= p.kv.q_dim))
+            *reinterpret_cast<uint4*>(kv_dst(p.kv, p.c, p.ldc, row_begin + wm * WM + r, off, n)) = v;
+        }
+        return;
+      }
+    }
     float a_s[TM];
     int64_t row_off[TM], rows[TM];
     bool live[TM];
@@ -626,8 +703,10 @@ static int launch_with_lds(Kern kern, bool& attr_done, int smem, int threads, co
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool KV = false>
 static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
   static bool attr_done = false;
+  // (fused QKV: 8 more bytes per tile row for the rows' cache offsets, after the 2 * BM * BN bytes of staged output)
+  constexpr int stages = tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), kv = 2 * BM * BN + 8 * BM * WAVES_N;
   return launch_with_lds(gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, KV>, attr_done,
-                         tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), WAVES_M * WAVES_N * 64, p, grid, stream, name);
+                         KV && kv > stages ? kv : stages, WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS, bool BLOCKSCALE = true>
