@@ -281,6 +281,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
 #pragma unroll
     for (int t = 0; t < TN; ++t) bf[t] = read_wfrag(sa + b_frag_base, t);
     v8i af = read_frag(sa + a_frag_base);
+    [[maybe_unused]] v4f part[2][TN];  // block scaling: products of the current and of the previous 16-row group
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) {
       // 16-row groups past the end of a short tile (an expert with few tokens) are skipped:
@@ -289,13 +290,25 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
         v8i af_next = af;
         if (mt + 1 < TM) af_next = read_frag(sa + a_frag_base + (mt + 1) * 2048);
         if constexpr (BLOCKSCALE) {
-          // the group's MFMAs first, then their promotions: the first product is ready when the last one issues
+          // the group's MFMAs first, then the promotions of the PREVIOUS group: the matrix pipe works on
+          // this group while the VALU folds the last one in
           const v4f zero = {0.f, 0.f, 0.f, 0.f};
-          v4f part[TN];
 #pragma unroll
-          for (int nt = 0; nt < TN; ++nt) part[nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
+          for (int nt = 0; nt < TN; ++nt)
+            part[mt & 1][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
+          if constexpr (!SKIP_ROWS) {
+            if (mt > 0) {
 #pragma unroll
-          for (int nt = 0; nt < TN; ++nt) acc[mt][nt] += part[nt] * s_cur[mt];
+              for (int nt = 0; nt < TN; ++nt) acc[mt - 1][nt] += part[(mt - 1) & 1][nt] * s_cur[mt - 1];
+            }
+            if (mt == TM - 1) {
+#pragma unroll
+              for (int nt = 0; nt < TN; ++nt) acc[mt][nt] += part[mt & 1][nt] * s_cur[mt];
+            }
+          } else {
+#pragma unroll
+            for (int nt = 0; nt < TN; ++nt) acc[mt][nt] += part[mt & 1][nt] * s_cur[mt];
+          }
         } else {
 #pragma unroll
           for (int nt = 0; nt < TN; ++nt)
