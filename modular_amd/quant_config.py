@@ -45,24 +45,17 @@ class QuantFormat(Enum):
     BLOCKSCALED_FP8 = "blockscaled-fp8"
 
 
+def _is(kind: "ScaleGranularity"):
+    return property(lambda self: self.granularity is kind)
+
+
 class _GranularityProps:
+    """is_tensor / is_rowwise / is_colwise / is_block of a spec."""
     granularity: ScaleGranularity
-
-    @property
-    def is_tensor(self) -> bool:
-        return self.granularity == ScaleGranularity.TENSOR
-
-    @property
-    def is_rowwise(self) -> bool:
-        return self.granularity == ScaleGranularity.ROWWISE
-
-    @property
-    def is_colwise(self) -> bool:
-        return self.granularity == ScaleGranularity.COLWISE
-
-    @property
-    def is_block(self) -> bool:
-        return self.granularity == ScaleGranularity.BLOCK
+    is_tensor = _is(ScaleGranularity.TENSOR)
+    is_rowwise = _is(ScaleGranularity.ROWWISE)
+    is_colwise = _is(ScaleGranularity.COLWISE)
+    is_block = _is(ScaleGranularity.BLOCK)
 
 
 def _check_block(granularity: ScaleGranularity, block_size) -> None:
@@ -109,24 +102,19 @@ class QuantConfig:
     def scales_granularity_mnk(self) -> tuple[int, int, int]:
         """(m, n, k) granularities; -1 = one scale along that axis
         (quant_config.py:313-351)."""
-        if self.input_scale.is_block:
-            assert self.input_scale.block_size is not None
-            m_g, k_in = self.input_scale.block_size
-        elif self.input_scale.is_colwise:
-            m_g, k_in = 1, -1
-        elif self.input_scale.is_tensor:
-            m_g, k_in = -1, -1
-        else:
-            raise ValueError("unsupported input scale granularity")
-        if self.weight_scale.is_block:
-            assert self.weight_scale.block_size is not None
-            n_g, k_w = self.weight_scale.block_size
-        elif self.weight_scale.is_rowwise:
-            n_g, k_w = 1, -1
-        elif self.weight_scale.is_tensor:
-            n_g, k_w = -1, -1
-        else:
-            raise ValueError("unsupported weight scale granularity")
+        def axes(spec, single, what):
+            # (granularity along the spec's own axis, granularity along K); -1 = one scale for the axis
+            if spec.is_block:
+                assert spec.block_size is not None
+                return tuple(spec.block_size)
+            if getattr(spec, single):
+                return (1, -1)
+            if spec.is_tensor:
+                return (-1, -1)
+            raise ValueError(f"unsupported {what} scale granularity")
+
+        m_g, k_in = axes(self.input_scale, "is_colwise", "input")
+        n_g, k_w = axes(self.weight_scale, "is_rowwise", "weight")
         assert k_in == k_w, "k_input_granularity and k_weight_granularity must be the same"
         return (m_g, n_g, k_in)
 
