@@ -13,6 +13,7 @@ from .kernels import (grouped_matmul_rowwise_dynamic_scaled_fp8, fused_qkv_ragge
                       quantize_static_scaled_float8, quantize_tensor_dynamic_scaled_float8,
                       quantize_dynamic_scaled_float8, rms_norm_fused_quantize_dynamic_scaled_fp8)
 from .moe_kernels import fused_silu, fused_silu_quantized, moe_create_indices
+from .moe import expert_matmuls_fp8
 from .quant_ops import matmul_float8, quantized_fused_qkv_matmul, quantized_matmul
 from .linear import Linear
 from .weights_quant import parse_quant_config
@@ -26,5 +27,5 @@ __all__ = [
     "quantize_static_scaled_float8", "matmul_static_scaled_float8", "parse_quant_config",
     "batched_dynamic_scaled_fp8_matmul", "batched_quantize_dynamic_scaled_fp8",
     "quantize_tensor_dynamic_scaled_float8", "fused_qkv_ragged_matmul_scaled_float8",
-    "matmul_k_cache_ragged_scaled_float8", "KVCacheParams", "PagedCacheValues", "quantized_fused_qkv_matmul", "grouped_matmul_rowwise_dynamic_scaled_fp8",
+    "matmul_k_cache_ragged_scaled_float8", "KVCacheParams", "PagedCacheValues", "quantized_fused_qkv_matmul", "grouped_matmul_rowwise_dynamic_scaled_fp8", "expert_matmuls_fp8",
 ]

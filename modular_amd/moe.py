@@ -1,0 +1,56 @@
+"""The expert matmuls of a block-scaled FP8 MoE layer, in the order of the reference's
+`_expert_matmuls` (max/python/max/nn/moe/moe_fp8.py:487-616, FP8 block-scaled strategy):
+
+    group the (token, expert) assignments by expert      moe_create_indices
+    gather the tokens into that order                    (an index_select: plumbing)
+    quantise 1 x 128                                     quantize_dynamic_scaled_float8
+    gate_up = grouped matmul                             grouped_dynamic_scaled_fp8_matmul
+    silu(gate) * up on the rows in use                   fused_silu
+    quantise 1 x 128, down = grouped matmul
+    put the rows back into (token, k) order              (an index_select)
+
+Every step with arithmetic in it is one of this package's HIP kernels."""
+from __future__ import annotations
+
+import torch
+
+from .kernels import grouped_dynamic_scaled_fp8_matmul, quantize_dynamic_scaled_float8
+from .moe_kernels import fused_silu, moe_create_indices
+from .quant_config import QuantConfig
+
+
+def expert_matmuls_fp8(
+    x: torch.Tensor,
+    router_idx: torch.Tensor,
+    gate_up_proj: torch.Tensor,
+    gate_up_proj_scales: torch.Tensor,
+    down_proj: torch.Tensor,
+    down_proj_scales: torch.Tensor,
+    quant_config: QuantConfig,
+) -> torch.Tensor:
+    """x [seq, hidden] bf16; router_idx [seq, k] expert ids; gate_up_proj [E, 2 * I, hidden] and
+    down_proj [E, hidden, I] e4m3fn with 128 x 128 block scales.  Returns the experts' outputs
+    [seq, k, hidden] (bf16), before the router weights are applied."""
+    if x.dim() != 2 or router_idx.dim() != 2 or router_idx.shape[0] != x.shape[0]:
+        raise ValueError("expected x [seq, hidden] and router_idx [seq, k]")
+    if not (quant_config.input_scale.is_block and quant_config.weight_scale.is_block):
+        raise ValueError("the FP8 MoE path of this package is the block-scaled one")
+    seq_len, top_k = router_idx.shape
+    num_experts = gate_up_proj.shape[0]
+    token_order, expert_start, restore_order, expert_ids, usage_stats = moe_create_indices(
+        router_idx.reshape(-1).to(torch.int32), num_experts)
+    permuted = x.index_select(0, (token_order.to(torch.int64) // top_k))
+    stats_host = usage_stats.cpu()  # [most tokens on one expert, active experts]: the op's two host scalars
+
+    def quantise(t: torch.Tensor):
+        return quantize_dynamic_scaled_float8(t, quant_config.input_scale, quant_config.weight_scale,
+                                              scales_type=torch.float32, group_size_or_per_token=128)
+
+    def grouped(t_q, t_s, weight, weight_scales):
+        return grouped_dynamic_scaled_fp8_matmul(t_q, weight, t_s, weight_scales, expert_start, expert_ids, stats_host,
+                                                 quant_config.input_scale, quant_config.weight_scale)
+
+    gate_up = grouped(*quantise(permuted), gate_up_proj, gate_up_proj_scales)
+    act = fused_silu(gate_up, expert_start)
+    down = grouped(*quantise(act), down_proj, down_proj_scales)
+    return down.index_select(0, restore_order.to(torch.int64)).reshape(seq_len, top_k, down.shape[-1])
