@@ -93,6 +93,19 @@ int maxfp8_quantize_dynamic_scaled_fp8(
     int in_dtype, int scales_dtype, float scale_ub, void* stream);
 
 /*
+ * The same with a row gather in front: output row r is quantised from input row
+ * row_index[r] / index_div.  The FFI form of the fused input the reference's op takes
+ * (FusedInputTensor, builtin_kernels/quantization.mojo:1376-1390): the MoE layer quantises
+ * x gathered by token_expert_order / top_k (max/python/max/nn/moe/moe_fp8.py:525-560)
+ * without materialising the gathered copy.  row_index is a device array of M uint32.
+ */
+int maxfp8_quantize_dynamic_scaled_fp8_gather(
+    void* out_fp8, void* out_scales, const void* in, const uint32_t* row_index, int64_t index_div,
+    int64_t M, int64_t K, int64_t in_row_stride, int64_t out_row_stride,
+    int64_t group_size, int64_t scales_ld,
+    int in_dtype, int scales_dtype, float scale_ub, void* stream);
+
+/*
  * Batched dynamic activation quantisation: B independent [M, K] problems in one
  * launch.  Replaces batched_quantize_dynamic_scaled_fp8
  *   (max/kernels/src/linalg/fp8_quantization.mojo:779-954), which the MLA
@@ -261,6 +274,21 @@ int maxfp8_fused_qkv_matmul_ragged_paged_scale(
  */
 int maxfp8_grouped_matmul_dynamic_scaled_fp8(
     void* c, const void* a, const void* b,
+    const void* a_scales, const void* b_scales,
+    const uint32_t* expert_start_indices, const int32_t* expert_ids,
+    int64_t T, int64_t N, int64_t K, int64_t num_experts,
+    int64_t max_num_tokens_per_expert, int64_t num_active_experts,
+    int64_t a_scales_ld, int c_dtype, int scales_dtype, int algo, void* stream);
+
+/*
+ * maxfp8_grouped_matmul_dynamic_scaled_fp8 with a row scatter behind it: row m of the result
+ * is stored at row c_row_index[m] of c (a device array of T uint32, every row of c written at
+ * most once).  The FFI form of the op's output lambda: the MoE layer puts the rows of the down
+ * projection back into (token, k) order -- c_row_index = token_expert_order --
+ * (moe_fp8.py:614-616) without a second pass.  MFMA kernel only.
+ */
+int maxfp8_grouped_matmul_dynamic_scaled_fp8_scatter(
+    void* c, const uint32_t* c_row_index, const void* a, const void* b,
     const void* a_scales, const void* b_scales,
     const uint32_t* expert_start_indices, const int32_t* expert_ids,
     int64_t T, int64_t N, int64_t K, int64_t num_experts,

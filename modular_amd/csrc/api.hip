@@ -24,7 +24,7 @@ int launch_status(const char* what) {
 
 // kernels (defined in the other translation units)
 int quantize_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, int,
-                      float, int64_t, int64_t, int64_t, int64_t, hipStream_t);
+                      float, int64_t, int64_t, int64_t, int64_t, const uint32_t*, uint32_t, hipStream_t);
 int rmsnorm_quantize_dispatch(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float,
                               float, float, hipStream_t);
 int quantize_static_dispatch(void*, const void*, int64_t, int64_t, int64_t, int64_t, int, float, hipStream_t);
@@ -76,10 +76,11 @@ extern "C" {
 const char* maxfp8_last_error(void) { return g_error; }
 const char* maxfp8_version(void) { return "maxfp8 0.1 (gfx950)"; }
 
-int maxfp8_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, int64_t M, int64_t K,
-                                       int64_t in_row_stride, int64_t out_row_stride, int64_t group_size,
-                                       int64_t scales_ld, int in_dtype, int scales_dtype, float scale_ub,
-                                       void* stream) {
+}  // extern "C"
+
+static int quantize_common(void* out_fp8, void* out_scales, const void* in, const uint32_t* row_index, uint32_t index_div,
+                           int64_t M, int64_t K, int64_t in_row_stride, int64_t out_row_stride, int64_t group_size,
+                           int64_t scales_ld, int in_dtype, int scales_dtype, float scale_ub, void* stream) {
   if (in_dtype != MAXFP8_BF16 && in_dtype != MAXFP8_F16 && in_dtype != MAXFP8_F32)
     MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize: input dtype %d is not bf16, f16 or f32", in_dtype);
   if (scales_dtype != MAXFP8_F32 && scales_dtype != MAXFP8_BF16)
@@ -96,7 +97,27 @@ int maxfp8_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const vo
                 (long long)in_row_stride, (long long)out_row_stride, (long long)scales_ld);
   if (!out_fp8 || !out_scales || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize: null pointer");
   return quantize_dispatch(out_fp8, out_scales, in, M, K, in_row_stride, out_row_stride, group_size, scales_ld,
-                           in_dtype, scales_dtype, scale_ub, 1, 0, 0, 0, (hipStream_t)stream);
+                           in_dtype, scales_dtype, scale_ub, 1, 0, 0, 0, row_index, index_div, (hipStream_t)stream);
+}
+
+extern "C" {
+
+int maxfp8_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, int64_t M, int64_t K,
+                                       int64_t in_row_stride, int64_t out_row_stride, int64_t group_size,
+                                       int64_t scales_ld, int in_dtype, int scales_dtype, float scale_ub,
+                                       void* stream) {
+  return quantize_common(out_fp8, out_scales, in, nullptr, 1, M, K, in_row_stride, out_row_stride, group_size, scales_ld,
+                         in_dtype, scales_dtype, scale_ub, stream);
+}
+
+int maxfp8_quantize_dynamic_scaled_fp8_gather(void* out_fp8, void* out_scales, const void* in, const uint32_t* row_index,
+                                              int64_t index_div, int64_t M, int64_t K, int64_t in_row_stride,
+                                              int64_t out_row_stride, int64_t group_size, int64_t scales_ld, int in_dtype,
+                                              int scales_dtype, float scale_ub, void* stream) {
+  if (M > 0 && K > 0 && !row_index) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize (gather): null row index");
+  if (index_div < 1 || index_div > 0xffffffffll) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize (gather): index_div must be at least 1");
+  return quantize_common(out_fp8, out_scales, in, row_index, (uint32_t)index_div, M, K, in_row_stride, out_row_stride,
+                         group_size, scales_ld, in_dtype, scales_dtype, scale_ub, stream);
 }
 
 int maxfp8_batched_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, int64_t B, int64_t M, int64_t K,
@@ -122,7 +143,7 @@ int maxfp8_batched_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, 
     MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: strides smaller than the extents");
   if (!out_fp8 || !out_scales || !in) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize: null pointer");
   return quantize_dispatch(out_fp8, out_scales, in, M, K, in_row_stride, out_row_stride, group_size, scales_ld, in_dtype,
-                           scales_dtype, scale_ub, B, in_batch_stride, out_batch_stride, scales_batch_stride,
+                           scales_dtype, scale_ub, B, in_batch_stride, out_batch_stride, scales_batch_stride, nullptr, 1,
                            (hipStream_t)stream);
 }
 
@@ -410,12 +431,13 @@ int maxfp8_fused_qkv_matmul_ragged_paged_scale(void* output, const void* input, 
   return gemm_tiled_dispatch(p, block, 0, 1, st);
 }
 
-int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
-                                             const void* b_scales, const uint32_t* expert_start_indices,
-                                             const int32_t* expert_ids, int64_t T, int64_t N, int64_t K,
-                                             int64_t num_experts, int64_t max_num_tokens_per_expert,
-                                             int64_t num_active_experts, int64_t a_scales_ld, int c_dtype,
-                                             int scales_dtype, int algo, void* stream) {
+}  // extern "C"
+
+static int grouped_block_common(void* c, const uint32_t* c_row_index, const void* a, const void* b, const void* a_scales,
+                                const void* b_scales, const uint32_t* expert_start_indices, const int32_t* expert_ids,
+                                int64_t T, int64_t N, int64_t K, int64_t num_experts, int64_t max_num_tokens_per_expert,
+                                int64_t num_active_experts, int64_t a_scales_ld, int c_dtype, int scales_dtype, int algo,
+                                void* stream) {
   if (c_dtype != MAXFP8_BF16 && c_dtype != MAXFP8_F32)
     MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "grouped matmul: output dtype %d is not bf16 or f32", c_dtype);
   if (scales_dtype != MAXFP8_F32)
@@ -436,6 +458,8 @@ int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void*
   hipStream_t st = (hipStream_t)stream;
   const bool fast_layout = is_aligned(a, 16) && is_aligned(b, 16) && K % 16 == 0 && K > 0;
   if (algo == MAXFP8_ALGO_AUTO) algo = fast_layout ? MAXFP8_ALGO_TILED : MAXFP8_ALGO_NAIVE;
+  if (algo == MAXFP8_ALGO_NAIVE && c_row_index)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: the row scatter needs the MFMA kernel (16-byte aligned rows, K %% 16 == 0)");
   if (algo == MAXFP8_ALGO_NAIVE)
     return naive_grouped_dispatch(c, a, b, a_scales, b_scales, expert_start_indices, expert_ids, N, K,
                                   max_num_tokens_per_expert, num_active_experts, a_scales_ld, c_dtype, st);
@@ -461,7 +485,32 @@ int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void*
   p.num_active = (int)num_active_experts;
   p.b_expert_stride = N * K;
   p.bs_expert_stride = ceil_div(N, 128) * ceil_div(K, 128);
+  p.c_row_index = c_row_index;
   return gemm_grouped_dispatch(p, true, T, max_num_tokens_per_expert, st);
+}
+
+extern "C" {
+
+int maxfp8_grouped_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,
+                                             const void* b_scales, const uint32_t* expert_start_indices,
+                                             const int32_t* expert_ids, int64_t T, int64_t N, int64_t K,
+                                             int64_t num_experts, int64_t max_num_tokens_per_expert,
+                                             int64_t num_active_experts, int64_t a_scales_ld, int c_dtype,
+                                             int scales_dtype, int algo, void* stream) {
+  return grouped_block_common(c, nullptr, a, b, a_scales, b_scales, expert_start_indices, expert_ids, T, N, K, num_experts,
+                              max_num_tokens_per_expert, num_active_experts, a_scales_ld, c_dtype, scales_dtype, algo, stream);
+}
+
+int maxfp8_grouped_matmul_dynamic_scaled_fp8_scatter(void* c, const uint32_t* c_row_index, const void* a, const void* b,
+                                                     const void* a_scales, const void* b_scales,
+                                                     const uint32_t* expert_start_indices, const int32_t* expert_ids,
+                                                     int64_t T, int64_t N, int64_t K, int64_t num_experts,
+                                                     int64_t max_num_tokens_per_expert, int64_t num_active_experts,
+                                                     int64_t a_scales_ld, int c_dtype, int scales_dtype, int algo,
+                                                     void* stream) {
+  if (T > 0 && N > 0 && !c_row_index) MAXFP8_FAIL(MAXFP8_ERR_NULL, "grouped matmul (scatter): null row index");
+  return grouped_block_common(c, c_row_index, a, b, a_scales, b_scales, expert_start_indices, expert_ids, T, N, K, num_experts,
+                              max_num_tokens_per_expert, num_active_experts, a_scales_ld, c_dtype, scales_dtype, algo, stream);
 }
 
 int maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,

@@ -46,6 +46,7 @@ struct GemmArgs {
   int big_rows, big_bm;      // slots with at least big_rows rows give their full big_bm-row tiles to the large-tile launch (0: none)
   int64_t b_expert_stride;   // bytes between experts in b
   int64_t bs_expert_stride;  // elements between experts in b_scales
+  const uint32_t* c_row_index;  // grouped only, optional: row m of the result is stored at row c_row_index[m] of c
   // batched only: blockIdx.z (tiled) / blockIdx.y (skinny) steps the five base pointers, in elements
   int64_t a_batch, b_batch, c_batch, a_scales_batch, b_scales_batch;
   // split-K / skinny only

@@ -544,6 +544,9 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     const int ml = wm * WM + mt * 16 + lm;
     if (ml >= rows_here) continue;
     const int64_t m = row_begin + ml;
+    int64_t cm = m;  // the row of C that receives row m
+    if constexpr (GROUPED)
+      if (p.c_row_index) cm = p.c_row_index[m];
     float a_s = 1.f;
     if constexpr (!BLOCKSCALE) a_s = p.a_scales[m * p.a_scale_stride];
 #pragma unroll
@@ -561,7 +564,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
           hi[i] = t_hi * bs_ptr[(int64_t)n_hi * p.b_scale_stride];
         }
       }
-      store8(m, n, lo, hi);
+      store8(cm, n, lo, hi);
     }
   }
 }
@@ -633,7 +636,8 @@ template <int NTHREADS>
 __device__ __forceinline__ void grouped_zero_tile(const GemmArgs& p, int64_t row_begin, int rows_here, int n0, int bn) {
   const int cols_here = (p.N - n0) < bn ? (p.N - n0) : bn;
   for (int i = threadIdx.x; i < rows_here * cols_here; i += NTHREADS) {
-    const int64_t m = row_begin + i / cols_here;
+    int64_t m = row_begin + i / cols_here;
+    if (p.c_row_index) m = p.c_row_index[m];
     const int n = n0 + i % cols_here;
     if (p.c_dtype == MAXFP8_BF16) reinterpret_cast<uint16_t*>(p.c)[m * p.ldc + n] = 0;
     else reinterpret_cast<float*>(p.c)[m * p.ldc + n] = 0.f;

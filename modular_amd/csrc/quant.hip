@@ -25,13 +25,15 @@ namespace maxfp8 {
 
 // Batched launches (blockIdx.y = batch) step the three base pointers by these element counts.
 struct BatchStep { int64_t in, out, scales; };
+// Optional row gather: output row r is quantised from input row index[r] / div (index == nullptr: row r).
+struct RowGather { const uint32_t* index; uint32_t div; };
 
 // ---------------------------------------------------------------------------
 template <int U>
 __global__ __launch_bounds__(256) void quant_g128_bf16_kernel(
     uint8_t* __restrict__ out, float* __restrict__ scales, const uint16_t* __restrict__ in,
     int M, int ngroups, int nxb, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
-    float scale_ub, BatchStep bs) {
+    float scale_ub, BatchStep bs, RowGather rg) {
   in += blockIdx.y * bs.in;
   out += blockIdx.y * bs.out;
   scales += blockIdx.y * bs.scales;
@@ -42,13 +44,14 @@ __global__ __launch_bounds__(256) void quant_g128_bf16_kernel(
   // Each wave owns 4 rows (one per 16-lane segment) and the block's U consecutive groups.
   const int gbase = xb * U;
   const bool row_ok = row < M;
+  const int64_t src_row = (rg.index && row_ok) ? (int64_t)(rg.index[row] / rg.div) : row;
 
   uint4 v[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int g = gbase + u;
     if (row_ok && g < ngroups)
-      v[u] = *reinterpret_cast<const uint4*>(in + (int64_t)row * in_stride + (int64_t)g * 128 + sl * 8);
+      v[u] = *reinterpret_cast<const uint4*>(in + src_row * in_stride + (int64_t)g * 128 + sl * 8);
     else
       v[u] = make_uint4(0, 0, 0, 0);
   }
@@ -89,13 +92,13 @@ __global__ __launch_bounds__(256) void quant_g128_bf16_kernel(
 template <int NV>
 __global__ __launch_bounds__(256) void quant_row_bf16_kernel(
     uint8_t* __restrict__ out, float* __restrict__ scales, const uint16_t* __restrict__ in,
-    int K, int64_t in_stride, int64_t out_stride, float scale_ub, BatchStep bs) {
+    int K, int64_t in_stride, int64_t out_stride, float scale_ub, BatchStep bs, RowGather rg) {
   in += blockIdx.y * bs.in;
   out += blockIdx.y * bs.out;
   scales += blockIdx.y * bs.scales;
   __shared__ float red[4];
   const int row = blockIdx.x, tid = threadIdx.x;
-  const uint16_t* src = in + (int64_t)row * in_stride;
+  const uint16_t* src = in + (rg.index ? (int64_t)(rg.index[row] / rg.div) : (int64_t)row) * in_stride;
   const int nvec = K >> 3;
   uint4 v[NV];
 #pragma unroll
@@ -167,14 +170,14 @@ __device__ __forceinline__ float guarded_recip(float scale) {
 __global__ __launch_bounds__(256) void quant_generic_kernel(
     uint8_t* __restrict__ out, void* __restrict__ scales, const void* __restrict__ in,
     int ngroups, int G, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
-    int in_dtype, int scales_dtype, float scale_ub, BatchStep bs) {
+    int in_dtype, int scales_dtype, float scale_ub, BatchStep bs, RowGather rg) {
   in = reinterpret_cast<const uint8_t*>(in) + blockIdx.y * bs.in * (in_dtype == MAXFP8_F32 ? 4 : 2);
   out += blockIdx.y * bs.out;
   scales = reinterpret_cast<uint8_t*>(scales) + blockIdx.y * bs.scales * (scales_dtype == MAXFP8_F32 ? 4 : 2);
   __shared__ float red[4];
   const int row = blockIdx.x / ngroups, g = blockIdx.x - row * ngroups;
   const int tid = threadIdx.x;
-  const int64_t base = (int64_t)row * in_stride + (int64_t)g * G;
+  const int64_t base = (rg.index ? (int64_t)(rg.index[row] / rg.div) : (int64_t)row) * in_stride + (int64_t)g * G;
   float amax = 0.0f;
   for (int i = tid; i < G; i += 256) amax = fmaxf(amax, fabsf(load_elem(in, in_dtype, base + i)));
   amax = wave_max(amax);
@@ -463,8 +466,10 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M, int64_t K,
                       int64_t in_row_stride, int64_t out_row_stride, int64_t G, int64_t scales_ld,
                       int in_dtype, int scales_dtype, float scale_ub, int64_t batch, int64_t in_batch_stride,
-                      int64_t out_batch_stride, int64_t scales_batch_stride, hipStream_t stream) {
+                      int64_t out_batch_stride, int64_t scales_batch_stride, const uint32_t* row_index, uint32_t index_div,
+                      hipStream_t stream) {
   const BatchStep bs = {in_batch_stride, out_batch_stride, scales_batch_stride};
+  const RowGather rg = {row_index, index_div ? index_div : 1u};
   const unsigned nb = (unsigned)batch;
   const int64_t ngroups = K / G;
   const bool fast_types = in_dtype == MAXFP8_BF16 && scales_dtype == MAXFP8_F32;
@@ -477,7 +482,7 @@ int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M
     if (blocks < (int64_t)1 << 31) {
       hipLaunchKernelGGL(quant_g128_bf16_kernel<U>, dim3((unsigned)blocks, nb), dim3(256), 0, stream,
                          (uint8_t*)out_fp8, (float*)out_scales, (const uint16_t*)in, (int)M, (int)ngroups,
-                         (int)nxb, in_row_stride, out_row_stride, scales_ld, scale_ub, bs);
+                         (int)nxb, in_row_stride, out_row_stride, scales_ld, scale_ub, bs, rg);
       return launch_status("quant_g128_bf16");
     }
   }
@@ -489,7 +494,7 @@ int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M
     const uint16_t* x = (const uint16_t*)in;
 #define LAUNCH_ROW(NV)                                                                            \
   hipLaunchKernelGGL(quant_row_bf16_kernel<NV>, dim3((unsigned)M, nb), dim3(256), 0, stream, o, s, x, \
-                     (int)K, in_row_stride, out_row_stride, scale_ub, bs)
+                     (int)K, in_row_stride, out_row_stride, scale_ub, bs, rg)
     if (nv <= 1) LAUNCH_ROW(1);
     else if (nv <= 2) LAUNCH_ROW(2);
     else if (nv <= 4) LAUNCH_ROW(4);
@@ -502,7 +507,7 @@ int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M
   if (blocks >= (int64_t)1 << 31) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize: M * K/group_size = %lld exceeds the grid limit", (long long)blocks);
   hipLaunchKernelGGL(quant_generic_kernel, dim3((unsigned)blocks, nb), dim3(256), 0, stream, (uint8_t*)out_fp8,
                      out_scales, in, (int)ngroups, (int)G, in_row_stride, out_row_stride, scales_ld, in_dtype,
-                     scales_dtype, scale_ub, bs);
+                     scales_dtype, scale_ub, bs, rg);
   return launch_status("quant_generic");
 }
 

@@ -66,12 +66,20 @@ def quantize_dynamic_scaled_float8(
     group_size_or_per_token: int = -1,
     out_type: torch.dtype = _FP8,
     scales_type: torch.dtype = torch.bfloat16,
+    *,
+    row_index: torch.Tensor | None = None,
+    index_div: int = 1,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """Dynamically quantize `input` [M, K] to fp8.
 
     Returns (quantized [M, K] e4m3fn, scales [K / group, M_pad]) where, for block
     specs, M_pad rounds M up to a multiple of 16 bytes / sizeof(scale); the padding
     columns are allocated but never written.
+
+    With `row_index` (uint32 [R] on the device) the result has R rows and row r is
+    quantised from `input[row_index[r] // index_div]`: the gather that the reference's
+    graph compiler fuses into the op's input (builtin_kernels/quantization.mojo:1376-1390),
+    e.g. `row_index=token_expert_order, index_div=top_k` in the MoE layer.
     """
     if input.dim() != 2:
         raise ValueError("input must be rank 2 tensor")
@@ -79,6 +87,12 @@ def quantize_dynamic_scaled_float8(
         # e4m3fnuz is only ever requested on gfx94x (kernels.py:8408-8417)
         raise ValueError("out_type must be float8_e4m3fn or float8_e4m3fnuz")
     M, K = input.shape
+    if row_index is not None:
+        if row_index.dtype != torch.uint32 or row_index.dim() != 1:
+            raise TypeError("row_index must be a rank 1 uint32 tensor")
+        if index_div < 1:
+            raise ValueError("index_div must be positive")
+        src_rows, M = M, row_index.shape[0]
 
     group_size, a_scales_dim1 = quantize_output_geometry(
         M, K, input_scale_spec, weight_scale_spec, group_size_or_per_token, scales_type)
@@ -95,6 +109,14 @@ def quantize_dynamic_scaled_float8(
         input = input.contiguous()
     out = torch.empty((M, K), dtype=_FP8, device=input.device)
     scales = torch.empty((K // group_size, a_scales_dim1), dtype=scales_type, device=input.device)
+    if row_index is not None:
+        _require_gpu(row_index)
+        st = _lib.lib().maxfp8_quantize_dynamic_scaled_fp8_gather(
+            out.data_ptr(), scales.data_ptr(), input.data_ptr(), row_index.data_ptr(), index_div, M, K,
+            input.stride(0) if src_rows > 1 else K, K,
+            group_size, a_scales_dim1, _DT[input.dtype], _DT[scales_type], float(scale_ub), _stream(input))
+        _lib.check(st)
+        return out, scales
     st = _lib.lib().maxfp8_quantize_dynamic_scaled_fp8(
         out.data_ptr(), scales.data_ptr(), input.data_ptr(), M, K, input.stride(0) if M > 1 else K, K,
         group_size, a_scales_dim1, _DT[input.dtype], _DT[scales_type], float(scale_ub), _stream(input))
@@ -587,11 +609,17 @@ def grouped_dynamic_scaled_fp8_matmul(
     out_type: torch.dtype = torch.bfloat16,
     *,
     algo: str = "auto",
+    out_row_index: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Grouped blockwise scaled matmul of the MoE layer: rows of `hidden_states`
     are sorted by expert, `expert_start_indices` delimits the groups,
     `expert_usage_stats_host` = [max tokens of any expert, number of active experts]
-    on the CPU."""
+    on the CPU.
+
+    With `out_row_index` (uint32 [T], a permutation) row m of the result lands in row
+    `out_row_index[m]` of the returned tensor: the scatter that puts the down projection
+    back into token order (max/python/max/nn/moe/moe_fp8.py:614-616) fused into the
+    matmul's store, as the reference's compiler does with the op's output lambda."""
     if weight.dim() != 3:
         raise ValueError(f"expected weight of rank 3 but got {weight.dim()}")
     if hidden_states.dim() != 2:
@@ -650,6 +678,16 @@ def grouped_dynamic_scaled_fp8_matmul(
     b_scales = b_scales.contiguous()
     c = torch.empty((T, N), dtype=out_type, device=hidden_states.device)
     a_ld = a_scales.stride(0) if a_scales.shape[0] > 1 else a_scales.shape[1]
+    if out_row_index is not None:
+        if out_row_index.dtype != torch.uint32 or tuple(out_row_index.shape) != (T,):
+            raise TypeError(f"out_row_index must be a uint32 tensor of shape ({T},)")
+        _require_gpu(out_row_index)
+        st = _lib.lib().maxfp8_grouped_matmul_dynamic_scaled_fp8_scatter(
+            c.data_ptr(), out_row_index.data_ptr(), hidden_states.data_ptr(), weight.data_ptr(), a_scales.data_ptr(),
+            b_scales.data_ptr(), expert_start_indices.data_ptr(), expert_ids.data_ptr(), T, N, K, E, max_tokens,
+            num_active, a_ld, _DT[out_type], _DT[a_scales.dtype], _ALGOS[algo], _stream(hidden_states))
+        _lib.check(st)
+        return c
     st = _lib.lib().maxfp8_grouped_matmul_dynamic_scaled_fp8(
         c.data_ptr(), hidden_states.data_ptr(), weight.data_ptr(), a_scales.data_ptr(), b_scales.data_ptr(),
         expert_start_indices.data_ptr(), expert_ids.data_ptr(), T, N, K, E, max_tokens, num_active, a_ld,

@@ -2,14 +2,14 @@
 `_expert_matmuls` (max/python/max/nn/moe/moe_fp8.py:487-616, FP8 block-scaled strategy):
 
     group the (token, expert) assignments by expert      moe_create_indices
-    gather the tokens into that order                    (an index_select: plumbing)
-    quantise 1 x 128                                     quantize_dynamic_scaled_float8
+    gather the tokens into that order and quantise       quantize_dynamic_scaled_float8(row_index=...)
+    1 x 128 (the gather rides on the quantiser's loads)
     gate_up = grouped matmul                             grouped_dynamic_scaled_fp8_matmul
     silu(gate) * up on the rows in use                   fused_silu
-    quantise 1 x 128, down = grouped matmul
-    put the rows back into (token, k) order              (an index_select)
+    quantise 1 x 128, down = grouped matmul that stores  grouped_dynamic_scaled_fp8_matmul(out_row_index=...)
+    its rows back in (token, k) order
 
-Every step with arithmetic in it is one of this package's HIP kernels."""
+Every step is one of this package's HIP kernels; the two row permutations cost no pass of their own."""
 from __future__ import annotations
 
 import torch
@@ -39,18 +39,19 @@ def expert_matmuls_fp8(
     num_experts = gate_up_proj.shape[0]
     token_order, expert_start, restore_order, expert_ids, usage_stats = moe_create_indices(
         router_idx.reshape(-1).to(torch.int32), num_experts)
-    permuted = x.index_select(0, (token_order.to(torch.int64) // top_k))
     stats_host = usage_stats.cpu()  # [most tokens on one expert, active experts]: the op's two host scalars
 
-    def quantise(t: torch.Tensor):
+    def quantise(t: torch.Tensor, **gather):
         return quantize_dynamic_scaled_float8(t, quant_config.input_scale, quant_config.weight_scale,
-                                              scales_type=torch.float32, group_size_or_per_token=128)
+                                              scales_type=torch.float32, group_size_or_per_token=128, **gather)
 
-    def grouped(t_q, t_s, weight, weight_scales):
+    def grouped(t_q, t_s, weight, weight_scales, **scatter):
         return grouped_dynamic_scaled_fp8_matmul(t_q, weight, t_s, weight_scales, expert_start, expert_ids, stats_host,
-                                                 quant_config.input_scale, quant_config.weight_scale)
+                                                 quant_config.input_scale, quant_config.weight_scale, **scatter)
 
-    gate_up = grouped(*quantise(permuted), gate_up_proj, gate_up_proj_scales)
+    # sorted row r is assignment token_order[r] = token * top_k + slot: it reads token token_order[r] // top_k
+    gate_up = grouped(*quantise(x, row_index=token_order, index_div=top_k), gate_up_proj, gate_up_proj_scales)
     act = fused_silu(gate_up, expert_start)
-    down = grouped(*quantise(act), down_proj, down_proj_scales)
-    return down.index_select(0, restore_order.to(torch.int64)).reshape(seq_len, top_k, down.shape[-1])
+    # ... and its result belongs in row token_order[r] of the [seq * top_k, hidden] output
+    down = grouped(*quantise(act), down_proj, down_proj_scales, out_row_index=token_order)
+    return down.reshape(seq_len, top_k, down.shape[-1])
