@@ -292,6 +292,8 @@ def result_line(name, steps, warmup, with_cpu=True):
     elif kind in ("block", "row") and M > 64:
         from modular_amd import _lib
         roof["launches"] = _lib.matmul_describe(M, N, K, kind == "block", True)
+        if roof["launches"].split(" + ")[0].endswith("persistent"):
+            roof["kernel"] = "gemm_persist_kernel"
     roof["kernel_ms_avg"], roof["kernel_ms_median"], roof["kernel_ms_min"] = mm_avg, mm_med, mm_min
     out = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,

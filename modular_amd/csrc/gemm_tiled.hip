@@ -569,6 +569,18 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   }
 }
 
+// tile number -> (row tile, column tile): groups of GROUP_M row tiles share weight columns, walked column-major
+__device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  constexpr int GROUP_M = 4;
+  const int per_group = GROUP_M * tiles_n;
+  const int group = pid / per_group;
+  const int first_m = group * GROUP_M;
+  const int gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int in_group = pid - group * per_group;
+  tm = first_m + in_group % gsize;
+  tn = in_group / gsize;
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool KV = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -581,16 +593,288 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
     const int base = total >> 3, rem = total & 7;
     pid = xcd * base + (xcd < rem ? xcd : rem) + local;
   }
-  constexpr int GROUP_M = 4;
-  const int per_group = GROUP_M * tiles_n;
-  const int group = pid / per_group;
-  const int first_m = group * GROUP_M;
-  const int gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-  const int in_group = pid - group * per_group;
-  const int tm = first_m + in_group % gsize;
-  const int tn = in_group / gsize;
+  int tm, tn;
+  tile_coords(pid, tiles_m, tiles_n, tm, tn);
   const GemmArgs q = gridDim.z == 1 ? p : batch_view(p, blockIdx.z);
   tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false, KV>(q, smem, (int64_t)tm * BM, q.M, tn * BN, q.b, q.b_scales);
+}
+
+// ---- persistent variant ------------------------------------------------------------------------
+// For matmuls made of whole BM x BN tiles with bf16 output.  One block per CU walks its share of
+// the tiles and the slab stream never stops at a tile boundary: while the last slab of a tile is
+// multiplied, slab 0 of the block's next tile is already being copied into the other stage.  The
+// finished tile leaves through a 2 KB LDS side buffer of the wave's own (16 rows at a time, so
+// that a store instruction still writes whole 128-byte lines), which keeps the stage memory free
+// for those copies; the stores of one tile drain while the next one is multiplied.
+//
+// The wait at the top of a tile's first slab must not wait for those stores.  Vector memory
+// operations of a wave complete in order, and after the copy of that slab the wave issued exactly
+// NSTORE unconditional stores, so the copy has landed once at most NSTORE operations are
+// outstanding.  (This is why only whole tiles run here: a predicated store that the compiler
+// may skip would make the count a guess.)
+//
+// Same arithmetic, in the same order, as tile_body: results are bit-equal to gemm_tiled_kernel's.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE>
+__device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
+  constexpr int NS = 2;
+  constexpr int NWAVES = WAVES_M * WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 16, TN = WN / 16;
+  constexpr int IA = BM / 8 / NWAVES, IB = BN / 8 / NWAVES;
+  constexpr int SCALE_BYTES = BLOCKSCALE ? BM * 4 : 0;
+  constexpr int STAGE_BYTES = (BM + BN) * 128 + SCALE_BYTES;
+  constexpr int PER = IA + IB + (BLOCKSCALE ? 1 : 0);
+  constexpr int SIDE_BYTES = 16 * WN * 2;  // a wave's side buffer: 16 rows of its part of the tile
+  constexpr int NSTORE = TM * 2;           // 16-byte stores per lane and tile
+  static_assert(WN == 64 && BM % 64 == 0 && NWAVES % 2 == 0 && IA >= 1 && IB >= 1 && TN % 2 == 0, "tile / wave layout");
+  static_assert(NSTORE < 64, "the count must fit the vmcnt field");
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int lm = lane & 15, lq = lane >> 4;
+
+  // ---- this block's tiles: every 'nb'-th tile of its XCD's contiguous run (blocks are dealt to the XCDs round-robin)
+  const int tiles_m = p.M / BM, tiles_n = p.N / BN, total = tiles_m * tiles_n;
+  const int xcd = blockIdx.x & 7;
+  const int run_begin = xcd * (total >> 3) + (xcd < (total & 7) ? xcd : (total & 7));
+  const int run_len = (total >> 3) + (xcd < (total & 7) ? 1 : 0);
+  const int nb = ((int)gridDim.x - xcd + 7) >> 3;
+  int my = blockIdx.x >> 3;
+  if (my >= run_len) return;
+
+  // ---- global -> LDS copy plan: as in tile_body, with the tile's position in the scalar offset
+  const __amdgpu_buffer_rsrc_t a_rsrc = t2_rsrc(p.a, t2_clamp_u32((int64_t)(p.M - 1) * p.lda + p.K));
+  const __amdgpu_buffer_rsrc_t b_rsrc = t2_rsrc(p.b, t2_clamp_u32((int64_t)(p.N - 1) * p.ldb + p.K));
+  const int cr = lane >> 3, cp = lane & 7;
+  const int cchunk = cp ^ cr;
+  const int cchunk_b = cp ^ (((wave & 1) << 2) | (cr & 3));
+  const uint32_t a_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.lda + cchunk * 16;
+  const uint32_t b_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.ldb + cchunk_b * 16;
+  const uint32_t a_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.lda;
+  const uint32_t b_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.ldb;
+  const int nslab = (p.K + 127) / 128;
+  const int s_chunk = wave % (BM / 64);
+  __amdgpu_buffer_rsrc_t s_rsrc = t2_rsrc(nullptr, 0);
+  uint32_t s_voff = 0, s_slab_step = 0;
+  if constexpr (BLOCKSCALE) {
+    s_rsrc = t2_rsrc(p.a_scales, t2_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + p.M) * 4));
+    s_voff = (uint32_t)(s_chunk * 64 + lane) * 4u;
+    s_slab_step = (uint32_t)p.a_scales_ld * 4u;
+  }
+  struct TileAt { uint32_t a, b, s; };  // byte offsets of a tile's activation rows, weight rows and activation scales
+  auto tile_at = [&](int tm, int tn) {
+    return TileAt{(uint32_t)(tm * BM) * (uint32_t)p.lda, (uint32_t)(tn * BN) * (uint32_t)p.ldb, (uint32_t)(tm * BM) * 4u};
+  };
+  auto dma_one = [&](const TileAt& at, int slab, int buf, int idx, uint32_t dead) {
+    const uint32_t koff = (uint32_t)slab * 128u;
+    uint32_t kill = dead, kill_b = dead;
+    if (koff + cchunk * 16 >= (uint32_t)p.K) kill = 0x80000000u;
+    if (koff + cchunk_b * 16 >= (uint32_t)p.K) kill_b = 0x80000000u;
+    uint8_t* sa = smem + buf * STAGE_BYTES + wave * 1024;
+    uint8_t* sb = sa + BM * 128;
+    if (idx < IA) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(sa + idx * NWAVES * 1024), 16, a_voff | kill,
+                                               at.a + koff + idx * a_istep, 0, 0);
+    } else if (idx < IA + IB) {
+      const int i = idx - IA;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(sb + i * NWAVES * 1024), 16, b_voff | kill_b,
+                                               at.b + koff + i * b_istep, 0, 0);
+    } else if constexpr (BLOCKSCALE) {
+      uint8_t* ss = smem + buf * STAGE_BYTES + (BM + BN) * 128 + s_chunk * 256;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(s_rsrc, (lds_ptr_t)ss, 4, s_voff | dead, at.s + (uint32_t)slab * s_slab_step, 0, 0);
+    }
+  };
+
+  // ---- fragment read plan: as in tile_body
+  const int sw = lm & 7;
+  const uint32_t frag0 = lm * 128 + ((lq ^ sw) << 4);
+  const uint32_t frag1 = lm * 128 + (((lq + 4) ^ sw) << 4);
+  const uint32_t a_frag_base = (uint32_t)(wm * WM) * 128;
+  const uint32_t b_frag_base = (uint32_t)(BM + wn * WN) * 128;
+  auto read_frag = [&](const uint8_t* base) -> v8i {
+    const v4i lo = *reinterpret_cast<const v4i*>(base + frag0);
+    const v4i hi = *reinterpret_cast<const v4i*>(base + frag1);
+    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+  const int wrow = 8 * (lm >> 2) + (lm & 3);
+  const int wsw = (((wrow >> 3) & 1) << 2) | (wrow & 3);
+  const uint32_t wfrag0 = wrow * 128 + ((lq ^ wsw) << 4);
+  const uint32_t wfrag1 = wrow * 128 + (((lq + 4) ^ wsw) << 4);
+  auto read_wfrag = [&](const uint8_t* base, int t) -> v8i {
+    const uint8_t* g = base + (t >> 1) * 4096 + (t & 1) * 512;
+    const v4i lo = *reinterpret_cast<const v4i*>(g + wfrag0);
+    const v4i hi = *reinterpret_cast<const v4i*>(g + wfrag1);
+    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+  const uint32_t s_rd = (uint32_t)((BM + BN) * 128 + (wm * WM + lm) * 4);
+  uint8_t* wbuf = smem + NS * STAGE_BYTES + wave * SIDE_BYTES;
+  const int rr = lane >> 3, cc = lane & 7;
+  const __amdgpu_buffer_rsrc_t c_rsrc = t2_rsrc(p.c, t2_clamp_u32(((int64_t)(p.M - 1) * p.ldc + p.N) * 2));
+  const uint32_t c_row_bytes = (uint32_t)p.ldc * 2u;
+  const uint32_t c_lane = (uint32_t)rr * c_row_bytes + (uint32_t)cc * 16u;
+
+  int tm, tn;
+  tile_coords(run_begin + my, tiles_m, tiles_n, tm, tn);
+  TileAt cur = tile_at(tm, tn);
+#pragma unroll
+  for (int idx = 0; idx < PER; ++idx) dma_one(cur, 0, 0, idx, 0u);
+  float bs_nxt = 1.f;
+  if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld];
+
+  int buf = 0;
+  bool stored = false;  // the wave's last vector memory operations are a tile's NSTORE stores
+  while (true) {
+    const int nxt = my + nb;
+    const bool has_next = nxt < run_len;
+    int tm2 = tm, tn2 = tn;
+    if (has_next) tile_coords(run_begin + nxt, tiles_m, tiles_n, tm2, tn2);
+    const TileAt next = tile_at(tm2, tn2);
+    const float* bs_row = nullptr;
+    if constexpr (BLOCKSCALE) bs_row = p.b_scales + (int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld;
+
+    v4f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    for (int slab = 0; slab < nslab; ++slab) {
+      if (slab == 0 && stored) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTORE) : "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      const float bs = bs_nxt;
+      if constexpr (BLOCKSCALE) {
+        if (slab + 1 < nslab) bs_nxt = bs_row[slab + 1];
+      }
+      asm volatile("" ::: "memory");
+      // the copy issued during this slab: the tile's next slab, or slab 0 of the next tile
+      const bool last = slab + 1 == nslab;
+      const uint32_t dead = (last && !has_next) ? 0x80000000u : 0u;
+      const TileAt dat = last ? next : cur;
+      const int dma_slab = last ? 0 : slab + 1, dma_buf = buf ^ 1;
+      constexpr int SPREAD = TM >= 4 ? TM / 2 : TM;
+
+      const uint8_t* sa = smem + buf * STAGE_BYTES;
+      float s_cur[TM];
+      if constexpr (BLOCKSCALE) {
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) s_cur[mt] = *reinterpret_cast<const float*>(sa + s_rd + mt * 64) * bs;
+      }
+      v8i bf[TN];
+#pragma unroll
+      for (int t = 0; t < TN; ++t) bf[t] = read_wfrag(sa + b_frag_base, t);
+      v8i af = read_frag(sa + a_frag_base);
+      [[maybe_unused]] v4f part[2][TN];
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        v8i af_next = af;
+        if (mt + 1 < TM) af_next = read_frag(sa + a_frag_base + (mt + 1) * 2048);
+        if constexpr (BLOCKSCALE) {
+          const v4f zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int nt = 0; nt < TN; ++nt)
+            part[mt & 1][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
+          // Issue order, pinned: one MFMA of this group, then four promotions of the previous one, four times.
+          // (Left to itself the scheduler put each group's promotions straight behind its own MFMAs and
+          // filled the wait with idle cycles.)
+          if (mt > 0) {
+#pragma unroll
+            for (int nt = 0; nt < TN; ++nt) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+              __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
+            }
+          } else {
+            __builtin_amdgcn_sched_group_barrier(0x008, TN, 0);
+          }
+          if (mt > 0) {
+#pragma unroll
+            for (int nt = 0; nt < TN; ++nt) acc[mt - 1][nt] += part[(mt - 1) & 1][nt] * s_cur[mt - 1];
+          }
+          if (mt == TM - 1) {
+#pragma unroll
+            for (int nt = 0; nt < TN; ++nt) acc[mt][nt] += part[mt & 1][nt] * s_cur[mt];
+          }
+        } else {
+#pragma unroll
+          for (int nt = 0; nt < TN; ++nt)
+            acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
+        }
+        af = af_next;
+#pragma unroll
+        for (int idx = 0; idx < PER; ++idx)
+          if (idx * SPREAD / PER == mt) dma_one(dat, dma_slab, dma_buf, idx, dead);
+      }
+      buf ^= 1;
+    }
+    // the first weight-block scale of the next tile travels while this one is stored
+    if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn2 * BN + wn * WN) / 128) * p.b_scales_ld];
+
+    // ---- the tile leaves, 16 rows of the wave's part at a time
+    // (row scaling: every scale of the tile is loaded before the first store, so that no later wait for a
+    // load also waits for the stores in front of it)
+    float b_s[TN / 2][8], a_s_all[TM];
+    if constexpr (!BLOCKSCALE) {
+#pragma unroll
+      for (int q = 0; q < TN / 2; ++q)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          b_s[q][i] = p.b_scales[(int64_t)(tn * BN + wn * WN + q * 32 + lq * 8 + i) * p.b_scale_stride];
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt)
+        a_s_all[mt] = p.a_scales[((int64_t)tm * BM + wm * WM + mt * 16 + lm) * p.a_scale_stride];
+      asm volatile("" ::: "memory");
+    }
+    // (C goes out through a buffer descriptor: one 32-bit lane offset for all of a lane's stores, the rest scalar)
+    const uint32_t c_tile = ((uint32_t)(tm * BM + wm * WM) * (uint32_t)p.ldc + (uint32_t)(tn * BN + wn * WN)) * 2u;
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) {
+      float a_s = 1.f;
+      if constexpr (!BLOCKSCALE) a_s = a_s_all[mt];
+#pragma unroll
+      for (int q = 0; q < TN / 2; ++q) {
+        v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
+        if constexpr (!BLOCKSCALE) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
+            lo[i] = t_lo * b_s[q][i];
+            hi[i] = t_hi * b_s[q][4 + i];
+          }
+        }
+        *reinterpret_cast<uint4*>(wbuf + lm * (WN * 2) + (((q * 4 + lq) ^ (lm & 7)) * 16)) =
+            make_uint4(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3]));
+      }
+      // (a wave reads back only what it wrote itself, and its LDS operations execute in order)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int r = i * 8 + rr;
+        typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+        const v4u v = *reinterpret_cast<const v4u*>(wbuf + r * (WN * 2) + ((cc ^ (r & 7)) * 16));
+                // (non-temporal: C is not read again here, and its lines should not push the operands out of L2)
+        __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, c_lane, c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes, 2);
+      }
+    }
+    stored = true;
+    if (!has_next) break;
+    my = nxt;
+    tm = tm2;
+    tn = tn2;
+    cur = next;
+  }
+  // the last copies (of nothing: every lane out of range) still write zeros into the stages: they
+  // must have landed before the block's LDS goes to another block
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_persist_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  persist_body<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE>(p, smem);
 }
 
 // ---- grouped (MoE) matmul ---------------------------------------------------------------------
@@ -739,6 +1023,47 @@ static int launch_grouped_large(const GemmArgs& p, dim3 grid, hipStream_t stream
   static bool attr_done = false;
   return launch_with_lds(gemm_grouped_large_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE>, attr_done,
                          tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), WAVES_M * WAVES_N * 64, p, grid, stream, name);
+}
+
+// The persistent kernel takes matmuls of whole 256 x 256 tiles with 16-byte aligned bf16 rows of C, one launch,
+// no K split, and operands whose byte offsets fit 31 bits (a tile's position rides in the copies' scalar offset).
+// MAXFP8_PERSIST=0 switches it off (A/B runs).
+static bool persist_shape(int64_t M, int64_t N, int variant) {
+  const char* e = getenv("MAXFP8_PERSIST");
+  if (e && atoi(e) == 0) return false;
+  return variant == 1 && M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0;
+}
+static bool persist_ok(const GemmArgs& p, bool blockscale, dim3 grid) {
+  if (!persist_shape(p.M, p.N, 1)) return false;
+  if (p.kv_on || p.splits > 1 || grid.y != 1 || grid.z != 1) return false;
+  if (p.c_dtype != MAXFP8_BF16 || !p.c_vec8_ok) return false;
+  const int64_t lim = 0x7ff00000ll, nslab = ceil_div(p.K, 128);
+  if ((int64_t)p.M * p.lda >= lim || (int64_t)p.N * p.ldb >= lim) return false;
+  if (blockscale && (nslab * p.a_scales_ld + p.M) * 4 >= lim) return false;
+  if ((int64_t)p.M * p.ldc * 2 >= lim) return false;
+  return true;
+}
+
+static int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cached[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+template <bool BLOCKSCALE>
+static int launch_persist(const GemmArgs& p, hipStream_t stream, const char* name) {
+  static bool attr_done = false;
+  constexpr int lds = tile_lds_bytes<256, 256, 2, BLOCKSCALE>() + 8 * 2048;  // stages + a 2 KB side buffer per wave
+  const int64_t tiles = (int64_t)(p.M / 256) * (p.N / 256);
+  const int cus = compute_units();
+  const dim3 grid((unsigned)(tiles < cus ? tiles : cus));
+  return launch_with_lds(gemm_persist_kernel<256, 256, 2, 4, BLOCKSCALE>, attr_done, lds, 512, p, grid, stream, name);
 }
 
 // Sums the split-K partial results in split order (deterministic), applies the row / tensor
@@ -898,17 +1223,19 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
 int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, char* buf, size_t len) {
   const TiledPlan plan = make_plan(M, N, K, blockscale, has_workspace, has_workspace ? gemm_tiled_workspace_bytes(M, N, K) : 0, 1, false);
   auto count = [](int64_t m, int64_t n, const TileShape& t) { return (long long)(ceil_div(m, t.bm) * ceil_div(n, t.bn)); };
+  // (what a bf16 result with 16-byte aligned rows gets)
+  auto how = [](int64_t m, int64_t n, int variant) { return persist_shape(m, n, variant) ? " persistent" : ""; };
   if (plan.two.axis) {
     const TileShape &a = kShapes[plan.two.v1 - 1], &b = kShapes[plan.two.v2 - 1];
     const bool cols = plan.two.axis == 1;
     const int64_t m1 = cols ? M : plan.two.cut, n1 = cols ? plan.two.cut : N;
     const int64_t m2 = cols ? M : M - plan.two.cut, n2 = cols ? N - plan.two.cut : N;
-    return snprintf(buf, len, "%dx%d x%lld + %s from %lld: %dx%d x%lld", a.bm, a.bn, count(m1, n1, a), cols ? "columns" : "rows",
-                    (long long)plan.two.cut, b.bm, b.bn, count(m2, n2, b));
+    return snprintf(buf, len, "%dx%d x%lld%s + %s from %lld: %dx%d x%lld%s", a.bm, a.bn, count(m1, n1, a), how(m1, n1, plan.two.v1),
+                    cols ? "columns" : "rows", (long long)plan.two.cut, b.bm, b.bn, count(m2, n2, b), how(m2, n2, plan.two.v2));
   }
   const TileShape& t = kShapes[plan.variant - 1];
   if (plan.splits > 1) return snprintf(buf, len, "%dx%d x%lld, K split %d", t.bm, t.bn, count(M, N, t), plan.splits);
-  return snprintf(buf, len, "%dx%d x%lld", t.bm, t.bn, count(M, N, t));
+  return snprintf(buf, len, "%dx%d x%lld%s", t.bm, t.bn, count(M, N, t), how(M, N, plan.variant));
 }
 
 int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, int64_t batch, hipStream_t stream) {
@@ -963,6 +1290,8 @@ static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, di
     if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false, true>(p, grid, stream, "gemm_qkv_row_256x256");
     return launch_tiled<128, 128, 2, 2, 2, false, true>(p, grid, stream, "gemm_qkv_row_128x128");
   }
+  if (variant == 1 && persist_ok(p, blockscale, grid))
+    return blockscale ? launch_persist<true>(p, stream, "gemm_persist_block_256x256") : launch_persist<false>(p, stream, "gemm_persist_row_256x256");
   if (blockscale) {
     if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, true>(p, grid, stream, "gemm_tiled_block_256x256");
     if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, true>(p, grid, stream, "gemm_tiled_block_256x128");

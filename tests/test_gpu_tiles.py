@@ -189,3 +189,51 @@ def test_two_region_launch(dev, M, K, N, kind):
     # and the f32 output path, against the same reference
     c32 = mx.dynamic_scaled_matmul(q, w, sa, sb, cfg.input_scale, cfg.weight_scale, out_type=torch.float32)
     assert_rel(f32_np(c32[rows]), f32_np(ref), TOL, f"two regions f32 {M}x{N}x{K} {kind}", abs_budget=F32_BUDGET)
+
+
+# ---- persistent kernel (whole 256 x 256 tiles, bf16 out) -----------------------------------------
+# Shapes: fewer tiles than CUs; two and four tiles per block; an uneven share (300 tiles);
+# one slab per tile; a K tail.  The persistent kernel forms every sum in the order of the
+# per-tile kernel, so the two agree bit for bit; exact cases pin both to the true result.
+PERSIST_SHAPES = [(512, 512, 256), (4096, 8192, 256), (2560, 7680, 384), (8192, 8192, 128), (1024, 4096, 144), (256, 256, 1024)]
+
+
+@pytest.mark.parametrize("M,N,K", PERSIST_SHAPES)
+@pytest.mark.parametrize("kind", ["block", "row"])
+def test_persistent_kernel_equals_per_tile_kernel(dev, monkeypatch, M, N, K, kind):
+    monkeypatch.setenv("MAXFP8_TILE", "1")
+    if kind == "block":
+        a, b, sa, sb = make_block(M, N, K, seed=M + K)
+        cfg = BLK
+    else:
+        a, b = synth.random_fp8((M, K), M), synth.random_fp8((N, K), N + 1)
+        sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+        cfg = ROW
+    assert "persistent" in _lib.matmul_describe(M, N, K, kind == "block", False)
+    ad, bd, sad, sbd = a.to(dev), b.to(dev), sa.to(dev), sb.to(dev)
+    run = lambda: mx.dynamic_scaled_matmul(ad, bd, sad, sbd, cfg.input_scale, cfg.weight_scale, out_type=torch.bfloat16,
+                                           algo="tiled")
+    got = run()
+    again = run()  # a second launch on the same stream: same bits
+    monkeypatch.setenv("MAXFP8_PERSIST", "0")
+    want = run()
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(again.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 768, 384), (2560, 7680, 144)])
+def test_persistent_kernel_exact(dev, monkeypatch, M, N, K):
+    monkeypatch.setenv("MAXFP8_TILE", "1")
+    a, b, sa, sb, want = exact_case(M, N, K, seed=M + N + K)
+    cb = mm(a, b, sa, sb, BLK, dev, out=torch.bfloat16, algo="tiled")
+    assert torch.equal(cb.cpu(), torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16))
+
+
+def test_persistent_kernel_leaves_other_outputs_alone(dev, monkeypatch):
+    # f32 output, rows of C that are not 16-byte aligned and partial tiles stay with the per-tile kernel
+    monkeypatch.setenv("MAXFP8_TILE", "1")
+    a, b, sa, sb, want = exact_case(512, 520, 256, seed=9)
+    assert np.array_equal(f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled")).astype(np.float64), want)
+    a, b, sa, sb, want = exact_case(512, 512, 256, seed=10)
+    assert np.array_equal(f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled")).astype(np.float64), want)

@@ -12,7 +12,8 @@ def parse(text):
 
 
 def test_single_shapes_and_k_split():
-    assert _lib.matmul_describe(2048, 6144, 4096) == "256x256 x192"
+    assert _lib.matmul_describe(2048, 6144, 4096) == "256x256 x192 persistent"
+    assert _lib.matmul_describe(2040, 6144, 4096) == "256x256 x192"
     assert _lib.matmul_describe(8, 4096, 4096) == "skinny"
     with_ws, without = _lib.matmul_describe(256, 7168, 16384), _lib.matmul_describe(256, 7168, 16384, True, False)
     assert "K split" in with_ws and "K split" not in without
