@@ -27,10 +27,19 @@ def expert_matmuls_fp8(
     down_proj: torch.Tensor,
     down_proj_scales: torch.Tensor,
     quant_config: QuantConfig,
+    *,
+    host_sync: bool = True,
 ) -> torch.Tensor:
     """x [seq, hidden] bf16; router_idx [seq, k] expert ids; gate_up_proj [E, 2 * I, hidden] and
     down_proj [E, hidden, I] e4m3fn with 128 x 128 block scales.  Returns the experts' outputs
-    [seq, k, hidden] (bf16), before the router weights are applied."""
+    [seq, k, hidden] (bf16), before the router weights are applied.
+
+    The grouped matmul op takes two host scalars (most tokens on one expert, active experts), which
+    the reference copies from the device between the grouping and the first matmul
+    (max/python/max/nn/moe/quant_strategy.py:175).  This package's kernels read the offsets on the
+    device and use the scalars only as upper bounds for their grids, so with `host_sync=False` the
+    bounds (every row on one expert, every expert active) stand in and nothing waits for the GPU:
+    same result, and the whole function can be captured in a HIP graph."""
     if x.dim() != 2 or router_idx.dim() != 2 or router_idx.shape[0] != x.shape[0]:
         raise ValueError("expected x [seq, hidden] and router_idx [seq, k]")
     if not (quant_config.input_scale.is_block and quant_config.weight_scale.is_block):
@@ -39,7 +48,10 @@ def expert_matmuls_fp8(
     num_experts = gate_up_proj.shape[0]
     token_order, expert_start, restore_order, expert_ids, usage_stats = moe_create_indices(
         router_idx.reshape(-1).to(torch.int32), num_experts)
-    stats_host = usage_stats.cpu()  # [most tokens on one expert, active experts]: the op's two host scalars
+    if host_sync:
+        stats_host = usage_stats.cpu()  # [most tokens on one expert, active experts]: the op's two host scalars
+    else:
+        stats_host = torch.tensor([seq_len * top_k, num_experts], dtype=torch.int64).to(torch.uint32)
 
     def quantise(t: torch.Tensor, **gather):
         return quantize_dynamic_scaled_float8(t, quant_config.input_scale, quant_config.weight_scale,
