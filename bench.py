@@ -162,16 +162,30 @@ class Workload:
         return self.matmul(c, q, sa)
 
 
-def run_gpu(name, steps, warmup):
-    """Times `steps` passes of the hot path with the host clock (whole-step throughput), then
+SETTLE_S = 0.5  # the workload runs this long, untimed, before the warm-up steps (see run_gpu)
+
+
+def run_gpu(name, steps, warmup, settle_s=None):
+    """Before anything is timed the workload runs for `settle_s` seconds: an idle MI355X starts at
+    low clocks and takes some tenths of a second of sustained load to reach the clocks it then
+    holds (the same 30 steps measure 10-15 % slower straight after start-up than after half a
+    second of load); a serving process lives in the settled state.  Then `warmup` untimed steps.
+
+    Times `steps` passes of the hot path with the host clock (whole-step throughput), then
     the matmul launches of the same passes with HIP events on the launch stream: once with a
     pair of events per launch (median, minimum) and once with one pair around all launches
-    (average).  Both passes queue their launches behind a bounded spin kernel, so the intervals
-    hold the kernels and not the host's launch latency."""
+    (average).  Both passes queue their launches behind untimed launches of the same matmul."""
     import torch
 
     dev = torch.device("cuda:0")
     wl = Workload(name, dev)
+    settle_s = SETTLE_S if settle_s is None else settle_s
+    t_end, i = time.perf_counter() + settle_s, 0
+    while time.perf_counter() < t_end:
+        for _ in range(16):
+            wl.step(i)
+            i += 1
+        torch.cuda.synchronize()
     for i in range(warmup):
         wl.step(i)
     torch.cuda.synchronize()
@@ -184,24 +198,33 @@ def run_gpu(name, steps, warmup):
 
     quantised = [wl.quantise(c) for c in range(wl.copies)]
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    torch.cuda.synchronize()
-    torch.cuda._sleep(20_000_000)  # ~10 ms: the queue fills while this runs
-    for i in range(steps):
+    # Runway: untimed launches of the same matmul in front of the timed ones.  While the GPU works through
+    # them the host queues the timed launches, so the intervals hold kernels and not launch latency, and the
+    # GPU stays under the load (and at the clocks) of the timed region above.
+    runway = min(2000, 20 + int(steps * 0.012 / max(ms_step, 1e-3)))
+
+    def launch(i):
         c = (warmup + i) % wl.copies
-        events[i][0].record()
         wl.matmul(c, *quantised[c])
+
+    torch.cuda.synchronize()
+    for i in range(runway):
+        launch(i)
+    for i in range(steps):
+        events[i][0].record()
+        launch(i)
         events[i][1].record()
     torch.cuda.synchronize()
     mm_ms = sorted(e[0].elapsed_time(e[1]) for e in events)
-    # The average comes from one pair of events around all `steps` launches, again queued behind the
-    # spin kernel: an event pair around a single launch also holds the few microseconds the command
-    # processor needs between the event and the dispatch, which back-to-back launches overlap.
+    # The average comes from one pair of events around all `steps` launches: an event pair around a single
+    # launch also holds the few microseconds the command processor needs between the event and the
+    # dispatch, which back-to-back launches overlap.
     first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda._sleep(20_000_000)
+    for i in range(runway):
+        launch(i)
     first.record()
     for i in range(steps):
-        c = (warmup + i) % wl.copies
-        wl.matmul(c, *quantised[c])
+        launch(i)
     last.record()
     torch.cuda.synchronize()
     mm_avg = first.elapsed_time(last) / steps
@@ -304,7 +327,7 @@ def result_line(name, steps, warmup, with_cpu=True):
                               "per-token x per-channel" if kind == "row" else "1x128 activations, 128x128 weights",
                    "step": "RMSNorm fused with dynamic quantise" if kind == "rmsq" else
                            "dynamic quantise + " + ("grouped " if kind == "grouped" else "") + "scaled matmul",
-                   "input_copies": wl.copies},
+                   "input_copies": wl.copies, "settle_s": SETTLE_S},
         "roofline": roof,
     }
     if with_cpu:
@@ -313,17 +336,21 @@ def result_line(name, steps, warmup, with_cpu=True):
 
 
 def main():
+    global SETTLE_S
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
+    ap.add_argument("--settle", type=float, default=SETTLE_S,
+                    help="seconds the workload runs, untimed, before the warm-up steps (clock ramp of an idle GPU)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--table", action="store_true", help="run every workload, write gpurun_out/bench_table.json")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB three times (the known-size unit that "
                          "hardware byte counters of a rocprofv3 --pmc run are scaled by)")
     args = ap.parse_args()
+    SETTLE_S = max(0.0, args.settle)
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collective); run with --gpus 1",
               file=sys.stderr)
