@@ -302,6 +302,7 @@ static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream)
 // Shape choice (measured on the Llama-70B decode shapes):
 //   N >= 16384: 32 rows per block (an activation fragment feeds two MFMAs), 16 KB of weights
 //               in flight per wave;
+//   the same with weights under 256 MB: 32 rows per block, 8 KB per wave;
 //   smaller N:  16 rows per block, 8 KB per wave: twice the blocks, and more of them per CU.
 // (8 waves per block were tried for the small-N shapes and were slower.)
 // MAXFP8_SKINNY=<ntw>4<ringKB>, e.g. 1408 or 2416, forces a shape for tuning runs.
@@ -309,7 +310,7 @@ template <int MT, bool BLOCKSCALE>
 static int pick_ntw(const GemmArgs& p, int64_t batch, hipStream_t stream) {
   const char* e = getenv("MAXFP8_SKINNY");
   int sel = e ? atoi(e) : 0;
-  if (!sel) sel = (p.N >= 16384 && MT <= 2) ? 2416 : 1408;
+  if (!sel) sel = (p.N >= 16384 && MT <= 2) ? ((int64_t)p.N * p.K >= ((int64_t)1 << 28) ? 2416 : 2408) : 1408;
   switch (sel) {
     case 1408: return launch_skinny_r<1, MT, BLOCKSCALE, 8, 4>(p, batch, stream);
     case 1416: return launch_skinny_r<1, MT, BLOCKSCALE, 16, 4>(p, batch, stream);

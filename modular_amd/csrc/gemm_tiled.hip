@@ -35,6 +35,7 @@
 // caps the wave tile at 128 x 64 with two waves per SIMD.
 #include <stdlib.h>
 
+#include <mutex>
 #include <utility>
 #include "common.h"
 #include "gemm_args.h"
@@ -1219,6 +1220,30 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
   return plan;
 }
 
+// make_plan tries every cut of every pair of shapes: microseconds of host time, as much as a small matmul
+// takes on the GPU.  Plans are kept in a small table, keyed by everything make_plan reads (the tuning
+// switches of the environment included, since tests and tuning runs flip them between calls).
+static TiledPlan cached_plan(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, size_t workspace_bytes,
+                             int64_t batch, bool kv_on) {
+  struct Entry { int64_t M, N, K, batch; size_t ws; int flags; bool valid; TiledPlan plan; };
+  static Entry table[128];
+  static std::mutex mu;
+  const char* sk = getenv("MAXFP8_SPLITK");
+  const int flags = (blockscale ? 1 : 0) | (has_workspace ? 2 : 0) | (kv_on ? 4 : 0) | (getenv("MAXFP8_ONE_REGION") ? 8 : 0) |
+                    (tile_override() << 4) | ((sk ? atoi(sk) & 0xff : 0) << 8);
+  const uint64_t h = ((uint64_t)M * 0x9e3779b97f4a7c15ull) ^ ((uint64_t)N * 0xc2b2ae3d27d4eb4full) ^ ((uint64_t)K * 0x165667b19e3779f9ull) ^
+                     ((uint64_t)batch << 7) ^ (uint64_t)flags;
+  Entry& e = table[(h >> 32) % 128];
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (e.valid && e.M == M && e.N == N && e.K == K && e.batch == batch && e.ws == workspace_bytes && e.flags == flags) return e.plan;
+  }
+  const TiledPlan plan = make_plan(M, N, K, blockscale, has_workspace, workspace_bytes, batch, kv_on);
+  std::lock_guard<std::mutex> lock(mu);
+  e = Entry{M, N, K, batch, workspace_bytes, flags, true, plan};
+  return plan;
+}
+
 // "256x256 x896" / "256x256 x448, K split 2" / "256x256 x768 + columns from 24576: 256x128 x256"
 int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, char* buf, size_t len) {
   const TiledPlan plan = make_plan(M, N, K, blockscale, has_workspace, has_workspace ? gemm_tiled_workspace_bytes(M, N, K) : 0, 1, false);
@@ -1240,7 +1265,7 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
 
 int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, int64_t batch, hipStream_t stream) {
   GemmArgs p = p_in;
-  const TiledPlan plan = make_plan(p.M, p.N, p.K, blockscale, p.workspace != nullptr, workspace_bytes, batch, p.kv_on != 0);
+  const TiledPlan plan = cached_plan(p.M, p.N, p.K, blockscale, p.workspace != nullptr, workspace_bytes, batch, p.kv_on != 0);
   if (plan.two.axis) {
     const TwoRegionPlan& two = plan.two;
     GemmArgs r1 = p, r2 = p;
