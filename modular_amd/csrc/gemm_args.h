@@ -44,6 +44,9 @@ struct GemmArgs {
   int num_active;
   int small_rows;            // slots with at most this many rows use the small tile (0: none do)
   int big_rows, big_bm;      // slots with at least big_rows rows give their full big_bm-row tiles to the large-tile launch (0: none)
+  // The large-tile launch as a fixed set of blocks that share the chip with the other launch (0: one block per tile):
+  int big_tile_rows;         // upper bound of the number of big_bm-row tiles over all slots
+  float share_bias;          // scales the other launch's estimated work when the blocks decide how many of them stay
   int64_t b_expert_stride;   // bytes between experts in b
   int64_t bs_expert_stride;  // elements between experts in b_scales
   const uint32_t* c_row_index;  // grouped only, optional: row m of the result is stored at row c_row_index[m] of c

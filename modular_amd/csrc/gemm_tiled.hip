@@ -967,22 +967,66 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
 }
 
 // The full BM-row tiles (BM == big_bm) of the slots with at least big_rows rows.
+//
+// Two launch forms.  One block per tile: grid (column tiles, upper bound of row tiles).  Or, with
+// p.big_tile_rows > 0, a one-dimensional grid of at most one block per CU whose blocks walk the same
+// (row tile, column tile) pairs with the grid's stride, so that this launch and gemm_grouped_kernel,
+// sent down another stream, share the chip: these tiles are bound by the matrix pipe, most of the
+// other launch's by HBM, and a block of this kernel fills a CU's LDS, so the two never share a CU.
+// How many blocks stay is decided on the device, where the group sizes are: every block adds up the
+// work of both launches (tiles x the per-tile costs of the host's cost model) and the blocks past this
+// launch's share of the chip exit at once, leaving their CUs to the other launch.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE = true>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   constexpr int NWAVES = WAVES_M * WAVES_N;
-  int slot, tile;
-  const int by = blockIdx.y, bx = blockIdx.x;
-  if (!grouped_find_tile<NWAVES>(p, by, [&](int rows_total) { return grouped_head_rows(p, rows_total) / BM; }, slot, tile)) return;
-  const int64_t row_begin = (int64_t)p.offsets[slot] + (int64_t)tile * BM;
-  const int n0 = bx * BN;
-  const int e = p.expert_ids[slot];
-  if (e < 0) {
-    grouped_zero_tile<NWAVES * 64>(p, row_begin, BM, n0, BN);
-    return;
+  const int ncol = (p.N + BN - 1) / BN;
+  int first = blockIdx.y * ncol + blockIdx.x, stride = 0, last = first + 1;
+  if (p.big_tile_rows > 0) {
+    __shared__ int s_big, s_mid, s_tiny;
+    if (threadIdx.x == 0) { s_big = 0; s_mid = 0; s_tiny = 0; }
+    __syncthreads();
+    int big = 0, mid = 0, tiny = 0;
+    for (int z = threadIdx.x; z < p.num_active; z += NWAVES * 64) {
+      const int rows = (int)(p.offsets[z + 1] - p.offsets[z]);
+      const int head = grouped_head_rows(p, rows), rest = rows - head;
+      big += head / BM;
+      if (rest > p.small_rows) mid += (rest + 127) / 128;
+      else if (rest > 0) tiny += 1;
+    }
+    if (big) atomicAdd(&s_big, big);
+    if (mid) atomicAdd(&s_mid, mid);
+    if (tiny) atomicAdd(&s_tiny, tiny);
+    __syncthreads();
+    const float nslab = (float)((p.K + 127) / 128), ncol_small = (float)((p.N + 127) / 128);
+    const float w_big = (float)s_big * (float)ncol * (nslab * 1.63f + 11.4f);
+    // (two of the other launch's blocks share a CU; tiles of at most small_rows rows only stream their weights)
+    const float w_rest = p.share_bias * 0.5f * ncol_small * ((float)s_mid * (nslab * 0.96f + 11.4f) + (float)s_tiny * (nslab * 0.5f + 6.0f));
+    int keep = (int)((float)gridDim.x * w_big / (w_big + w_rest + 1e-9f) + 0.5f);
+    keep = keep < 8 ? 8 : keep;
+    keep = (keep + 7) & ~7;  // whole rounds of the 8 XCDs
+    if (keep > (int)gridDim.x) keep = (int)gridDim.x;
+    if ((int)blockIdx.x >= keep) return;
+    first = blockIdx.x;
+    stride = keep;
+    last = p.big_tile_rows * ncol;
   }
-  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, true>(p, smem, row_begin, row_begin + BM, n0, p.b + (int64_t)e * p.b_expert_stride,
-                                                             p.b_scales + (int64_t)e * p.bs_expert_stride);
+  for (int t = first; t < last; t += stride) {
+    if (stride) __syncthreads();  // every wave is done with the last tile's LDS (and with the tile search's variables)
+    const int by = t / ncol, bx = t - by * ncol;
+    int slot, tile;
+    if (!grouped_find_tile<NWAVES>(p, by, [&](int rows_total) { return grouped_head_rows(p, rows_total) / BM; }, slot, tile)) return;
+    const int64_t row_begin = (int64_t)p.offsets[slot] + (int64_t)tile * BM;
+    const int n0 = bx * BN;
+    const int e = p.expert_ids[slot];
+    if (e < 0) {
+      grouped_zero_tile<NWAVES * 64>(p, row_begin, BM, n0, BN);
+    } else {
+      tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, true>(p, smem, row_begin, row_begin + BM, n0, p.b + (int64_t)e * p.b_expert_stride,
+                                                                 p.b_scales + (int64_t)e * p.bs_expert_stride);
+    }
+    if (!stride) return;
+  }
 }
 
 template <int BM, int BN, int NS, bool BLOCKSCALE>
@@ -1328,6 +1372,26 @@ static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, di
   return launch_tiled<128, 128, 2, 2, 2, false>(p, grid, stream, "gemm_tiled_row_128x128");
 }
 
+// One extra stream and two events per device, made at the first use and kept until the process ends
+// (default priority, like every stream this library touches).
+struct SideStream { hipStream_t stream; hipEvent_t fork, join; std::mutex mu; bool made, ok; };
+static SideStream* side_stream() {
+  static SideStream table[64];
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  SideStream& s = table[dev];
+  if (!s.made) {
+    s.made = true;
+    s.ok = hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) == hipSuccess &&
+           hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) == hipSuccess &&
+           hipEventCreateWithFlags(&s.join, hipEventDisableTiming) == hipSuccess;
+    if (!s.ok) (void)hipGetLastError();
+  }
+  return s.ok ? &s : nullptr;
+}
+
 int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int64_t max_tokens, hipStream_t stream) {
   GemmArgs p = p_in;
   // Slots with at least 1024 rows (the caller's bound on the largest slot says whether there can
@@ -1342,23 +1406,59 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int6
   p.big_rows = 0;
   p.big_bm = 256;
   const int big_rows = getenv("MAXFP8_BIG_ROWS") ? atoi(getenv("MAXFP8_BIG_ROWS")) : 1024;
-  if (!big && tune != 4 && max_tokens >= big_rows && T / 256 <= 65535) {
+  // The large-tile launch goes down a second stream, as a fixed set of blocks, so that its tiles (bound by the matrix
+  // pipe) and the other launch's (mostly bound by HBM) share the chip instead of taking turns; the caller's stream
+  // waits for both.  MAXFP8_GROUPED_OVERLAP=0 keeps the two launches in line on the caller's stream.
+  SideStream* side = nullptr;
+  const bool large = !big && tune != 4 && max_tokens >= big_rows && T / 256 <= 65535;
+  if (large) {
+    const char* ov = getenv("MAXFP8_GROUPED_OVERLAP");
+    if (!(ov && atoi(ov) == 0)) side = side_stream();
+  }
+  std::unique_lock<std::mutex> side_lock;
+  if (large) {
     p.big_rows = big_rows;
-    const dim3 lgrid((unsigned)ceil_div(p.N, 256), (unsigned)(T / 256));
-    const int rc = blockscale ? launch_grouped_large<256, 256, 2, 4, 2>(p, lgrid, stream, "gemm_grouped_block_256x256")
-                              : launch_grouped_large<256, 256, 2, 4, 2, false>(p, lgrid, stream, "gemm_grouped_row_256x256");
+    GemmArgs pl = p;
+    dim3 lgrid((unsigned)ceil_div(p.N, 256), (unsigned)(T / 256));
+    if (side) {
+      // The large-tile blocks must reach the CUs first (a CU that holds two blocks of the other launch has no room for
+      // one of these until both are gone), so this launch stays on the caller's stream and the other one, a few
+      // microseconds behind because it waits for the fork event, goes down the second stream.
+      side_lock = std::unique_lock<std::mutex>(side->mu);  // one fork / join at a time per device
+      if (hipEventRecord(side->fork, stream) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+        MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "grouped matmul: cannot order the second stream behind the caller's: %s", hipGetErrorString(hipGetLastError()));
+      const char* sb = getenv("MAXFP8_GROUPED_SHARE");
+      pl.big_tile_rows = (int)(T / 256);
+      pl.share_bias = sb ? (float)atof(sb) : 0.5f;  // (measured: the model overrates the other launch's need of CUs)
+      const int64_t pairs = (int64_t)lgrid.x * lgrid.y;
+      const int cus = compute_units();
+      lgrid = dim3((unsigned)(pairs < cus ? pairs : cus));
+    }
+    const int rc = blockscale ? launch_grouped_large<256, 256, 2, 4, 2>(pl, lgrid, stream, "gemm_grouped_block_256x256")
+                              : launch_grouped_large<256, 256, 2, 4, 2, false>(pl, lgrid, stream, "gemm_grouped_row_256x256");
     if (rc != MAXFP8_OK) return rc;
   }
+  // (every return below this line goes through join(): the caller's stream must wait for the second one)
+  auto join = [&](int rc) -> int {
+    if (side && (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(stream, side->join, 0) != hipSuccess) &&
+        rc == MAXFP8_OK)
+      MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "grouped matmul: cannot join the second stream: %s", hipGetErrorString(hipGetLastError()));
+    return rc;
+  };
   // a slot owns one small tile or ceil(rows / BM) tiles: their sum is <= T / BM + num_active
   const int64_t m_tiles = T / bm + p.num_active;
-  if (m_tiles > 65535) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: %lld row tiles exceed the launch limit", (long long)m_tiles);
+  if (m_tiles > 65535) {
+    join(MAXFP8_OK);
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: %lld row tiles exceed the launch limit", (long long)m_tiles);
+  }
   const dim3 grid((unsigned)ceil_div(p.N, 128), (unsigned)m_tiles);
+  hipStream_t rest_stream = side ? side->stream : stream;
   if (!blockscale) {
     if (big) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped rowwise matmul: the 256 x 128 shape is not built");
-    return launch_grouped<128, 128, 2, 2, 2, 32, 1, 4, 3, false>(p, grid, stream, "gemm_grouped_row_128x128");
+    return join(launch_grouped<128, 128, 2, 2, 2, 32, 1, 4, 3, false>(p, grid, rest_stream, "gemm_grouped_row_128x128"));
   }
   if (big) return launch_grouped<256, 128, 4, 2, 3, 64, 2, 4, 3>(p, grid, stream, "gemm_grouped_block_256x128");
-  return launch_grouped<128, 128, 2, 2, 2, 32, 1, 4, 3>(p, grid, stream, "gemm_grouped_block_128x128");
+  return join(launch_grouped<128, 128, 2, 2, 2, 32, 1, 4, 3>(p, grid, rest_stream, "gemm_grouped_block_128x128"));
 }
 
 }  // namespace maxfp8
