@@ -237,3 +237,21 @@ def test_persistent_kernel_leaves_other_outputs_alone(dev, monkeypatch):
     assert np.array_equal(f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled")).astype(np.float64), want)
     a, b, sa, sb, want = exact_case(512, 512, 256, seed=10)
     assert np.array_equal(f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled")).astype(np.float64), want)
+
+
+def test_persistent_kernel_many_tiles_per_block_repeated(dev, monkeypatch):
+    # short K, sixteen tiles per block: the stores of one tile are still in flight when the next tile's first slab
+    # is waited for.  Twelve launches with fresh activations, each compared with the per-tile kernel.
+    monkeypatch.setenv("MAXFP8_TILE", "1")
+    M, N, K = 8192, 32768, 256
+    b = synth.random_fp8((N, K), 77).to(dev)
+    sb = synth.random_scales((N // 128, K // 128), 78).to(dev)
+    sa = synth.random_scales((K // 128, M), 79).to(dev)
+    for seed in range(12):
+        a = synth.random_fp8((M, K), 100 + seed).to(dev)
+        monkeypatch.setenv("MAXFP8_PERSIST", "1")
+        got = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
+        monkeypatch.setenv("MAXFP8_PERSIST", "0")
+        want = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"launch {seed}"
