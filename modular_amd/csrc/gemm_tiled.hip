@@ -1155,7 +1155,7 @@ static const TileShape kShapes[4] = {
     {256, 256, 256, 1.63f, 1.40f, 11.4f},   // 8 waves, 2 stages
     {256, 128, 256, 0.92f, 0.82f, 9.0f},    // 8 waves, 3 stages
     {128, 128, 512, 0.96f, 0.86f, 11.4f},   // 4 waves, 2 stages, two blocks per CU
-    {128, 128, 256, 9.99f, 9.99f, 9.0f},    // 4 waves, 3 stages, one block per CU (tuning only)
+    {128, 128, 256, 0.74f, 0.66f, 9.0f},    // 4 waves, 3 stages, one block per CU: problems of at most one round of such tiles
 };
 
 // MAXFP8_TILE=1/2/3 forces a shape (for tuning runs); anything else lets the cost model pick.
@@ -1186,7 +1186,7 @@ static int pick_splits(int64_t tiles, int slots, int nslab) {
 static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can_split, int64_t batch = 1) {
   int best = 0;
   float best_cost = 0.f;
-  for (int i = 0; i < 3; ++i) {
+  for (int i = 0; i < 4; ++i) {
     const TileShape& t = kShapes[i];
     const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn) * batch;
     const int sp = can_split ? pick_splits(tiles, t.slots, nslab) : 1;
@@ -1203,7 +1203,7 @@ size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   // the largest split count any shape could choose for this problem
   size_t worst = 0;
   const int nslab = (int)ceil_div(K, 128);
-  for (int i = 0; i < 3; ++i) {
+  for (int i = 0; i < 4; ++i) {
     const TileShape& t = kShapes[i];
     const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
     const int sp = pick_splits(tiles, t.slots, nslab);
@@ -1293,7 +1293,7 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
   const TiledPlan plan = make_plan(M, N, K, blockscale, has_workspace, has_workspace ? gemm_tiled_workspace_bytes(M, N, K) : 0, 1, false);
   auto count = [](int64_t m, int64_t n, const TileShape& t) { return (long long)(ceil_div(m, t.bm) * ceil_div(n, t.bn)); };
   // (what a bf16 result with 16-byte aligned rows gets)
-  auto how = [](int64_t m, int64_t n, int variant) { return persist_shape(m, n, variant) ? " persistent" : ""; };
+  auto how = [](int64_t m, int64_t n, int variant) { return persist_shape(m, n, variant) ? " persistent" : (variant == 4 ? " three-stage" : ""); };
   if (plan.two.axis) {
     const TileShape &a = kShapes[plan.two.v1 - 1], &b = kShapes[plan.two.v2 - 1];
     const bool cols = plan.two.axis == 1;
@@ -1369,6 +1369,7 @@ static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, di
   }
   if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false>(p, grid, stream, "gemm_tiled_row_256x256");
   if (variant == 2) return launch_tiled<256, 128, 4, 2, 3, false>(p, grid, stream, "gemm_tiled_row_256x128");
+  if (variant == 4) return launch_tiled<128, 128, 2, 2, 3, false>(p, grid, stream, "gemm_tiled_row_128x128x3");
   return launch_tiled<128, 128, 2, 2, 2, false>(p, grid, stream, "gemm_tiled_row_128x128");
 }
 
