@@ -7,7 +7,7 @@
 //     p = lane & 7) fetches the logical 16-byte chunk p ^ (row & 7) of its row, so the bytes
 //     land in LDS already swizzled for conflict-free MFMA fragment reads.  Rows past the tile
 //     edge read as zero through the buffer descriptor, so partial tiles need no branches.
-//   * NS LDS stages (2 or 3), one barrier per slab, DMA issued NS-1 slabs ahead.
+//   * NS LDS stages (2 or 3; 4 measured no better), one barrier per slab, DMA issued NS-1 slabs ahead.
 //   * every wave issues v_mfma_f32_16x16x128_f8f6f4 on its (BM/WAVES_M) x (BN/WAVES_N)
 //     sub-tile.  The weight fragment is the MFMA's row operand and the activation fragment its
 //     column operand, so a lane ends up with 4 consecutive n for ONE m: the per-token scale is
@@ -77,7 +77,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   constexpr int STAGE_BYTES = (BM + BN) * 128 + SCALE_BYTES;
   constexpr int PER = IA + IB + (BLOCKSCALE ? 1 : 0);  // LDS-DMA instructions per wave and slab
   static_assert(NWAVES % 2 == 0 && IA >= 1 && IB >= 1, "tile / wave layout");
-  static_assert(NS == 2 || NS == 3, "two or three LDS stages");
+  static_assert(NS >= 2 && NS <= 4 && (NS - 2) * PER < 64, "two to four LDS stages; the wait count must fit the vmcnt field");
   static_assert(!BLOCKSCALE || SCALE_ROWS % 64 == 0, "scale rows are copied 64 at a time");
   static_assert(!BLOCKSCALE || (WN <= 128 && 128 % WN == 0), "a wave's columns must sit inside one 128-wide scale block");
 
@@ -250,11 +250,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
 
   int buf = 0;
   for (int slab = slab_begin; slab < slab_end; ++slab) {
-    if (NS == 3) {
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * PER) : "memory");  // the NS - 2 younger slabs may stay in flight
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     const float bs = bs_nxt;
