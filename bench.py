@@ -2,7 +2,7 @@
 """Benchmark of the MI355X FP8 linear hot path.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
-    python bench.py --table          # every BASELINE shape -> gpurun_out/bench_table.json
+    python bench.py --table          # every shape of the benchmark configurations -> bench_table.json in the results folder
 
 A "step" is one pass of the hot path over one batch of synthetic input already resident
 in HBM: dynamic activation quantisation (bf16 -> e4m3fn + f32 scales) followed by the
@@ -162,6 +162,7 @@ class Workload:
         return self.matmul(c, q, sa)
 
 
+RESULTS_DIR = "gpurun_out"
 SETTLE_S = 0.5  # the workload runs this long, untimed, before the warm-up steps (see run_gpu)
 
 
@@ -345,7 +346,7 @@ def main():
     ap.add_argument("--settle", type=float, default=SETTLE_S,
                     help="seconds the workload runs, untimed, before the warm-up steps (clock ramp of an idle GPU)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
-    ap.add_argument("--table", action="store_true", help="run every workload, write gpurun_out/bench_table.json")
+    ap.add_argument("--table", action="store_true", help="run every workload, write bench_table.json into the results folder")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB three times (the known-size unit that "
                          "hardware byte counters of a rocprofv3 --pmc run are scaled by)")
@@ -361,7 +362,7 @@ def main():
         print("bench.py: no GPU visible; the HIP kernels are the only compute path", file=sys.stderr)
         sys.exit(1)
     if args.table:
-        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        os.makedirs(os.path.join(ROOT, RESULTS_DIR), exist_ok=True)
         rows = []
         for name in WORKLOADS:
             print(f"[bench] {name}", file=sys.stderr, flush=True)
@@ -370,7 +371,7 @@ def main():
             print(json.dumps({"workload": name, "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
                               "kernel_ms": r["roofline"]["kernel_ms_avg"], "frac": r["roofline"]["frac"]}),
                   file=sys.stderr, flush=True)
-            with open(os.path.join(ROOT, "gpurun_out", "bench_table.json"), "w") as f:
+            with open(os.path.join(ROOT, RESULTS_DIR, "bench_table.json"), "w") as f:
                 json.dump(rows, f, indent=1)
             torch.cuda.empty_cache()
         return
