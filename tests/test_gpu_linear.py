@@ -58,3 +58,34 @@ def test_rowwise_linear_and_bias(dev):
     y0.weight.copy_(wq.to(dev))
     y0.weight_scale.copy_(ws.to(dev))
     assert_rel(f32_np(y0(x.to(dev))), ref, 1e-2, "rowwise linear")
+
+
+@pytest.mark.parametrize("M,K,N", [(2048, 1024, 28672), (16, 512, 4096), (256, 1024, 1536)])
+def test_linear_replays_from_a_graph(dev, M, K, N):
+    """An FP8 linear (quantise + matmul) has no host synchronisation, so it records into a HIP graph: the
+    persistent kernel with a second region in another tile shape, the decode kernel, and the K-split shapes with
+    their workspace.  Every replay, with eager work and synchronisations between them and new activations in the
+    same buffer, must give the eager result."""
+    from modular_amd import _lib
+    cfg = mx.blockwise_fp8_config()
+    wq, ws = synth.quantize_weight_block(synth.weights_f32(N, K, seed=3))
+    lin = mx.Linear(K, N, cfg, device=dev)
+    lin.weight.copy_(wq.to(dev))
+    lin.weight_scale.copy_(ws.to(dev))
+    x = synth.activations(M, K, seed=4).to(dev)
+    if M == 2048:
+        assert " + " in _lib.matmul_describe(M, N, K) and "persistent" in _lib.matmul_describe(M, N, K)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        lin(x)  # first call outside the capture: it sets the kernels' LDS attributes
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = lin(x)
+    for i in range(3):
+        x.copy_(synth.activations(M, K, seed=10 + i).to(dev))
+        want = lin(x)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {i}"
