@@ -1178,6 +1178,13 @@ static int pick_splits(int64_t tiles, int slots, int nslab) {
   return (nslab + per - 1) / per;  // no empty share
 }
 
+// The per-tile overhead of shape i on an M x N region: the persistent kernel (whole 256 x 256 tiles, no K split)
+// hides 3.5 of the 11.4 microseconds between two tiles (measured: 3.2 per round on q_b, 4.4 on kv_b).
+static bool persist_shape(int64_t M, int64_t N, int variant);
+static float tile_overhead(int64_t M, int64_t N, int i, int splits) {
+  return kShapes[i].t_tile - ((splits == 1 && persist_shape(M, N, i + 1)) ? 3.5f : 0.f);
+}
+
 // cost of a shape (microseconds) = rounds of resident blocks * time of one tile
 static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can_split, int64_t batch = 1) {
   int best = 0;
@@ -1187,7 +1194,7 @@ static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can
     const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn) * batch;
     const int sp = can_split ? pick_splits(tiles, t.slots, nslab) : 1;
     float cost = (float)ceil_div(tiles * sp, t.slots) *
-                 ((float)ceil_div(nslab, sp) * (blockscale ? t.t_slab_block : t.t_slab_row) + t.t_tile);
+                 ((float)ceil_div(nslab, sp) * (blockscale ? t.t_slab_block : t.t_slab_row) + tile_overhead(M, N, i, sp));
     // a split pays a second launch and one write + one read of sp * M * N f32 partial sums (~4 TB/s)
     if (sp > 1) cost += 5.0f + (float)sp * (float)M * (float)N * 8.0f / 4.0e6f;
     if (i == 0 || cost < best_cost) { best = i; best_cost = cost; }
@@ -1211,7 +1218,8 @@ size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 // cost (microseconds) of an unsplit M x N region in tiles of shape t
 static float region_cost(int64_t M, int64_t N, int nslab, const TileShape& t, bool blockscale) {
   const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
-  return (float)ceil_div(tiles, t.slots) * ((float)nslab * (blockscale ? t.t_slab_block : t.t_slab_row) + t.t_tile);
+  return (float)ceil_div(tiles, t.slots) *
+         ((float)nslab * (blockscale ? t.t_slab_block : t.t_slab_row) + tile_overhead(M, N, (int)(&t - kShapes), 1));
 }
 
 // A matmul whose tiles fill the chip a whole number of times plus a small rest wastes most of its
