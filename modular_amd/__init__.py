@@ -15,14 +15,14 @@ from .kernels import (grouped_matmul_rowwise_dynamic_scaled_fp8, fused_qkv_ragge
 from .moe_kernels import fused_silu, fused_silu_quantized, moe_create_indices
 from .moe import expert_matmuls_fp8
 from .quant_ops import matmul_float8, quantized_fused_qkv_matmul, quantized_matmul
-from .linear import Linear
+from .linear import MLP, Linear
 from .weights_quant import parse_quant_config
 
 __all__ = [
     "InputScaleSpec", "QuantConfig", "QuantFormat", "ScaleGranularity", "ScaleOrigin", "WeightScaleSpec",
     "blockwise_fp8_config", "rowwise_fp8_config", "dynamic_scaled_matmul",
     "grouped_dynamic_scaled_fp8_matmul", "quantize_dynamic_scaled_float8", "matmul_float8",
-    "quantized_matmul", "Linear", "rms_norm_fused_quantize_dynamic_scaled_fp8",
+    "quantized_matmul", "Linear", "MLP", "rms_norm_fused_quantize_dynamic_scaled_fp8",
     "moe_create_indices", "fused_silu", "fused_silu_quantized",
     "quantize_static_scaled_float8", "matmul_static_scaled_float8", "parse_quant_config",
     "batched_dynamic_scaled_fp8_matmul", "batched_quantize_dynamic_scaled_fp8",

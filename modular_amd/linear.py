@@ -57,3 +57,91 @@ class Linear(torch.nn.Module):
         if self.bias is not None:
             y = y + self.bias.to(y.dtype)
         return y.reshape(*lead, self.out_dim)
+
+
+class MLP(torch.nn.Module):
+    """Gated feed-forward block `down(act(gate(x)) * up(x))` with FP8 linears, mirroring
+    max/python/max/nn/linear.py:865-1095.
+
+    Like the reference, the gate and up projections run as ONE matmul over their concatenated
+    weights when the quantisation allows it (`QuantConfig.can_use_fused_mlp`, linear.py:1029-1035);
+    here the two weights ARE one buffer (`gate_up_weight`, with `gate_proj.weight` / `up_proj.weight`
+    views of its halves), so nothing is concatenated per call.  For dynamic block scaling with SiLU the
+    activation, the product with `up` and the quantisation of the result for `down_proj` are one
+    kernel (`fused_silu_quantized`): four launches for the whole block, no bf16 intermediate between
+    the activation and the second matmul.  Every other case (bias, another activation, a clamp,
+    static or per-tensor scales) takes the reference's unfused route through the three `Linear`s.
+    """
+
+    _ACTIVATIONS = {
+        "silu": torch.nn.functional.silu,
+        "gelu": torch.nn.functional.gelu,
+        "gelu_tanh": lambda t: torch.nn.functional.gelu(t, approximate="tanh"),
+        "relu": torch.nn.functional.relu,
+        "tanh": torch.tanh,
+        "sigmoid": torch.sigmoid,
+    }
+
+    def __init__(self, hidden_dim: int, feed_forward_length: int, quant_config: QuantConfig, device=None,
+                 has_bias: bool = False, activation_function: str = "silu", swiglu_limit: float = 0.0) -> None:
+        super().__init__()
+        if activation_function not in self._ACTIVATIONS:
+            raise ValueError(f"Unsupported activation function: {activation_function}. "
+                             f"Supported: {sorted(self._ACTIVATIONS)}")
+        self.hidden_dim, self.feed_forward_length = hidden_dim, feed_forward_length
+        self.quant_config = quant_config
+        self.activation_function = activation_function
+        self.swiglu_limit = swiglu_limit
+        self.gate_proj = Linear(hidden_dim, feed_forward_length, quant_config, device=device, has_bias=has_bias)
+        self.up_proj = Linear(hidden_dim, feed_forward_length, quant_config, device=device, has_bias=has_bias)
+        self.down_proj = Linear(feed_forward_length, hidden_dim, quant_config, device=device, has_bias=has_bias)
+        ws = quant_config.weight_scale
+        block_ok = ws.is_block and ws.block_size is not None and feed_forward_length % ws.block_size[0] == 0
+        self._one_matmul = (ws.is_rowwise or block_ok) and quant_config.input_scale.origin == ScaleOrigin.DYNAMIC
+        if self._one_matmul:
+            # one buffer for both weights (and one for their scales); the projections keep views of the halves
+            f = feed_forward_length
+            self.register_buffer("gate_up_weight", torch.zeros((2 * f, hidden_dim), dtype=torch.uint8, device=device)
+                                 .view(torch.float8_e4m3fn))
+            rows = self.gate_proj.weight_scale.shape[0]
+            self.register_buffer("gate_up_weight_scale",
+                                 torch.ones((2 * rows,) + tuple(self.gate_proj.weight_scale.shape[1:]),
+                                            dtype=ws.dtype, device=device))
+            self.gate_proj.weight, self.up_proj.weight = self.gate_up_weight[:f], self.gate_up_weight[f:]
+            self.gate_proj.weight_scale, self.up_proj.weight_scale = (self.gate_up_weight_scale[:rows],
+                                                                      self.gate_up_weight_scale[rows:])
+
+    def _fused(self) -> bool:
+        cfg = self.quant_config
+        return (self._one_matmul and cfg.input_scale.is_block and cfg.weight_scale.is_block
+                and cfg.input_scale.block_size == (1, 128) and self.activation_function == "silu"
+                and self.swiglu_limit == 0 and self.gate_proj.bias is None and self.down_proj.bias is None
+                and self.feed_forward_length % 128 == 0)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from .kernels import dynamic_scaled_matmul, quantize_dynamic_scaled_float8
+        from .moe_kernels import fused_silu_quantized
+
+        cfg = self.quant_config
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        if self._fused():
+            rows = x2.shape[0]
+            xq, xs = quantize_dynamic_scaled_float8(x2, cfg.input_scale, cfg.weight_scale, scales_type=torch.float32)
+            gate_up = dynamic_scaled_matmul(xq, self.gate_up_weight, xs, self.gate_up_weight_scale, cfg.input_scale,
+                                            cfg.weight_scale, out_type=torch.bfloat16)
+            all_rows = torch.tensor([0, rows], dtype=torch.int64).to(torch.uint32).to(x2.device)
+            hq, hs = fused_silu_quantized(gate_up, all_rows, cfg)
+            y = dynamic_scaled_matmul(hq, self.down_proj.weight, hs, self.down_proj.weight_scale, cfg.input_scale,
+                                      cfg.weight_scale, out_type=torch.bfloat16)
+            return y.reshape(*lead, self.hidden_dim)
+        act = self._ACTIVATIONS[self.activation_function]
+        if self._one_matmul and self.gate_proj.bias is None:
+            both = quantized_matmul(x2, self.gate_up_weight, self.gate_up_weight_scale, None, cfg)
+            gate_out, up_out = act(both[:, :self.feed_forward_length]), both[:, self.feed_forward_length:]
+        else:
+            gate_out, up_out = act(self.gate_proj(x2)), self.up_proj(x2)
+        if self.swiglu_limit > 0:
+            gate_out = gate_out.clamp(max=self.swiglu_limit)
+            up_out = up_out.clamp(min=-self.swiglu_limit, max=self.swiglu_limit)
+        return self.down_proj(gate_out * up_out).reshape(*lead, self.hidden_dim)

@@ -1,0 +1,121 @@
+"""The FP8 gated MLP block (`MLP`, mirroring max/python/max/nn/linear.py:865-1095) on the GPU.
+
+Block-scaled with SiLU it is four of this package's kernels: quantise, one matmul over the stacked gate / up
+weights, silu(gate) * up fused with the quantisation for the second matmul, and the down matmul.  Each stage
+is checked against the CPU oracle ON THE GPU'S OWN INPUT of that stage (end to end, two correct runs differ
+by more than a matmul's tolerance: a bf16 flip in gate_up moves the second quantiser's scales), the block
+against float64 arithmetic on the dequantised weights, and the other routes (per-token scales, bias, clamp,
+another activation) against the same block put together from its three `Linear`s."""
+import numpy as np
+import pytest
+import torch
+
+import modular_amd as mx
+import oracle
+from modular_amd import synth
+from util import assert_rel, bf16_bits, f32_np, fp8_bytes
+
+pytestmark = pytest.mark.gpu
+NT = oracle.default_threads()
+BLK = mx.blockwise_fp8_config()
+
+
+def make_block_mlp(hidden, ffl, dev, **kw):
+    mlp = mx.MLP(hidden, ffl, BLK, device=dev, **kw)
+    parts = {}
+    for name, (n, k, seed) in {"gate_proj": (ffl, hidden, 1), "up_proj": (ffl, hidden, 2), "down_proj": (hidden, ffl, 3)}.items():
+        w = synth.weights_f32(n, k, seed=seed)
+        wq, ws = synth.quantize_weight_block(w)
+        getattr(mlp, name).weight.copy_(wq.to(dev))
+        getattr(mlp, name).weight_scale.copy_(ws.to(dev))
+        parts[name] = (wq, ws)
+    return mlp, parts
+
+
+@pytest.mark.parametrize("M,hidden,ffl", [(64, 512, 1024), (300, 1024, 3584), (2048, 512, 2048), (1, 256, 512)])
+def test_block_scaled_mlp_stage_by_stage(dev, M, hidden, ffl):
+    mlp, parts = make_block_mlp(hidden, ffl, dev)
+    assert mlp._fused()
+    # the projections' weights are the halves of one buffer: nothing is concatenated per call
+    assert mlp.gate_proj.weight.data_ptr() == mlp.gate_up_weight.data_ptr()
+    assert torch.equal(mlp.gate_up_weight[ffl:].view(torch.uint8), parts["up_proj"][0].to(dev).view(torch.uint8))
+    x = synth.activations(M, hidden, seed=5)
+    y = mlp(x.to(dev).reshape(1, M, hidden))
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (1, M, hidden) and y.dtype == torch.bfloat16
+
+    # stage 1: quantise + stacked matmul
+    xq, xs = mx.quantize_dynamic_scaled_float8(x.to(dev), BLK.input_scale, BLK.weight_scale, scales_type=torch.float32)
+    gu = mx.dynamic_scaled_matmul(xq, mlp.gate_up_weight, xs, mlp.gate_up_weight_scale, BLK.input_scale, BLK.weight_scale)
+    qo, so = oracle.quantize_dynamic_scaled_fp8(bf16_bits(x), 128, threads=NT)
+    assert np.array_equal(fp8_bytes(xq), qo)
+    w_gu = np.concatenate([fp8_bytes(parts["gate_proj"][0]), fp8_bytes(parts["up_proj"][0])])
+    s_gu = np.concatenate([parts["gate_proj"][1].numpy(), parts["up_proj"][1].numpy()])
+    assert_rel(f32_np(gu), oracle.matmul_blockwise(qo, w_gu, so, s_gu, threads=NT), 1e-2, "gate_up")
+    # stage 2: silu(gate) * up, quantised (scales to the last bits of exp, bytes equal or neighbours)
+    rows = torch.tensor([0, M], dtype=torch.int64).to(torch.uint32).to(dev)
+    hq, hs = mx.fused_silu_quantized(gu, rows, BLK)
+    want_q, want_s = oracle.fused_silu(bf16_bits(gu), M, quantize=True, threads=NT)
+    # (the GPU's exp and the host's differ in the last bits, so now and then a product rounds to the neighbouring
+    # bf16 value; where that product is its group's largest, the group's scale moves by that one bf16 step)
+    got_s = f32_np(hs)
+    close = np.isclose(got_s, want_s, rtol=2 * 2.0 ** -23, atol=0)
+    assert close.mean() >= 0.99 and np.allclose(got_s, want_s, rtol=2.0 ** -7, atol=0)
+    assert (fp8_bytes(hq) != want_q).mean() <= 5e-3
+    # stage 3: the down matmul on the GPU's own quantised activations
+    down = mx.dynamic_scaled_matmul(hq, mlp.down_proj.weight, hs, mlp.down_proj.weight_scale, BLK.input_scale, BLK.weight_scale)
+    ref = oracle.matmul_blockwise(fp8_bytes(hq), fp8_bytes(parts["down_proj"][0]), f32_np(hs), parts["down_proj"][1].numpy(), threads=NT)
+    assert_rel(f32_np(down), ref, 1e-2, "down")
+    assert torch.equal(y.reshape(M, hidden), down), "the block is exactly its stages"
+
+    # against float64 on the dequantised weights: quantisation noise only
+    def deq(name):
+        wq, ws = parts[name]
+        return wq.double() * ws.double().repeat_interleave(128, 0).repeat_interleave(128, 1)[:wq.shape[0], :wq.shape[1]]
+    xd = x.double()
+    full = (torch.nn.functional.silu(xd @ deq("gate_proj").t()) * (xd @ deq("up_proj").t())) @ deq("down_proj").t()
+    err = (y.reshape(M, hidden).double().cpu() - full).norm() / full.norm()
+    assert err < 0.06, f"relative error {err:.3f} against float64 on dequantised weights"
+
+
+@pytest.mark.parametrize("kw", [dict(has_bias=True), dict(activation_function="gelu"), dict(swiglu_limit=0.5)])
+def test_block_scaled_mlp_other_routes(dev, kw):
+    M, hidden, ffl = 48, 512, 1024
+    mlp, _ = make_block_mlp(hidden, ffl, dev, **kw)
+    assert not mlp._fused()
+    if kw.get("has_bias"):
+        for lin, seed in ((mlp.gate_proj, 1), (mlp.up_proj, 2), (mlp.down_proj, 3)):
+            lin.bias.copy_(torch.randn(lin.bias.shape, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16))
+    x = synth.activations(M, hidden, seed=6).to(dev)
+    y = mlp(x)
+    act = mx.MLP._ACTIVATIONS[mlp.activation_function]
+    g, u = act(mlp.gate_proj(x)), mlp.up_proj(x)
+    if mlp.swiglu_limit > 0:
+        g, u = g.clamp(max=mlp.swiglu_limit), u.clamp(min=-mlp.swiglu_limit, max=mlp.swiglu_limit)
+    want = mlp.down_proj(g * u)
+    torch.cuda.synchronize()
+    if kw.get("has_bias"):
+        assert torch.equal(y, want)          # with bias the block IS its three linears
+    else:                                    # one stacked matmul instead of two: other tile shapes, other summation order
+        assert_rel(f32_np(y), f32_np(want), 2e-2, str(kw))
+
+
+def test_per_token_mlp_runs_gate_and_up_as_one_matmul(dev):
+    M, hidden, ffl = 40, 512, 768
+    cfg = mx.rowwise_fp8_config()
+    mlp = mx.MLP(hidden, ffl, cfg, device=dev)
+    assert mlp._one_matmul and not mlp._fused()
+    for lin, (n, k, seed) in ((mlp.gate_proj, (ffl, hidden, 1)), (mlp.up_proj, (ffl, hidden, 2)), (mlp.down_proj, (hidden, ffl, 3))):
+        wq, ws = synth.quantize_weight_rowwise(synth.weights_f32(n, k, seed=seed))
+        lin.weight.copy_(wq.to(dev))
+        lin.weight_scale.copy_(ws.to(dev))
+    x = synth.activations(M, hidden, seed=7, outlier_frac=0.0).to(dev)
+    y = mlp(x)
+    want = mlp.down_proj(torch.nn.functional.silu(mlp.gate_proj(x)) * mlp.up_proj(x))
+    torch.cuda.synchronize()
+    assert_rel(f32_np(y), f32_np(want), 2e-2, "per-token MLP")
+
+
+def test_mlp_argument_checks(dev):
+    with pytest.raises(ValueError):
+        mx.MLP(256, 512, BLK, activation_function="swish")
