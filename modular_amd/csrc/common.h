@@ -12,7 +12,19 @@ namespace maxfp8 {
 // ---- error reporting (host) -------------------------------------------------
 
 void set_error(const char* fmt, ...);
-int launch_status(const char* what);  // MAXFP8_OK or MAXFP8_ERR_LAUNCH after hipGetLastError
+int launch_status(const char* what);
+
+// "done once per device" flags (a kernel's LDS attribute is a property of the device's copy of the kernel)
+struct PerDeviceFlag {
+  bool done[64] = {};
+  // the flag of the current device (the last slot stands for every device past 62)
+  bool& here() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) dev = 63;
+    return done[dev];
+  }
+};
+  // MAXFP8_OK or MAXFP8_ERR_LAUNCH after hipGetLastError
 
 #define MAXFP8_FAIL(code, ...)        \
   do {                                \

@@ -288,7 +288,8 @@ template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
 static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream) {
   using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
   auto kern = gemm_skinny_kernel<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
-  static bool attr_done = false;
+  static PerDeviceFlag attr;
+  bool& attr_done = attr.here();
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM);
     if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "gemm_skinny: cannot reserve %d bytes of LDS: %s", Cfg::SMEM, hipGetErrorString(e));

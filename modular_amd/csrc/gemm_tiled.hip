@@ -1031,8 +1031,9 @@ constexpr int tile_lds_bytes() {
 }
 
 template <typename Kern>
-static int launch_with_lds(Kern kern, bool& attr_done, int smem, int threads, const GemmArgs& p, dim3 grid, hipStream_t stream,
+static int launch_with_lds(Kern kern, PerDeviceFlag& attr, int smem, int threads, const GemmArgs& p, dim3 grid, hipStream_t stream,
                            const char* name) {
+  bool& attr_done = attr.here();
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, smem, hipGetErrorString(e));
@@ -1044,7 +1045,7 @@ static int launch_with_lds(Kern kern, bool& attr_done, int smem, int threads, co
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool KV = false>
 static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
-  static bool attr_done = false;
+  static PerDeviceFlag attr_done;
   // (fused QKV: 8 more bytes per tile row for the rows' cache offsets, after the 2 * BM * BN bytes of staged output)
   constexpr int stages = tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), kv = 2 * BM * BN + 8 * BM * WAVES_N;
   return launch_with_lds(gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, KV>, attr_done,
@@ -1053,7 +1054,7 @@ static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const 
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, int SBM, int SWAVES_M, int SWAVES_N, int SNS, bool BLOCKSCALE = true>
 static int launch_grouped(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
-  static bool attr_done = false;
+  static PerDeviceFlag attr_done;
   constexpr int big = tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), small = tile_lds_bytes<SBM, BN, SNS, BLOCKSCALE>();
   return launch_with_lds(gemm_grouped_kernel<BM, BN, WAVES_M, WAVES_N, NS, SBM, SWAVES_M, SWAVES_N, SNS, BLOCKSCALE>, attr_done,
                          big > small ? big : small, WAVES_M * WAVES_N * 64, p, grid, stream, name);
@@ -1061,7 +1062,7 @@ static int launch_grouped(const GemmArgs& p, dim3 grid, hipStream_t stream, cons
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE = true>
 static int launch_grouped_large(const GemmArgs& p, dim3 grid, hipStream_t stream, const char* name) {
-  static bool attr_done = false;
+  static PerDeviceFlag attr_done;
   return launch_with_lds(gemm_grouped_large_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE>, attr_done,
                          tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
@@ -1099,7 +1100,7 @@ static int compute_units() {
 
 template <bool BLOCKSCALE>
 static int launch_persist(const GemmArgs& p, hipStream_t stream, const char* name) {
-  static bool attr_done = false;
+  static PerDeviceFlag attr_done;
   constexpr int lds = tile_lds_bytes<256, 256, 2, BLOCKSCALE>() + 8 * 2048;  // stages + a 2 KB side buffer per wave
   const int64_t tiles = (int64_t)(p.M / 256) * (p.N / 256);
   const int cus = compute_units();

@@ -60,7 +60,7 @@ def test_rowwise_linear_and_bias(dev):
     assert_rel(f32_np(y0(x.to(dev))), ref, 1e-2, "rowwise linear")
 
 
-@pytest.mark.parametrize("M,K,N", [(2048, 1024, 28672), (16, 512, 4096), (256, 1024, 1536)])
+@pytest.mark.parametrize("M,K,N", [(2048, 2048, 28672), (16, 512, 4096), (256, 1024, 1536)])
 def test_linear_replays_from_a_graph(dev, M, K, N):
     """An FP8 linear (quantise + matmul) has no host synchronisation, so it records into a HIP graph: the
     persistent kernel with a second region in another tile shape, the decode kernel, and the K-split shapes with
