@@ -312,7 +312,8 @@ def result_line(name, steps, warmup, with_cpu=True):
     # the matmul can be more than one launch (two regions in different tile shapes; the grouped matmul's
     # large-tile launch and the rest): kernel_ms_* is the time of all of them, one after the other
     if kind == "grouped":
-        roof["launches"] = "gemm_grouped_large_kernel (full 256-row tiles of experts with >= 1024 rows) + gemm_grouped_kernel (the rest)"
+        roof["launches"] = ("gemm_grouped_large_kernel (full 256-row tiles of experts with >= 1024 rows) + gemm_grouped_kernel "
+                            "(the rest), side by side on two streams")
     elif kind in ("block", "row") and M > 64:
         from modular_amd import _lib
         roof["launches"] = _lib.matmul_describe(M, N, K, kind == "block", True)
