@@ -42,7 +42,7 @@ struct GemmArgs {
   const uint32_t* offsets;
   const int32_t* expert_ids;
   int num_active;
-  int small_rows;            // slots with at most this many rows use the small tile (0: none do)
+  int small_rows;            // a tile with at most this many rows left for it uses the small tile shape (0: none does)
   int big_rows, big_bm;      // slots with at least big_rows rows give their full big_bm-row tiles to the large-tile launch (0: none)
   // The large-tile launch as a fixed set of blocks that share the chip with the other launch (0: one block per tile):
   int big_tile_rows;         // upper bound of the number of big_bm-row tiles over all slots

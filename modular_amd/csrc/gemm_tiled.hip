@@ -948,8 +948,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
   if (!found) return;
   const int64_t slot_begin = p.offsets[slot], row_end = p.offsets[slot + 1];
   const int64_t rest_begin = slot_begin + grouped_head_rows(p, (int)(row_end - slot_begin));
-  const bool small = row_end - rest_begin <= p.small_rows;
   const int64_t row_begin = rest_begin + (int64_t)tile * BM;
+  const bool small = row_end - row_begin <= p.small_rows;  // also the last tile of a longer slot, when few rows are left for it
   const int n0 = bx * BN;
   const int e = p.expert_ids[slot];
   if (e < 0) {
