@@ -15,7 +15,7 @@ from __future__ import annotations
 import torch
 
 from .kernels import grouped_dynamic_scaled_fp8_matmul, quantize_dynamic_scaled_float8
-from .moe_kernels import fused_silu, moe_create_indices
+from .moe_kernels import fused_silu, fused_silu_quantized, moe_create_indices
 from .quant_config import QuantConfig
 
 
@@ -29,6 +29,7 @@ def expert_matmuls_fp8(
     quant_config: QuantConfig,
     *,
     host_sync: bool = True,
+    fuse_activation_quant: bool = False,
 ) -> torch.Tensor:
     """x [seq, hidden] bf16; router_idx [seq, k] expert ids; gate_up_proj [E, 2 * I, hidden] and
     down_proj [E, hidden, I] e4m3fn with 128 x 128 block scales.  Returns the experts' outputs
@@ -39,7 +40,13 @@ def expert_matmuls_fp8(
     (max/python/max/nn/moe/quant_strategy.py:175).  This package's kernels read the offsets on the
     device and use the scalars only as upper bounds for their grids, so with `host_sync=False` the
     bounds (every row on one expert, every expert active) stand in and nothing waits for the GPU:
-    same result, and the whole function can be captured in a HIP graph."""
+    same result, and the whole function can be captured in a HIP graph.
+
+    `fuse_activation_quant=True` runs silu(gate) * up and the quantisation for the down projection as one kernel
+    (`fused_silu_quantized`, the form the reference's expert-parallel path uses, ep_kernels.py:1168-1290) instead of
+    `fused_silu` followed by the quantiser: one pass over gate_up instead of three passes over it and its
+    activation; the product is quantised from f32 instead of from its bf16 rounding, so the fp8 codes can differ
+    by one step from the two-kernel form."""
     if x.dim() != 2 or router_idx.dim() != 2 or router_idx.shape[0] != x.shape[0]:
         raise ValueError("expected x [seq, hidden] and router_idx [seq, k]")
     if not (quant_config.input_scale.is_block and quant_config.weight_scale.is_block):
@@ -63,7 +70,10 @@ def expert_matmuls_fp8(
 
     # sorted row r is assignment token_order[r] = token * top_k + slot: it reads token token_order[r] // top_k
     gate_up = grouped(*quantise(x, row_index=token_order, index_div=top_k), gate_up_proj, gate_up_proj_scales)
-    act = fused_silu(gate_up, expert_start)
+    if fuse_activation_quant:
+        act_q = fused_silu_quantized(gate_up, expert_start, quant_config)
+    else:
+        act_q = quantise(fused_silu(gate_up, expert_start))
     # ... and its result belongs in row token_order[r] of the [seq * top_k, hidden] output
-    down = grouped(*quantise(act), down_proj, down_proj_scales, out_row_index=token_order)
+    down = grouped(*act_q, down_proj, down_proj_scales, out_row_index=token_order)
     return down.reshape(seq_len, top_k, down.shape[-1])

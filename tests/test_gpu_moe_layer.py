@@ -66,6 +66,10 @@ def test_expert_matmuls_fp8(dev, seq, k, E, hidden, inter, zipf):
     free = mx.expert_matmuls_fp8(x.to(dev), router_idx.to(dev), wgu.to(dev), sgu.to(dev), wd.to(dev), sd.to(dev), BLK,
                                  host_sync=False)
     assert torch.equal(free, got), "upper bounds in place of the two host scalars change nothing"
+    fused = mx.expert_matmuls_fp8(x.to(dev), router_idx.to(dev), wgu.to(dev), sgu.to(dev), wd.to(dev), sd.to(dev), BLK,
+                                  fuse_activation_quant=True)
+    rel = (fused.double() - got.double()).norm() / got.double().norm()
+    assert rel < 0.02, f"one-kernel activation + quantisation: {rel:.4f} from the two-kernel form"
     # and against plain float64 arithmetic on the dequantised weights (quantisation error only)
     wgu_f = wgu.double() * sgu.double().repeat_interleave(128, 1).repeat_interleave(128, 2)[:, :2 * inter, :hidden]
     wd_f = wd.double() * sd.double().repeat_interleave(128, 1).repeat_interleave(128, 2)[:, :hidden, :inter]
