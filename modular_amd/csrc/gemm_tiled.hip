@@ -26,7 +26,12 @@
 //
 // Grouped (MoE) mode maps blocks to (expert slot, m-tile, n-tile) from the device-resident
 // offsets with a block-wide prefix sum, so no host synchronisation is needed
-// (semantics: fp8_quantization.mojo:1745-1865).
+// (semantics: fp8_quantization.mojo:1745-1865).  Its large-tile launch and the launch of the rest
+// run side by side on two streams (gemm_grouped_dispatch).
+//
+// Matmuls made of whole 256 x 256 tiles with bf16 output run in gemm_persist_kernel: one block
+// per CU, the slab stream carried across tile boundaries, tiles stored through a small LDS side
+// buffer while the next tile is already being multiplied.
 //
 // Why the tiles are what they are (measured on MI355X): LDS serves ~128 B/clk/CU to
 // ds_read_b128 and LDS-DMA together, the L1 -> LDS path ~50 B/clk/CU, and an MFMA retires in
