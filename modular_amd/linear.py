@@ -101,15 +101,27 @@ class MLP(torch.nn.Module):
         if self._one_matmul:
             # one buffer for both weights (and one for their scales); the projections keep views of the halves
             f = feed_forward_length
+            # (not part of the state dict: a checkpoint names gate_proj / up_proj, and loading those fills the halves)
             self.register_buffer("gate_up_weight", torch.zeros((2 * f, hidden_dim), dtype=torch.uint8, device=device)
-                                 .view(torch.float8_e4m3fn))
+                                 .view(torch.float8_e4m3fn), persistent=False)
             rows = self.gate_proj.weight_scale.shape[0]
             self.register_buffer("gate_up_weight_scale",
                                  torch.ones((2 * rows,) + tuple(self.gate_proj.weight_scale.shape[1:]),
-                                            dtype=ws.dtype, device=device))
-            self.gate_proj.weight, self.up_proj.weight = self.gate_up_weight[:f], self.gate_up_weight[f:]
-            self.gate_proj.weight_scale, self.up_proj.weight_scale = (self.gate_up_weight_scale[:rows],
-                                                                      self.gate_up_weight_scale[rows:])
+                                            dtype=ws.dtype, device=device), persistent=False)
+            self._tie_halves()
+
+    def _tie_halves(self) -> None:
+        f, rows = self.feed_forward_length, self.gate_up_weight_scale.shape[0] // 2
+        self.gate_proj.weight, self.up_proj.weight = self.gate_up_weight[:f], self.gate_up_weight[f:]
+        self.gate_proj.weight_scale, self.up_proj.weight_scale = (self.gate_up_weight_scale[:rows],
+                                                                  self.gate_up_weight_scale[rows:])
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to(device) and friends replace every buffer by a copy: afterwards the halves are views again
+        out = super()._apply(fn, *args, **kwargs)
+        if self._one_matmul:
+            self._tie_halves()
+        return out
 
     def _fused(self) -> bool:
         cfg = self.quant_config

@@ -188,3 +188,29 @@ def test_product_package_does_not_touch_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "import oracle" not in src and "from oracle" not in src and "maxfp8_oracle" not in src, f
+
+
+def test_mlp_stacks_gate_and_up_in_one_buffer():
+    """The gate / up weights of `MLP` are views of one stacked buffer (so the two projections run as one
+    matmul without a per-call concatenation); checkpoints name the three projections only, and moving the
+    module keeps the views tied."""
+    import torch
+    import modular_amd as mx
+
+    m = mx.MLP(256, 512, mx.blockwise_fp8_config())
+    assert m._one_matmul and m._fused()
+    assert sorted(m.state_dict()) == ["down_proj.weight", "down_proj.weight_scale", "gate_proj.weight",
+                                      "gate_proj.weight_scale", "up_proj.weight", "up_proj.weight_scale"]
+    new = {k: (torch.randint(0, 100, v.shape, dtype=torch.uint8).view(v.dtype) if v.dtype == torch.float8_e4m3fn
+               else torch.rand(v.shape)) for k, v in m.state_dict().items()}
+    m.load_state_dict(new)
+    assert torch.equal(m.gate_up_weight[512:].view(torch.uint8), new["up_proj.weight"].view(torch.uint8))
+    assert torch.equal(m.gate_up_weight_scale[:4], new["gate_proj.weight_scale"])
+    m._apply(lambda t: t.clone())  # what .to(device) does to every buffer
+    assert m.gate_proj.weight.data_ptr() == m.gate_up_weight.data_ptr()
+    assert m.up_proj.weight_scale.data_ptr() == m.gate_up_weight_scale[4:].data_ptr()
+    assert torch.equal(m.gate_up_weight[:512].view(torch.uint8), new["gate_proj.weight"].view(torch.uint8))
+    # per-token scales stack as well; static or per-tensor scales, bias or another activation take the unfused route
+    assert mx.MLP(256, 512, mx.rowwise_fp8_config())._one_matmul
+    assert not mx.MLP(256, 512, mx.blockwise_fp8_config(), has_bias=True)._fused()
+    assert not mx.MLP(256, 512, mx.blockwise_fp8_config(), activation_function="gelu")._fused()
