@@ -297,7 +297,9 @@ def result_line(name, steps, warmup, with_cpu=True):
         # weights of every expert that received tokens are streamed once (experts without tokens are never read)
         active = int((wl.counts > 0).sum())
         mm_bytes += (active - 1) * N * K + 4 * (active - 1) * math.ceil(N / 128) * (K // 128)
-    hbm_bound = kind in ("row", "rmsq") or M <= 16
+    # the roof that binds at the published peaks: a matmul is HBM-bound when moving its bytes at 8 TB/s takes longer
+    # than its flops at 5 PFLOP/s (under ~625 flops per byte: every decode shape, and prefill shapes up to M ~ 256)
+    hbm_bound = kind in ("row", "rmsq") or mm_bytes / (PEAK_HBM_GBS * 1e9) > flops / (PEAK_FP8_TFLOPS * 1e12)
     if hbm_bound:
         value, unit = (mm_bytes + q_bytes) / (ms_step * 1e-3) / 1e9, "GB/s"
         roof = {"bound": "hbm", "achieved": mm_bytes / (mm_avg * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s"}
