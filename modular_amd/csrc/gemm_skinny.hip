@@ -300,23 +300,42 @@ static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream)
   return launch_status("gemm_skinny");
 }
 
-// Shape choice (measured on the Llama-70B decode shapes):
-//   N >= 16384: 32 rows per block (an activation fragment feeds two MFMAs), 16 KB of weights
-//               in flight per wave;
-//   the same with weights under 256 MB: 32 rows per block, 8 KB per wave;
-//   smaller N:  16 rows per block, 8 KB per wave: twice the blocks, and more of them per CU.
-// (8 waves per block were tried for the small-N shapes and were slower.)
+// Shape choice.  A block re-reads its M x K activations for every 16 * NTW weight rows, through L1 and L2, so the
+// activation traffic is M / (16 * NTW) times the weight traffic: more rows per block as M grows, as long as there
+// are blocks enough to fill the chip.  Measured on Llama-70B / Llama-8B / DeepSeek-V3 decode shapes, both scale modes:
+//   N <  6144:           16 rows per block, 8 KB of weights in flight per wave (most blocks per CU);
+//   M <= 4:              32 rows per block from N = 16384 up, else 16;
+//   M <= 16:             32 rows per block; 64 for 10240 <= N < 16384;
+//   M >  16:             64 rows per block from N = 10240 up (M = 64, N = 10240, K = 8192: 32 us against 56), else 32
+//                        (M = 64, N = 8192, K = 28672: 75 us against 122);
+//   64 rows per block need K >= 4096 (with few slabs per wave the long epilogue shows) and take 32 KB per wave;
+//   32 rows per block take 16 KB per wave when M <= 16 and the weights exceed 256 MB, else 8 KB.
+// (8 waves per block were tried for the small-N shapes and were slower.)  Every shape splits K over its four waves
+// in the same way and adds the partial sums in the same order: the result does not depend on the choice.
 // MAXFP8_SKINNY=<ntw>4<ringKB>, e.g. 1408 or 2416, forces a shape for tuning runs.
+static int skinny_shape(int64_t M, int64_t N, int64_t K) {
+  int ntw;
+  if (N < 6144) ntw = 1;
+  else if (M <= 4) ntw = N >= 16384 ? 2 : 1;
+  else if (M <= 16) ntw = (N >= 10240 && N < 16384) ? 4 : 2;
+  else ntw = N >= 10240 ? 4 : 2;
+  if (ntw == 4 && K < 4096) ntw = 2;
+  if (ntw == 4) return 4432;
+  if (ntw == 2) return (M <= 16 && N >= 16384 && N * K >= ((int64_t)1 << 28)) ? 2416 : 2408;
+  return 1408;
+}
+
 template <int MT, bool BLOCKSCALE>
 static int pick_ntw(const GemmArgs& p, int64_t batch, hipStream_t stream) {
   const char* e = getenv("MAXFP8_SKINNY");
   int sel = e ? atoi(e) : 0;
-  if (!sel) sel = (p.N >= 16384 && MT <= 2) ? ((int64_t)p.N * p.K >= ((int64_t)1 << 28) ? 2416 : 2408) : 1408;
+  if (!sel) sel = skinny_shape(p.M, p.N, p.K);
   switch (sel) {
     case 1408: return launch_skinny_r<1, MT, BLOCKSCALE, 8, 4>(p, batch, stream);
     case 1416: return launch_skinny_r<1, MT, BLOCKSCALE, 16, 4>(p, batch, stream);
     case 2416: return launch_skinny_r<2, MT, BLOCKSCALE, 16, 4>(p, batch, stream);
     case 2408: return launch_skinny_r<2, MT, BLOCKSCALE, 8, 4>(p, batch, stream);
+    case 4432: return launch_skinny_r<4, MT, BLOCKSCALE, 32, 4>(p, batch, stream);
     default: MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "skinny matmul: unknown shape selector %d", sel);
   }
 }

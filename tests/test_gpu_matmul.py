@@ -113,6 +113,42 @@ def test_mfma_rowwise_exact(dev, algo, M):
     assert np.array_equal(f32_np(c).astype(np.float64), want)
 
 
+@pytest.mark.parametrize("sel", ["1408", "1416", "2408", "2416", "4432"])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (8, 200, 1040), (16, 272, 640), (33, 100, 512), (64, 336, 1152)])
+def test_every_decode_shape_is_exact(dev, monkeypatch, sel, M, N, K):
+    """The decode kernel's shapes (weight rows per block, bytes in flight per wave) forced one by one, on ragged N and
+    K: exact on integer data in both scale modes, so the choice between them cannot change a result."""
+    monkeypatch.setenv("MAXFP8_SKINNY", sel)
+    a, b, sa, sb, want = exact_case(M, N, K, seed=M + N + K)
+    got = f32_np(mm(a, b, sa, sb, BLK, dev, algo="skinny")).astype(np.float64)
+    assert np.array_equal(got, want), f"block mode, shape {sel}: {np.argwhere(got != want)[:4].tolist()}"
+    rng = np.random.default_rng(K + M)
+    ra = torch.from_numpy(np.exp2(rng.integers(-3, 3, (1, M))).astype(np.float32))
+    rb = torch.from_numpy(np.exp2(rng.integers(-3, 3, (N, 1))).astype(np.float32))
+    ai = oracle.e4m3fn_decode(fp8_bytes(a)).astype(np.float64)
+    bi = oracle.e4m3fn_decode(fp8_bytes(b)).astype(np.float64)
+    want_row = (ai @ bi.T) * ra.numpy().reshape(-1, 1) * rb.numpy().reshape(1, -1)
+    got_row = f32_np(mm(a, b, ra, rb, ROW, dev, algo="skinny")).astype(np.float64)
+    assert np.array_equal(got_row, want_row), f"row mode, shape {sel}"
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 16400, 4096), (12, 10256, 4096), (24, 10304, 4224), (40, 12288, 4096),
+                                   (64, 8192, 2048), (20, 20480, 1536), (16, 16384, 16384)])
+def test_chosen_decode_shapes_match_the_scalar_kernel(dev, M, N, K):
+    """Sizes that reach each shape through the kernel's own choice (16, 32 and 64 weight rows per block, both ring
+    sizes), on integer data where both kernels are exact: equal to the scalar kernel bit for bit."""
+    rng = np.random.default_rng(M + N)
+    a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (M, K)).astype(np.float32)))
+    b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (N, K)).astype(np.float32)))
+    kb, nb = -(-K // 128), -(-N // 128)
+    sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (kb, -(-M // 4) * 4))).astype(np.float32))
+    sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (nb, kb))).astype(np.float32))
+    assert torch.equal(mm(a, b, sa, sb, BLK, dev, algo="skinny"), mm(a, b, sa, sb, BLK, dev, algo="naive"))
+    ra = torch.from_numpy(np.exp2(rng.integers(-3, 3, (1, M))).astype(np.float32))
+    rb = torch.from_numpy(np.exp2(rng.integers(-3, 3, (N, 1))).astype(np.float32))
+    assert torch.equal(mm(a, b, ra, rb, ROW, dev, algo="skinny"), mm(a, b, ra, rb, ROW, dev, algo="naive"))
+
+
 # ---- MFMA kernels: tolerance against the oracle ------------------------------------------
 
 @pytest.mark.parametrize("algo,M,N,K", [
