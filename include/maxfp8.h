@@ -153,8 +153,9 @@ int maxfp8_batched_quantize_dynamic_scaled_fp8(
  *   workspace   optional device scratch for split-K, 16-byte aligned, of
  *               workspace_bytes bytes (maxfp8_matmul_workspace_bytes gives the
  *               size that allows every split the library would choose).  NULL
- *               or too small: the matmul runs unsplit, which is slower only
- *               when its tiles cover a small part of the chip.  The contents
+ *               or too small: the matmul runs unsplit (with at most 64 rows:
+ *               on the weight-streaming kernel), which is slower only when
+ *               its tiles cover a small part of the chip.  The contents
  *               are scratch: overwritten by the call, meaningless afterwards.
  */
 int maxfp8_matmul_dynamic_scaled_fp8(

@@ -49,7 +49,7 @@ int gemm_tiled_describe(int64_t, int64_t, int64_t, bool, bool, char*, size_t);
 int gemm_grouped_dispatch(const GemmArgs&, bool, int64_t, int64_t, hipStream_t);
 int gemm_skinny_dispatch(const GemmArgs&, bool, int64_t, hipStream_t);
 int gemm_skinny_max_m();
-bool gemm_skinny_preferred(int64_t M, int64_t N);
+bool gemm_skinny_preferred(int64_t M, int64_t N, int64_t K);
 
 // v rounded to bf16 / f16 and widened back: how an op parameter of the input's dtype arrives
 static float round_to_dtype(float v, int dtype) {
@@ -228,7 +228,7 @@ int maxfp8_fused_silu(void* out, void* out_scales, const void* in, const uint32_
 }
 
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  if (M <= 0 || N <= 0 || K <= 0 || gemm_skinny_preferred(M, N)) return 0;
+  if (M <= 0 || N <= 0 || K <= 0 || gemm_skinny_preferred(M, N, K)) return 0;
   return gemm_tiled_workspace_bytes(M, N, K);  // split-K partial sums; 0 when no split would be used
 }
 
@@ -273,8 +273,13 @@ static int matmul_common(void* c, const void* a, const void* b, const void* a_sc
                            (bt.n == 1 || (bt.a % 16 == 0 && bt.b % 16 == 0));
   if (algo == MAXFP8_ALGO_AUTO) {
     if (!fast_layout) algo = MAXFP8_ALGO_NAIVE;
-    else if (gemm_skinny_preferred(M, N)) algo = MAXFP8_ALGO_SKINNY;
+    else if (gemm_skinny_preferred(M, N, K)) algo = MAXFP8_ALGO_SKINNY;
     else algo = MAXFP8_ALGO_TILED;
+    // 33 to 64 rows: the tiles win through their K split.  Without the workspace the split needs, a narrow weight
+    // matrix would run on a fraction of the chip: the streaming kernel then.
+    if (algo == MAXFP8_ALGO_TILED && M <= gemm_skinny_max_m() && bt.n == 1 &&
+        gemm_tiled_workspace_bytes(M, N, K) > (workspace ? workspace_bytes : 0))
+      algo = MAXFP8_ALGO_SKINNY;
   }
   if (algo == MAXFP8_ALGO_NAIVE) {
     if (block)
@@ -323,7 +328,8 @@ extern "C" {
 int maxfp8_matmul_describe(int64_t M, int64_t N, int64_t K, int block_scaling, int with_workspace, char* buf, size_t len) {
   if (!buf || len == 0) return 0;
   if (M <= 0 || N <= 0 || K <= 0) return snprintf(buf, len, "nothing to do");
-  if (gemm_skinny_preferred(M, N)) return snprintf(buf, len, "skinny");
+  if (gemm_skinny_preferred(M, N, K)) return snprintf(buf, len, "skinny");
+  if (M <= gemm_skinny_max_m() && !with_workspace && gemm_tiled_workspace_bytes(M, N, K) > 0) return snprintf(buf, len, "skinny");
   return gemm_tiled_describe(M, N, K, block_scaling != 0, with_workspace != 0, buf, len);
 }
 

@@ -343,12 +343,13 @@ static int pick_ntw(const GemmArgs& p, int64_t batch, hipStream_t stream) {
 int gemm_skinny_max_m() { return 64; }
 
 // What MAXFP8_ALGO_AUTO gives the weight-streaming kernel: every matmul of at most 32 rows, and those of 33 to 64 rows
-// whose weight matrix has fewer than 10240 rows.  (With four 16-token groups per weight fragment every block re-reads
-// 64 rows of activations through its L1, about 8 TB/s over the chip; on the wide matrices -- Llama-8B gate_up,
-// Llama-70B qkv and gate_up, DeepSeek-V3 q_b -- the three-stage 128 x 128 tiles, which share the activations through
-// LDS, measured 30 us against 70, 39 against 54, 107 against 244 and 13 against 28.  With fewer than 80 column tiles
-// the tiled kernels have to split K and pay for the reduction: there the streaming kernel stays ahead.)
-bool gemm_skinny_preferred(int64_t M, int64_t N) { return M <= 32 || (M <= 64 && N < 10240); }
+// whose weights take less than 32 MB.  With four 16-token groups per weight fragment every block re-reads 64 rows of
+// activations through its L1 (about 8 TB/s over the chip) and its time grows with M, while the three-stage 128 x 128
+// tiles share the activations through LDS, split K over the chip when their column tiles are few, and take the same
+// time from 1 to 128 rows: at M = 64 they measured 54 us against 75 (N = 8192, K = 28672), 19 against 36 (2304 x
+// 16384), 25 against 32 (10240 x 8192), 30 against 40 (28672 x 4096).  Their floor is two launches, 16 to 17 us:
+// below 32 MB of weights the streaming kernel stays ahead (4096 x 4096: 12 us; 6144 x 4096: 14).
+bool gemm_skinny_preferred(int64_t M, int64_t N, int64_t K) { return M <= 32 || (M <= 64 && N * K < ((int64_t)1 << 25)); }
 
 int gemm_skinny_dispatch(const GemmArgs& p, bool blockscale, int64_t batch, hipStream_t stream) {
   if (p.M > 64) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "skinny matmul: M = %d exceeds 64", p.M);

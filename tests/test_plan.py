@@ -16,7 +16,10 @@ def test_single_shapes_and_k_split():
     assert _lib.matmul_describe(2040, 6144, 4096) == "256x256 x192"
     assert _lib.matmul_describe(8, 4096, 4096) == "skinny"
     assert _lib.matmul_describe(64, 4096, 4096) == "skinny" and _lib.matmul_describe(32, 28672, 4096) == "skinny"
-    assert _lib.matmul_describe(64, 28672, 4096).startswith("128x128")  # 33 to 64 rows on a wide weight matrix: tiles
+    # 33 to 64 rows go to the tiles unless the weights are small (under 32 MB): wide matrices, and narrow ones split over K
+    assert _lib.matmul_describe(64, 28672, 4096).startswith("128x128")
+    assert "K split" in _lib.matmul_describe(48, 8192, 28672) and _lib.matmul_describe(33, 6144, 4096) == "skinny"
+    assert _lib.matmul_describe(48, 8192, 28672, True, False) == "skinny"  # no workspace, no split: the streaming kernel
     with_ws, without = _lib.matmul_describe(256, 7168, 16384), _lib.matmul_describe(256, 7168, 16384, True, False)
     assert "K split" in with_ws and "K split" not in without
     assert _lib.matmul_describe(0, 10, 10) == "nothing to do"
