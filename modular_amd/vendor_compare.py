@@ -21,7 +21,8 @@ from modular_amd import synth
 
 DEFAULT_SHAPES = [
     (2048, 28672, 4096), (2048, 4096, 14336), (4096, 7168, 16384), (4096, 24576, 1536), (4096, 32768, 512),
-    (8192, 8192, 8192), (2048, 2304, 16384), (256, 2304, 16384), (16, 2304, 16384), (64, 28672, 4096),
+    (4096, 1536, 7168), (4096, 576, 7168), (8192, 8192, 8192), (2048, 2304, 16384), (256, 2304, 16384),
+    (16, 2304, 16384), (256, 8192, 28672), (128, 8192, 28672), (64, 28672, 4096), (48, 8192, 28672),
     (32, 8192, 28672), (16, 57344, 8192), (8, 57344, 8192), (1, 57344, 8192),
 ]
 
