@@ -149,6 +149,38 @@ def test_chosen_decode_shapes_match_the_scalar_kernel(dev, M, N, K):
     assert torch.equal(mm(a, b, ra, rb, ROW, dev, algo="skinny"), mm(a, b, ra, rb, ROW, dev, algo="naive"))
 
 
+def test_random_shapes_through_the_automatic_choice_are_exact(dev):
+    """A seeded sweep of shapes over every regime of the automatic choice (decode kernel, K-split tiles, three-stage
+    tiles, two regions, the persistent kernel), ragged and aligned, both scale modes, f32 and bf16 out: on integer
+    data, where every kernel is exact, the result equals the scalar kernel's bit for bit."""
+    rng = np.random.default_rng(2024)
+    for it in range(60):
+        kind = it % 6
+        if kind == 0:
+            M, N, K = int(rng.integers(1, 65)), int(rng.integers(1, 12000)), 16 * int(rng.integers(1, 300))
+        elif kind == 1:
+            M, N, K = int(rng.integers(33, 65)), 128 * int(rng.integers(40, 120)), 128 * int(rng.integers(16, 64))
+        elif kind == 2:
+            M, N, K = 256 * int(rng.integers(1, 6)), 256 * int(rng.integers(1, 40)), 128 * int(rng.integers(1, 24))
+        elif kind == 3:
+            M, N, K = int(rng.integers(65, 900)), int(rng.integers(1, 4000)), 16 * int(rng.integers(1, 200))
+        elif kind == 4:
+            M, N, K = int(rng.integers(100, 2100)), 8 * int(rng.integers(100, 1200)), 128 * int(rng.integers(1, 20))
+        else:
+            M, N, K = int(rng.integers(1, 33)), 16 * int(rng.integers(600, 1400)), 128 * int(rng.integers(30, 70))
+        a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (M, K)).astype(np.float32)))
+        b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (N, K)).astype(np.float32)))
+        kb, nb = -(-K // 128), -(-N // 128)
+        sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (kb, -(-M // 4) * 4))).astype(np.float32))
+        sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (nb, kb))).astype(np.float32))
+        ra = torch.from_numpy(np.exp2(rng.integers(-3, 3, (1, M))).astype(np.float32))
+        rb = torch.from_numpy(np.exp2(rng.integers(-3, 3, (N, 1))).astype(np.float32))
+        out = torch.bfloat16 if it % 2 else torch.float32
+        for cfg, x, y in ((BLK, sa, sb), (ROW, ra, rb)):
+            got, ref = mm(a, b, x, y, cfg, dev, out=out), mm(a, b, x, y, cfg, dev, out=out, algo="naive")
+            assert torch.equal(got, ref), f"{M}x{N}x{K} {out} {'block' if cfg is BLK else 'row'}"
+
+
 # ---- MFMA kernels: tolerance against the oracle ------------------------------------------
 
 @pytest.mark.parametrize("algo,M,N,K", [
