@@ -140,3 +140,38 @@ def test_moe_config_sampled(dev):
                                         BLK.weight_scale, out_type=torch.float32, algo="naive")
         torch.cuda.synchronize()
         assert_rel(f32_np(c[rows]), f32_np(refc), TOL, f"expert {e} rows {r0}:{r1}")
+
+
+def test_random_groupings_are_exact(dev):
+    """A seeded sweep of groupings (empty, tiny, mid-size and >= 1024-row slots side by side, skipped experts, rows
+    past the last slot, ragged and aligned N): on integer data the automatic choice -- large-tile launch, 128-row
+    tiles, 32-row tiles -- equals the scalar kernel bit for bit on every row that belongs to a slot."""
+    rng = np.random.default_rng(77)
+    for it in range(36):
+        E = int(rng.integers(1, 24))
+        active = int(rng.integers(1, E + 1))
+        if it % 3 == 0:
+            counts = rng.integers(0, 70, active)
+        elif it % 3 == 1:
+            counts = rng.choice([0, 1, 5, 31, 32, 33, 127, 128, 129, 300, 1023, 1024, 1025, 1300, 2600], active)
+        else:
+            counts = (rng.zipf(1.3, active) * 7 % 3000).astype(np.int64)
+        ids = rng.permutation(E)[:active].astype(np.int32)
+        ids[rng.random(active) < 0.1] = -1
+        extra = int(rng.integers(0, 9)) if it % 4 == 0 else 0
+        N = 8 * int(rng.integers(8, 160)) if it % 2 else 128 * int(rng.integers(1, 12))
+        K = 128 * int(rng.integers(1, 12))
+        if counts.sum() == 0:
+            counts[0] = 3
+        live = int(counts.sum())
+        T = live + extra
+        a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (T, K)).astype(np.float32)))
+        b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (E, N, K)).astype(np.float32)))
+        sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (K // 128, -(-T // 4) * 4))).astype(np.float32))
+        sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (E, -(-N // 128), K // 128))).astype(np.float32))
+        off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32)
+        idt = torch.tensor(list(ids) + [-1] * (E - active), dtype=torch.int32)
+        out = torch.bfloat16 if it % 2 else torch.float32
+        got = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=out)
+        want = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=out, algo="naive")
+        assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, N {N}, K {K}, {out}"
