@@ -301,27 +301,32 @@ static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream)
 }
 
 // Shape choice.  A block re-reads its M x K activations for every 16 * NTW weight rows, through L1 and L2, so the
-// activation traffic is M / (16 * NTW) times the weight traffic: more rows per block as M grows, as long as there
-// are blocks enough to fill the chip.  Measured on Llama-70B / Llama-8B / DeepSeek-V3 decode shapes, both scale modes:
-//   N <  6144:           16 rows per block, 8 KB of weights in flight per wave (most blocks per CU);
-//   M <= 4:              32 rows per block from N = 16384 up, else 16;
-//   M <= 16:             32 rows per block; 64 for 10240 <= N < 16384;
-//   M >  16:             64 rows per block from N = 10240 up (M = 64, N = 10240, K = 8192: 32 us against 56), else 32
-//                        (M = 64, N = 8192, K = 28672: 75 us against 122);
-//   64 rows per block need K >= 4096 (with few slabs per wave the long epilogue shows) and take 32 KB per wave;
-//   32 rows per block take 16 KB per wave when M <= 16 and the weights exceed 256 MB, else 8 KB.
-// (8 waves per block were tried for the small-N shapes and were slower.)  Every shape splits K over its four waves
+// activation traffic is M / (16 * NTW) times the weight traffic, and all blocks are resident at once, so a CU's
+// share is ceil(blocks / CUs) blocks.  The shape with the smallest
+//     ceil(blocks / CUs) * (16 * NTW + M + 8)        (8: ring fill and the epilogue of a block, in the same unit)
+// wins; 64-row blocks count 25 % more (one block per CU: 32 KB of weights in flight per wave, but fewer waves to
+// hide latency with) and need K >= 4096 (with few slabs per wave the long epilogue shows).  Measured on Llama-70B /
+// Llama-8B / DeepSeek-V3 decode shapes in both scale modes the rule lands on the fastest shape or within 4 % of it;
+// e.g. M = 64, N = 8192, K = 28672: 32 rows per block, 75 us (16 rows: 122); M = 32, N = 10240, K = 8192: 64 rows,
+// 23 us (16 rows: 33); M = 32, N = 5120, K = 5120: 32 rows, 12 us (16 rows: 18); N = 4096: 16 rows, one block per CU.
+// 32-row blocks keep 16 KB per wave in flight when M <= 16 and the weights exceed 256 MB, else 8 KB.
+// (8 waves per block were tried for the small-N shapes and were no faster.)  Every shape splits K over its four waves
 // in the same way and adds the partial sums in the same order: the result does not depend on the choice.
 // MAXFP8_SKINNY=<ntw>4<ringKB>, e.g. 1408 or 2416, forces a shape for tuning runs.
+int compute_units();
 static int skinny_shape(int64_t M, int64_t N, int64_t K) {
-  int ntw;
-  if (N < 6144) ntw = 1;
-  else if (M <= 4) ntw = N >= 16384 ? 2 : 1;
-  else if (M <= 16) ntw = (N >= 10240 && N < 16384) ? 4 : 2;
-  else ntw = N >= 10240 ? 4 : 2;
-  if (ntw == 4 && K < 4096) ntw = 2;
-  if (ntw == 4) return 4432;
-  if (ntw == 2) return (M <= 16 && N >= 16384 && N * K >= ((int64_t)1 << 28)) ? 2416 : 2408;
+  const int64_t cus = compute_units();
+  int best = 1;
+  float best_cost = 0.f;
+  for (int ntw = 1; ntw <= 4; ntw *= 2) {
+    if (ntw == 4 && K < 4096) break;
+    const int64_t blocks = ceil_div(N, 16 * ntw);
+    float cost = (float)ceil_div(blocks, cus) * (float)(16 * ntw + M + 8);
+    if (ntw == 4) cost *= 1.25f;
+    if (ntw == 1 || cost < best_cost) { best = ntw; best_cost = cost; }
+  }
+  if (best == 4) return 4432;
+  if (best == 2) return (M <= 16 && N >= 16384 && N * K >= ((int64_t)1 << 28)) ? 2416 : 2408;
   return 1408;
 }
 

@@ -1091,7 +1091,7 @@ static bool persist_ok(const GemmArgs& p, bool blockscale, dim3 grid) {
   return true;
 }
 
-static int compute_units() {
+int compute_units() {
   static int cached[64] = {0};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;

@@ -133,7 +133,8 @@ def test_every_decode_shape_is_exact(dev, monkeypatch, sel, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(3, 16400, 4096), (12, 10256, 4096), (24, 10304, 4224), (40, 12288, 4096),
-                                   (64, 8192, 2048), (20, 20480, 1536), (16, 16384, 16384)])
+                                   (64, 8192, 2048), (20, 20480, 1536), (16, 16384, 16384), (8, 16384, 16384),
+                                   (5, 4090, 2048), (32, 5120, 5120)])
 def test_chosen_decode_shapes_match_the_scalar_kernel(dev, M, N, K):
     """Sizes that reach each shape through the kernel's own choice (16, 32 and 64 weight rows per block, both ring
     sizes), on integer data where both kernels are exact: equal to the scalar kernel bit for bit."""
