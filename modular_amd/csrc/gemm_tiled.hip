@@ -1119,17 +1119,49 @@ template <bool BLOCKSCALE>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
   const int64_t total = (int64_t)p.M * p.N;
   const int64_t stride = (int64_t)gridDim.x * 256 * 4;
+  const bool quads = (total & 3) == 0;
+  // four consecutive elements sit in one row of C and may leave as one store
+  const bool row_quads = quads && (p.N & 3) == 0 && p.c_vec_ok;
   for (int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4; i < total; i += stride) {
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     const int cnt = (total - i) < 4 ? (int)(total - i) : 4;
-    for (int sp = 0; sp < p.splits; ++sp) {
-      const float* src = p.workspace + (int64_t)sp * total + i;
-      if (cnt == 4 && (total & 3) == 0) {
-        const float4 t = *reinterpret_cast<const float4*>(src);
+    if (cnt == 4 && quads) {
+      // the shares are added in their order, whatever the number of loads in flight
+      const float* src = p.workspace + i;
+      int sp = 0;
+      for (; sp + 4 <= p.splits; sp += 4) {
+        float4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t[u] = *reinterpret_cast<const float4*>(src + (int64_t)(sp + u) * total);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { v[0] += t[u].x; v[1] += t[u].y; v[2] += t[u].z; v[3] += t[u].w; }
+      }
+      for (; sp < p.splits; ++sp) {
+        const float4 t = *reinterpret_cast<const float4*>(src + (int64_t)sp * total);
         v[0] += t.x; v[1] += t.y; v[2] += t.z; v[3] += t.w;
-      } else {
+      }
+    } else {
+      for (int sp = 0; sp < p.splits; ++sp) {
+        const float* src = p.workspace + (int64_t)sp * total + i;
         for (int j = 0; j < cnt; ++j) v[j] += src[j];
       }
+    }
+    if (row_quads) {
+      const int64_t m = i / p.N;
+      const int64_t n = i - m * p.N;
+      if constexpr (!BLOCKSCALE) {
+        const float a_s = p.a_scales[m * p.a_scale_stride];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float r = v[j] * a_s;
+          v[j] = r * p.b_scales[(n + j) * p.b_scale_stride];
+        }
+      }
+      if (p.c_dtype == MAXFP8_BF16)
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.c) + m * p.ldc + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      else
+        *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.c) + m * p.ldc + n) = make_float4(v[0], v[1], v[2], v[3]);
+      continue;
     }
     for (int j = 0; j < cnt; ++j) {
       const int64_t m = (i + j) / p.N;
