@@ -347,14 +347,21 @@ static int pick_ntw(const GemmArgs& p, int64_t batch, hipStream_t stream) {
 
 int gemm_skinny_max_m() { return 64; }
 
-// What MAXFP8_ALGO_AUTO gives the weight-streaming kernel: every matmul of at most 32 rows, and those of 33 to 64 rows
-// whose weights take less than 32 MB.  With four 16-token groups per weight fragment every block re-reads 64 rows of
+// What MAXFP8_ALGO_AUTO gives the weight-streaming kernel: every matmul of at most 32 rows (but see below), and those
+// of 33 to 64 rows whose weights take less than 32 MB.  With four 16-token groups per weight fragment every block re-reads 64 rows of
 // activations through its L1 (about 8 TB/s over the chip) and its time grows with M, while the three-stage 128 x 128
 // tiles share the activations through LDS, split K over the chip when their column tiles are few, and take the same
 // time from 1 to 128 rows: at M = 64 they measured 54 us against 75 (N = 8192, K = 28672), 19 against 36 (2304 x
 // 16384), 25 against 32 (10240 x 8192), 30 against 40 (28672 x 4096).  Their floor is two launches, 16 to 17 us:
 // below 32 MB of weights the streaming kernel stays ahead (4096 x 4096: 12 us; 6144 x 4096: 14).
-bool gemm_skinny_preferred(int64_t M, int64_t N, int64_t K) { return M <= 32 || (M <= 64 && N * K < ((int64_t)1 << 25)); }
+// From 25 rows on the tiles are already ahead where K is long and N narrow (M = 32: 48 us against 53 on 8192 x 28672,
+// 17 against 21 on 4096 x 14336 and on 2304 x 16384); at 24 rows and below the streaming kernel wins or ties.
+bool gemm_skinny_preferred(int64_t M, int64_t N, int64_t K) {
+  const bool small_weights = N * K < ((int64_t)1 << 25);
+  if (M <= 24) return true;
+  if (M <= 32) return small_weights || K < 12288 || N >= 10240;
+  return M <= 64 && small_weights;
+}
 
 int gemm_skinny_dispatch(const GemmArgs& p, bool blockscale, int64_t batch, hipStream_t stream) {
   if (p.M > 64) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "skinny matmul: M = %d exceeds 64", p.M);

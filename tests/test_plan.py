@@ -20,6 +20,9 @@ def test_single_shapes_and_k_split():
     assert _lib.matmul_describe(64, 28672, 4096).startswith("128x128")
     assert "K split" in _lib.matmul_describe(48, 8192, 28672) and _lib.matmul_describe(33, 6144, 4096) == "skinny"
     assert _lib.matmul_describe(48, 8192, 28672, True, False) == "skinny"  # no workspace, no split: the streaming kernel
+    # 25 to 32 rows: the tiles only where K is long and N narrow
+    assert "K split" in _lib.matmul_describe(32, 8192, 28672) and _lib.matmul_describe(24, 8192, 28672) == "skinny"
+    assert _lib.matmul_describe(32, 8192, 8192) == "skinny" and _lib.matmul_describe(32, 10240, 16384) == "skinny"
     with_ws, without = _lib.matmul_describe(256, 7168, 16384), _lib.matmul_describe(256, 7168, 16384, True, False)
     assert "K split" in with_ws and "K split" not in without
     assert _lib.matmul_describe(0, 10, 10) == "nothing to do"
