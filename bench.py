@@ -10,7 +10,9 @@ scaled FP8 matmul (bf16 out), or the grouped matmul for the MoE workload.  Input
 through enough copies to exceed twice the 256 MB Infinity Cache, so no step finds its
 operands cached.  Prints ONE JSON line with the whole-step throughput, the roofline of
 the dominant kernel (timed with events on the launch stream inside the timed region) and
-the CPU oracle timed on this host's cores on a bounded slice of the same workload.
+the CPU oracle timed on this host's cores on a bounded slice of the same workload.  The
+default run times the block-scaled GEMM the MFMA target is quoted on and adds a "decode"
+record (same fields) for the HBM half of the metric; --workload NAME prints that workload alone.
 """
 from __future__ import annotations
 
@@ -63,7 +65,11 @@ WORKLOADS = {
     "rmsnorm_quant_m4096_k7168": ("rmsq", 4096, 7168, 0),
     "rmsnorm_quant_m32768_k7168": ("rmsq", 32768, 7168, 0),
 }
-DEFAULT = "llama8b_gate_up_m2048"
+# The two halves of the metric, each on the shape its target is quoted on: the block-scaled GEMM at M >= 2048 on a
+# DeepSeek-V3 projection (configs[2]; the headline line) and an M <= 8 decode matmul of configs[3] (the "decode"
+# record of the same line).
+DEFAULT = "dsv3_o_proj_m4096"
+DEFAULT_DECODE = "decode70b_gate_up_m8"
 
 
 def measured_traffic(name):
@@ -281,10 +287,32 @@ def cpu_baseline(wl, budget_s=15.0):
         value, unit = (N * K + rows * K + 2 * rows * N) / t / 1e9, "GB/s"
     else:
         value, unit = flops / t / 1e12, "TFLOP/s"
-    sample = (f"oracle quantise + matmul (per-128-slab order) on rows 0..{rows - 1} of M={M}"
+    order = "one f32 dot product per row pair, scales applied once" if kind == "row" else \
+        "oracle mode 1: one f32 partial sum per 128-wide K group, then acc += partial * (a_s * b_s) -- the order a tiled kernel uses, not the reference's element order (mode 0)"
+    sample = (f"oracle quantise + matmul ({order}) on rows 0..{rows - 1} of M={M}"
               + (" against expert 0's weights" if kind == "grouped" else "")
               + f", N={N}, K={K}: {t:.2f} s")
     return {"value": value, "unit": unit, "cores": threads, "kind": "port", "sample": sample}
+
+
+def kernels_launched(kind, M, K, N):
+    """(name of the dominant kernel, description of every launch of the matmul), from the plan the library itself
+    reports for the shape (maxfp8_matmul_describe)."""
+    if kind == "rmsq":
+        return "rmsnorm_quant_row_bf16_kernel", "one launch"
+    if kind == "grouped":
+        return "gemm_grouped_kernel", ("gemm_grouped_large_kernel (full 256-row tiles of experts with >= 1024 rows) + "
+                                       "gemm_grouped_kernel (the rest), side by side on two streams")
+    from modular_amd import _lib
+    plan = _lib.matmul_describe(M, N, K, kind == "block", True)
+    first = plan.split(" + ")[0]
+    if plan.startswith("skinny"):
+        return "gemm_skinny_kernel", plan
+    if "persistent" in first:
+        return "gemm_persist_kernel", plan
+    if "stream-K" in first:
+        return "gemm_streamk_kernel", plan
+    return "gemm_tiled_kernel", plan
 
 
 def result_line(name, steps, warmup, with_cpu=True):
@@ -307,20 +335,18 @@ def result_line(name, steps, warmup, with_cpu=True):
         value, unit = flops / (ms_step * 1e-3) / 1e12, "TFLOP/s"
         roof = {"bound": "mfma", "achieved": flops / (mm_avg * 1e-3) / 1e12, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = measured_traffic(name)
-    roof["algorithmic_bytes"] = mm_bytes
-    roof["kernel"] = {"grouped": "gemm_grouped_kernel", "row": "gemm_skinny_kernel", "rmsq": "rmsnorm_quant_row_bf16_kernel"}.get(
-        kind, "gemm_skinny_kernel" if M <= 64 else "gemm_tiled_kernel")
-    # the matmul can be more than one launch (two regions in different tile shapes; the grouped matmul's
-    # large-tile launch and the rest): kernel_ms_* is the time of all of them, one after the other
     if kind == "grouped":
-        roof["launches"] = ("gemm_grouped_large_kernel (full 256-row tiles of experts with >= 1024 rows) + gemm_grouped_kernel "
-                            "(the rest), side by side on two streams")
-    elif kind in ("block", "row") and M > 64:
-        from modular_amd import _lib
-        roof["launches"] = _lib.matmul_describe(M, N, K, kind == "block", True)
-        if roof["launches"].split(" + ")[0].endswith("persistent"):
-            roof["kernel"] = "gemm_persist_kernel"
+        # the grouped matmul is priced against both roofs: 2 * T * N * K flops of real rows, and the weights of the
+        # experts in use streamed once
+        roof["frac_mfma"] = flops / (mm_avg * 1e-3) / 1e12 / PEAK_FP8_TFLOPS
+        roof["frac_hbm"] = mm_bytes / (mm_avg * 1e-3) / 1e9 / PEAK_HBM_GBS
+    roof["traffic"] = measured_traffic(name)
+    roof["traffic_source"] = ("profiles/hbm_traffic_pmc.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
+                              "scaled by the copy kernel; a committed figure, not a value of this run")
+    roof["algorithmic_bytes"] = mm_bytes
+    # the matmul can be more than one launch (two regions in different tile shapes; the grouped matmul's
+    # large-tile launch and the rest): kernel_ms_* is the time of all of them
+    roof["kernel"], roof["launches"] = kernels_launched(kind, M, K, N)
     roof["kernel_ms_avg"], roof["kernel_ms_median"], roof["kernel_ms_min"] = mm_avg, mm_med, mm_min
     out = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -331,7 +357,10 @@ def result_line(name, steps, warmup, with_cpu=True):
                               "per-token x per-channel" if kind == "row" else "1x128 activations, 128x128 weights",
                    "step": "RMSNorm fused with dynamic quantise" if kind == "rmsq" else
                            "dynamic quantise + " + ("grouped " if kind == "grouped" else "") + "scaled matmul",
-                   "input_copies": wl.copies, "settle_s": SETTLE_S},
+                   "input_copies": wl.copies, "settle_s": SETTLE_S,
+                   "timing": "value: host clock around the steps (quantise + matmul); roofline: events around the matmul "
+                             "launches alone in passes of their own -- the passes differ by a few per cent, so "
+                             "ms_per_step is not kernel_ms_avg plus the quantiser"},
         "roofline": roof,
     }
     if with_cpu:
@@ -345,7 +374,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help=f"one workload alone (default: {DEFAULT}, with a 'decode' record for {DEFAULT_DECODE})")
     ap.add_argument("--settle", type=float, default=SETTLE_S,
                     help="seconds the workload runs, untimed, before the warm-up steps (clock ramp of an idle GPU)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
@@ -385,7 +415,15 @@ def main():
         for _ in range(3):
             kernels.copy_bytes(dst, src)
         torch.cuda.synchronize()
-    print(json.dumps(result_line(args.workload, args.steps, args.warmup, with_cpu=not args.no_cpu)))
+    if args.workload is not None:
+        print(json.dumps(result_line(args.workload, args.steps, args.warmup, with_cpu=not args.no_cpu)))
+        return
+    line = result_line(DEFAULT, args.steps, args.warmup, with_cpu=not args.no_cpu)
+    torch.cuda.empty_cache()
+    # the HBM half of the metric: same fields, its own timed region (more steps: a launch takes ~75 microseconds)
+    dec = result_line(DEFAULT_DECODE, max(args.steps, 200), args.warmup, with_cpu=False)
+    line["decode"] = {k: dec[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "config", "roofline")}
+    print(json.dumps(line))
 
 
 if __name__ == "__main__":

@@ -62,11 +62,19 @@ typedef enum maxfp8_algo {
   MAXFP8_ALGO_AUTO = 0,
   MAXFP8_ALGO_NAIVE = 1,  /* one thread per output, reference summation order */
   MAXFP8_ALGO_TILED = 2,  /* LDS-staged MFMA tiles                            */
-  MAXFP8_ALGO_SKINNY = 3  /* weight-streaming kernel for M <= 16              */
+  MAXFP8_ALGO_SKINNY = 3  /* weight-streaming kernel for M <= 64              */
 } maxfp8_algo;
 
 const char* maxfp8_last_error(void);
 const char* maxfp8_version(void);
+
+/*
+ * The kernel selection reads its tuning switches (MAXFP8_TILE, MAXFP8_SPLITK, MAXFP8_SKINNY, ...;
+ * the list is in modular_amd/csrc/tuning.h) from the environment once per process.  This call
+ * reads them again: for tuning runs and tests that change a switch between calls.  No counterpart
+ * in the reference.
+ */
+void maxfp8_tuning_reload(void);
 
 /*
  * Dynamic activation quantisation.
@@ -148,7 +156,9 @@ int maxfp8_batched_quantize_dynamic_scaled_fp8(
  *       C[m,n] = (sum_k A[m,k] B[n,k]) * a_scales[m] * b_scales[n]
  *   input TENSOR, weight TENSOR: a_scales[0], b_scales[0].
  *
- *   scales_dtype MAXFP8_F32 (block requires it) or MAXFP8_BF16 (rowwise/tensor).
+ *   scales_dtype MAXFP8_F32 (block requires it), or MAXFP8_BF16 / MAXFP8_F16 for rowwise / tensor scales
+ *               (the reference's three scale dtypes, fp8_quantization.mojo:996-1018): widened to f32
+ *               when the epilogue loads them, on every kernel.
  *   algo        a maxfp8_algo value.
  *   workspace   optional device scratch for split-K, 16-byte aligned, of
  *               workspace_bytes bytes (maxfp8_matmul_workspace_bytes gives the

@@ -13,8 +13,8 @@ from .kernels import (grouped_matmul_rowwise_dynamic_scaled_fp8, fused_qkv_ragge
                       quantize_static_scaled_float8, quantize_tensor_dynamic_scaled_float8,
                       quantize_dynamic_scaled_float8, rms_norm_fused_quantize_dynamic_scaled_fp8)
 from .moe_kernels import fused_silu, fused_silu_quantized, moe_create_indices
-from .moe import expert_matmuls_fp8
-from .quant_ops import matmul_float8, quantized_fused_qkv_matmul, quantized_matmul
+from .moe import Fp8Strategy, expert_matmuls_fp8
+from .quant_ops import matmul_float8, quantized_fused_qkv_matmul, quantized_grouped_matmul, quantized_matmul
 from .linear import MLP, Linear
 from .weights_quant import parse_quant_config
 
@@ -28,4 +28,5 @@ __all__ = [
     "batched_dynamic_scaled_fp8_matmul", "batched_quantize_dynamic_scaled_fp8",
     "quantize_tensor_dynamic_scaled_float8", "fused_qkv_ragged_matmul_scaled_float8",
     "matmul_k_cache_ragged_scaled_float8", "KVCacheParams", "PagedCacheValues", "quantized_fused_qkv_matmul", "grouped_matmul_rowwise_dynamic_scaled_fp8", "expert_matmuls_fp8",
+    "Fp8Strategy", "quantized_grouped_matmul",
 ]

@@ -23,6 +23,7 @@ OK, ERR_DTYPE, ERR_SHAPE, ERR_ALIGN, ERR_GRANULARITY, ERR_LAUNCH, ERR_NULL, ERR_
 EXPORTS = (
     "maxfp8_last_error",
     "maxfp8_version",
+    "maxfp8_tuning_reload",
     "maxfp8_quantize_dynamic_scaled_fp8",
     "maxfp8_batched_quantize_dynamic_scaled_fp8",
     "maxfp8_quantize_dynamic_scaled_fp8_gather",
@@ -67,6 +68,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_last_error.argtypes = []
     L.maxfp8_version.restype = ctypes.c_char_p
     L.maxfp8_version.argtypes = []
+    L.maxfp8_tuning_reload.restype = None
+    L.maxfp8_tuning_reload.argtypes = []
     L.maxfp8_quantize_dynamic_scaled_fp8.restype = ci
     L.maxfp8_quantize_dynamic_scaled_fp8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, cf, vp]
     L.maxfp8_quantize_dynamic_scaled_fp8_gather.restype = ci
@@ -127,6 +130,11 @@ def check(status: int) -> None:
     if status in (ERR_SHAPE, ERR_ALIGN, ERR_GRANULARITY, ERR_NULL, ERR_WORKSPACE):
         raise ValueError(msg)
     raise RuntimeError(msg)
+
+
+def tuning_reload() -> None:
+    """Re-reads the MAXFP8_* tuning switches from the environment (they are read once per process otherwise)."""
+    lib().maxfp8_tuning_reload()
 
 
 def matmul_describe(M: int, N: int, K: int, block_scaling: bool = True, with_workspace: bool = True) -> str:

@@ -1,9 +1,14 @@
 // C ABI of the library (include/maxfp8.h): argument checks, kernel selection, error text.
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
+
+#include <atomic>
+#include <mutex>
 
 #include "common.h"
 #include "gemm_args.h"
+#include "tuning.h"
 
 namespace maxfp8 {
 
@@ -42,7 +47,7 @@ int naive_blockwise_dispatch(void*, const void*, const void*, const void*, const
 int naive_rowwise_dispatch(void*, const void*, const void*, const void*, const void*, int64_t, int64_t, int64_t,
                            int64_t, int64_t, int64_t, int64_t, int64_t, int, int, hipStream_t);
 int naive_grouped_dispatch(void*, const void*, const void*, const void*, const void*, const uint32_t*,
-                           const int32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int, hipStream_t);
+                           const int32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, hipStream_t);
 int gemm_tiled_dispatch(const GemmArgs&, bool, size_t, int64_t, hipStream_t);
 size_t gemm_tiled_workspace_bytes(int64_t, int64_t, int64_t);
 int gemm_tiled_describe(int64_t, int64_t, int64_t, bool, bool, char*, size_t);
@@ -68,6 +73,56 @@ static float round_to_dtype(float v, int dtype) {
 
 static bool is_aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+// The MFMA kernels address a tile's operands with 32-bit buffer offsets whose top bit marks lanes that are out of
+// range: the rows of the tallest tile (256) times the row stride, and the activation scales of all slabs of a tile
+// (ceil(K / 128) rows of a_scales_ld floats), must stay below 2^31 bytes.
+static bool offsets_fit(int64_t K, int64_t lda, int64_t ldb, int64_t a_scales_ld, bool block) {
+  const int64_t lim = (int64_t)1 << 31;
+  if (256 * lda + K >= lim || 256 * ldb + K >= lim) return false;
+  return !block || (ceil_div(K, 128) * a_scales_ld + 256) * 4 < lim;
+}
+
+// ---- tuning switches: one immutable snapshot of the environment, replaced as a whole by a reload ----
+static std::atomic<const Tuning*> g_tuning{nullptr};
+static std::mutex g_tuning_mu;
+
+static const Tuning* read_tuning(unsigned generation) {
+  Tuning* t = new Tuning();
+  auto num = [](const char* name, int dflt) { const char* e = getenv(name); return e ? atoi(e) : dflt; };
+  const int tile = num("MAXFP8_TILE", 0);
+  t->tile = (tile >= 1 && tile <= 4) ? tile : 0;
+  t->splitk = num("MAXFP8_SPLITK", 0);
+  t->one_region = getenv("MAXFP8_ONE_REGION") != nullptr;
+  t->persist = num("MAXFP8_PERSIST", 1) != 0;
+  t->streamk = num("MAXFP8_STREAMK", 1) != 0;
+  t->big_rows = num("MAXFP8_BIG_ROWS", 1024);
+  t->grouped_overlap = num("MAXFP8_GROUPED_OVERLAP", 1) != 0;
+  const char* sb = getenv("MAXFP8_GROUPED_SHARE");
+  t->grouped_share = sb ? (float)atof(sb) : 0.5f;
+  t->skinny = num("MAXFP8_SKINNY", 0);
+  t->generation = generation;
+  return t;
+}
+
+const Tuning& tuning() {
+  const Tuning* t = g_tuning.load(std::memory_order_acquire);
+  if (t) return *t;
+  std::lock_guard<std::mutex> lock(g_tuning_mu);
+  t = g_tuning.load(std::memory_order_acquire);
+  if (!t) {
+    t = read_tuning(0);
+    g_tuning.store(t, std::memory_order_release);
+  }
+  return *t;
+}
+
+// (the old snapshot is left in place for threads that still read it: a few dozen bytes per reload)
+void tuning_reload() {
+  std::lock_guard<std::mutex> lock(g_tuning_mu);
+  const Tuning* old = g_tuning.load(std::memory_order_acquire);
+  g_tuning.store(read_tuning(old ? old->generation + 1 : 1), std::memory_order_release);
+}
+
 }  // namespace maxfp8
 
 using namespace maxfp8;
@@ -75,7 +130,8 @@ using namespace maxfp8;
 extern "C" {
 
 const char* maxfp8_last_error(void) { return g_error; }
-const char* maxfp8_version(void) { return "maxfp8 0.1 (gfx950)"; }
+const char* maxfp8_version(void) { return "maxfp8 0.2 (gfx950)"; }
+void maxfp8_tuning_reload(void) { tuning_reload(); }
 
 }  // extern "C"
 
@@ -262,15 +318,16 @@ static int matmul_common(void* c, const void* a, const void* b, const void* a_sc
     if (gm <= 0 || gn <= 0 || gk <= 0) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: block granularities must be positive");
     if (a_scales_ld < ceil_div(M, gm) || b_scales_ld < ceil_div(K, gk))
       MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: scale leading dimensions too small");
-  } else if (scales_dtype != MAXFP8_F32 && scales_dtype != MAXFP8_BF16) {
-    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "matmul: scales dtype %d is not f32 or bf16", scales_dtype);
+  } else if (scales_dtype != MAXFP8_F32 && scales_dtype != MAXFP8_BF16 && scales_dtype != MAXFP8_F16) {
+    // the three scale dtypes of the reference (fp8_quantization.mojo:996-1018)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "matmul: scales dtype %d is not f32, bf16 or f16", scales_dtype);
   }
 
-  // Fast kernels: f32 scales, 16-byte aligned rows, K a multiple of 16, and for
-  // block scaling the (1, 128, 128) granularity.
+  // Fast kernels: 16-byte aligned rows, K a multiple of 16, and for block scaling the
+  // (1, 128, 128) granularity.  (Row / tensor scales of any dtype are widened in the epilogue.)
   const bool fast_layout = is_aligned(a, 16) && is_aligned(b, 16) && lda % 16 == 0 && ldb % 16 == 0 && K % 16 == 0 &&
-                           K > 0 && scales_dtype == MAXFP8_F32 && (!block || (gm == 1 && gn == 128 && gk == 128)) &&
-                           (bt.n == 1 || (bt.a % 16 == 0 && bt.b % 16 == 0));
+                           K > 0 && (!block || (gm == 1 && gn == 128 && gk == 128)) &&
+                           (bt.n == 1 || (bt.a % 16 == 0 && bt.b % 16 == 0)) && offsets_fit(K, lda, ldb, a_scales_ld, block);
   if (algo == MAXFP8_ALGO_AUTO) {
     if (!fast_layout) algo = MAXFP8_ALGO_NAIVE;
     else if (gemm_skinny_preferred(M, N, K)) algo = MAXFP8_ALGO_SKINNY;
@@ -292,7 +349,8 @@ static int matmul_common(void* c, const void* a, const void* b, const void* a_sc
   if (algo != MAXFP8_ALGO_TILED && algo != MAXFP8_ALGO_SKINNY) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "matmul: unknown algo %d", algo);
   if (!fast_layout)
     MAXFP8_FAIL(MAXFP8_ERR_ALIGN,
-                "matmul: the MFMA kernels need 16-byte aligned rows, K %% 16 == 0, f32 scales and (1,128,128) blocks");
+                "matmul: the MFMA kernels need 16-byte aligned rows, K %% 16 == 0, (1,128,128) blocks and "
+                "row strides below 2^31 / 256 bytes");
 
   GemmArgs p;
   memset(&p, 0, sizeof(p));
@@ -308,6 +366,7 @@ static int matmul_common(void* c, const void* a, const void* b, const void* a_sc
   p.a_scale_stride = tensor ? 0 : 1;
   p.b_scale_stride = tensor ? 0 : b_scales_ld;
   p.c_dtype = c_dtype;
+  p.scales_dtype = scales_dtype;  // (f32 for block scaling, checked above)
   p.c_vec_ok = (ldc % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
   p.c_vec8_ok = (ldc % 8 == 0) && is_aligned(c, 16);
   if (bt.n != 1) {  // every batch's C must keep the alignment the vector stores assume
@@ -394,6 +453,8 @@ int maxfp8_fused_qkv_matmul_ragged_paged_scale(void* output, const void* input, 
   // the MFMA kernels' layout, and 8-element chunks that stay inside one of Q / K / V and one cache row
   if (!is_aligned(input, 16) || !is_aligned(wqkv, 16) || K % 16 != 0 || K <= 0)
     MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "fused qkv matmul: needs 16-byte aligned rows and K %% 16 == 0");
+  if (!offsets_fit(K, K, K, input_scale_ld, block))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused qkv matmul: K = %lld is too long for the kernels' 32-bit tile offsets", (long long)K);
   if (q_dim % 8 != 0 || k_dim % 8 != 0 || !is_aligned(kv_blocks, 16) || (q_dim > 0 && !is_aligned(output, 16)))
     MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "fused qkv matmul: q_dim and kv_heads * head_dim must be multiples of 8, buffers 16-byte aligned");
 
@@ -411,6 +472,7 @@ int maxfp8_fused_qkv_matmul_ragged_paged_scale(void* output, const void* input, 
   p.a_scale_stride = per_tensor ? 0 : 1;
   p.b_scale_stride = per_tensor ? 0 : weight_scale_ld;
   p.c_dtype = MAXFP8_BF16;
+  p.scales_dtype = MAXFP8_F32;
   p.c_vec_ok = 1;
   p.c_vec8_ok = 1;
   p.kv_on = 1;
@@ -463,12 +525,12 @@ static int grouped_block_common(void* c, const uint32_t* c_row_index, const void
   if (!c || !a || !b || !a_scales || !b_scales || !expert_start_indices || !expert_ids)
     MAXFP8_FAIL(MAXFP8_ERR_NULL, "grouped matmul: null pointer");
   hipStream_t st = (hipStream_t)stream;
-  const bool fast_layout = is_aligned(a, 16) && is_aligned(b, 16) && K % 16 == 0 && K > 0;
+  const bool fast_layout = is_aligned(a, 16) && is_aligned(b, 16) && K % 16 == 0 && K > 0 && offsets_fit(K, K, K, a_scales_ld, true);
   if (algo == MAXFP8_ALGO_AUTO) algo = fast_layout ? MAXFP8_ALGO_TILED : MAXFP8_ALGO_NAIVE;
   if (algo == MAXFP8_ALGO_NAIVE && c_row_index)
     MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: the row scatter needs the MFMA kernel (16-byte aligned rows, K %% 16 == 0)");
   if (algo == MAXFP8_ALGO_NAIVE)
-    return naive_grouped_dispatch(c, a, b, a_scales, b_scales, expert_start_indices, expert_ids, N, K,
+    return naive_grouped_dispatch(c, a, b, a_scales, b_scales, expert_start_indices, expert_ids, T, N, K,
                                   max_num_tokens_per_expert, num_active_experts, a_scales_ld, c_dtype, st);
   if (algo != MAXFP8_ALGO_TILED) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped matmul: unknown algo %d", algo);
   if (!fast_layout) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "grouped matmul: the MFMA kernel needs 16-byte aligned rows and K %% 16 == 0");
@@ -485,6 +547,7 @@ static int grouped_block_common(void* c, const uint32_t* c_row_index, const void
   p.a_scales_ld = a_scales_ld;
   p.b_scales_ld = ceil_div(K, 128);
   p.c_dtype = c_dtype;
+  p.scales_dtype = MAXFP8_F32;
   p.c_vec_ok = (N % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
   p.c_vec8_ok = (N % 8 == 0) && is_aligned(c, 16);
   p.offsets = expert_start_indices;
@@ -542,6 +605,8 @@ int maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8(void* c, const void* a, con
     MAXFP8_FAIL(MAXFP8_ERR_NULL, "grouped rowwise matmul: null pointer");
   if (!(is_aligned(a, 16) && is_aligned(b, 16) && K % 16 == 0 && K > 0))
     MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "grouped rowwise matmul: needs 16-byte aligned rows and K %% 16 == 0");
+  if (!offsets_fit(K, K, K, 0, false))
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "grouped rowwise matmul: K = %lld is too long for the kernels' 32-bit tile offsets", (long long)K);
   GemmArgs p;
   memset(&p, 0, sizeof(p));
   p.a = (const uint8_t*)a;
@@ -554,6 +619,7 @@ int maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8(void* c, const void* a, con
   p.a_scale_stride = 1;
   p.b_scale_stride = 1;
   p.c_dtype = c_dtype;
+  p.scales_dtype = MAXFP8_F32;
   p.c_vec_ok = (N % 4 == 0) && is_aligned(c, c_dtype == MAXFP8_BF16 ? 8 : 16);
   p.c_vec8_ok = (N % 8 == 0) && is_aligned(c, 16);
   p.offsets = expert_start_indices;

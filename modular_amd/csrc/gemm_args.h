@@ -36,6 +36,7 @@ struct GemmArgs {
   int64_t a_scales_ld, b_scales_ld;
   int64_t a_scale_stride, b_scale_stride;
   int c_dtype;
+  int scales_dtype;        // row / tensor scaling: MAXFP8_F32, MAXFP8_BF16 or MAXFP8_F16 (block scaling is always f32)
   int c_vec_ok;            // C base and ldc allow 4-element vector stores
   int c_vec8_ok;           // ... and 8-element ones (16-byte aligned rows)
   // grouped only
@@ -61,6 +62,15 @@ struct GemmArgs {
 };
 
 #if defined(__HIPCC__)
+// Element idx of a row / tensor scale vector of the given dtype, widened to f32 (exact): how the reference's
+// epilogue reads its scales (max/kernels/src/linalg/fp8_quantization.mojo:1218-1240: load, cast, multiply in f32).
+__device__ __forceinline__ float scale_at(const float* base, int64_t idx, int dtype) {
+  if (dtype == 2 /* MAXFP8_F32 */) return base[idx];
+  const uint16_t h = reinterpret_cast<const uint16_t*>(base)[idx];
+  if (dtype == 0 /* MAXFP8_BF16 */) return __uint_as_float((uint32_t)h << 16);
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+
 // offsets (elements from k_base / v_base) of the cache rows that receive rows m[0..R); -1 for a
 // row that is not live or that the lookup table has no page for (nothing is stored then).  The R
 // binary searches run in lockstep with a trip count that only depends on the batch size, so

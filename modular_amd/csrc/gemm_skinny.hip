@@ -28,6 +28,7 @@
 
 #include "common.h"
 #include "gemm_args.h"
+#include "tuning.h"
 
 namespace maxfp8 {
 
@@ -256,12 +257,12 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
       continue;
     }
     if constexpr (!BLOCKSCALE) {
-      const float a_s = p.a_scales[(int64_t)m * p.a_scale_stride];
+      const float a_s = scale_at(p.a_scales, (int64_t)m * p.a_scale_stride, p.scales_dtype);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int nn = (n + i < p.N) ? n + i : p.N - 1;
         const float t = v[i] * a_s;
-        v[i] = t * p.b_scales[(int64_t)nn * p.b_scale_stride];
+        v[i] = t * scale_at(p.b_scales, (int64_t)nn * p.b_scale_stride, p.scales_dtype);
       }
     }
     if (p.c_dtype == MAXFP8_BF16) {
@@ -312,7 +313,7 @@ static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream)
 // 32-row blocks keep 16 KB per wave in flight when M <= 16 and the weights exceed 256 MB, else 8 KB.
 // (8 waves per block were tried for the small-N shapes and were no faster.)  Every shape splits K over its four waves
 // in the same way and adds the partial sums in the same order: the result does not depend on the choice.
-// MAXFP8_SKINNY=<ntw>4<ringKB>, e.g. 1408 or 2416, forces a shape for tuning runs.
+// The tuning switch `skinny` = <ntw>4<ringKB>, e.g. 1408 or 2416, forces a shape for tuning runs.
 int compute_units();
 static int skinny_shape(int64_t M, int64_t N, int64_t K) {
   const int64_t cus = compute_units();
@@ -332,8 +333,7 @@ static int skinny_shape(int64_t M, int64_t N, int64_t K) {
 
 template <int MT, bool BLOCKSCALE>
 static int pick_ntw(const GemmArgs& p, int64_t batch, hipStream_t stream) {
-  const char* e = getenv("MAXFP8_SKINNY");
-  int sel = e ? atoi(e) : 0;
+  int sel = tuning().skinny;
   if (!sel) sel = skinny_shape(p.M, p.N, p.K);
   switch (sel) {
     case 1408: return launch_skinny_r<1, MT, BLOCKSCALE, 8, 4>(p, batch, stream);

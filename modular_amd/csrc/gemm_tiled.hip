@@ -44,6 +44,7 @@
 #include <utility>
 #include "common.h"
 #include "gemm_args.h"
+#include "tuning.h"
 
 namespace maxfp8 {
 
@@ -268,10 +269,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     // duration, and since the barrier lines all waves up, the matrix pipe idles meanwhile.
     const uint32_t dead = slab + NS - 1 < slab_end ? 0u : 0x80000000u;
     const int dma_slab = slab + NS - 1, dma_buf = buf == 0 ? NS - 1 : buf - 1;
-#ifndef MAXFP8_DMA_SPREAD
-#define MAXFP8_DMA_SPREAD (NS == 2 && TM >= 4 ? TM / 2 : TM)
-#endif
-    constexpr int SPREAD = MAXFP8_DMA_SPREAD < 1 ? 1 : (MAXFP8_DMA_SPREAD > TM ? TM : MAXFP8_DMA_SPREAD);
+    constexpr int SPREAD = (NS == 2 && TM >= 4) ? TM / 2 : TM;
 
     const uint8_t* sa = smem + buf * STAGE_BYTES;
     float s_cur[TM];
@@ -321,9 +319,6 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
 #pragma unroll
       for (int idx = 0; idx < PER; ++idx)
         if (idx * SPREAD / PER == mt) dma_one(dma_slab, dma_buf, idx, dead);
-#ifdef MAXFP8_SCHED_BARRIER
-      __builtin_amdgcn_sched_barrier(0);
-#endif
     }
     buf = buf + 1 == NS ? 0 : buf + 1;
   }
@@ -510,7 +505,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
         float a_s = 1.f;
         if constexpr (!BLOCKSCALE) {
           const int64_t mm = row_begin + wm * WM + r;
-          a_s = p.a_scales[(mm < p.M ? mm : p.M - 1) * p.a_scale_stride];
+          a_s = scale_at(p.a_scales, (mm < p.M ? mm : p.M - 1) * p.a_scale_stride, p.scales_dtype);
         }
 #pragma unroll
         for (int q = 0; q < TN / 2; ++q) {
@@ -520,8 +515,8 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
-              lo[i] = t_lo * p.b_scales[(int64_t)(n + i) * p.b_scale_stride];
-              hi[i] = t_hi * p.b_scales[(int64_t)(n + 4 + i) * p.b_scale_stride];
+              lo[i] = t_lo * scale_at(p.b_scales, (int64_t)(n + i) * p.b_scale_stride, p.scales_dtype);
+              hi[i] = t_hi * scale_at(p.b_scales, (int64_t)(n + 4 + i) * p.b_scale_stride, p.scales_dtype);
             }
           }
           const int chunk = (q * 4 + lq) ^ (r & 7);
@@ -550,7 +545,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     if constexpr (GROUPED)
       if (p.c_row_index) cm = p.c_row_index[m];
     float a_s = 1.f;
-    if constexpr (!BLOCKSCALE) a_s = p.a_scales[m * p.a_scale_stride];
+    if constexpr (!BLOCKSCALE) a_s = scale_at(p.a_scales, m * p.a_scale_stride, p.scales_dtype);
 #pragma unroll
     for (int q = 0; q < TN / 2; ++q) {
       const int n = n0 + wn * WN + q * 32 + lq * 8;
@@ -562,8 +557,8 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
           const int n_lo = (n + i < p.N) ? n + i : p.N - 1;
           const int n_hi = (n + 4 + i < p.N) ? n + 4 + i : p.N - 1;
           const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
-          lo[i] = t_lo * bs_ptr[(int64_t)n_lo * p.b_scale_stride];  // (bs_ptr: this expert's scales when grouped)
-          hi[i] = t_hi * bs_ptr[(int64_t)n_hi * p.b_scale_stride];
+          lo[i] = t_lo * scale_at(bs_ptr, (int64_t)n_lo * p.b_scale_stride, p.scales_dtype);  // (bs_ptr: this expert's scales when grouped)
+          hi[i] = t_hi * scale_at(bs_ptr, (int64_t)n_hi * p.b_scale_stride, p.scales_dtype);
         }
       }
       store8(cm, n, lo, hi);
@@ -825,10 +820,10 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
       for (int q = 0; q < TN / 2; ++q)
 #pragma unroll
         for (int i = 0; i < 8; ++i)
-          b_s[q][i] = p.b_scales[(int64_t)(tn * BN + wn * WN + q * 32 + lq * 8 + i) * p.b_scale_stride];
+          b_s[q][i] = scale_at(p.b_scales, (int64_t)(tn * BN + wn * WN + q * 32 + lq * 8 + i) * p.b_scale_stride, p.scales_dtype);
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt)
-        a_s_all[mt] = p.a_scales[((int64_t)tm * BM + wm * WM + mt * 16 + lm) * p.a_scale_stride];
+        a_s_all[mt] = scale_at(p.a_scales, ((int64_t)tm * BM + wm * WM + mt * 16 + lm) * p.a_scale_stride, p.scales_dtype);
       asm volatile("" ::: "memory");
     }
     // (C goes out through a buffer descriptor: one 32-bit lane offset for all of a lane's stores, the rest scalar)
@@ -883,6 +878,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_persist_kernel(
 // Slot z owns rows [offsets[z], offsets[z+1]).  blockIdx.y counts row tiles over all slots,
 // blockIdx.x is the column tile; a block finds its (slot, tile) with a block-wide prefix sum of
 // tiles_of(slot) over the device-resident offsets: no host synchronisation, no list of tiles.
+// Rows [begin, end) of slot z, held inside [0, M): the activations, their scales and C have M rows, so offsets
+// beyond that (a stale or damaged routing tensor) must not turn into accesses outside them.
+__device__ __forceinline__ void grouped_slot_rows(const GemmArgs& p, int z, int64_t& begin, int64_t& end) {
+  const int64_t M = p.M, b = p.offsets[z], e = p.offsets[z + 1];
+  begin = b < M ? b : M;
+  end = e < M ? e : M;
+  if (end < begin) end = begin;
+}
+__device__ __forceinline__ int grouped_slot_count(const GemmArgs& p, int z) {
+  int64_t b, e;
+  grouped_slot_rows(p, z, b, e);
+  return (int)(e - b);
+}
+
 template <int NWAVES, typename TilesOf>
 __device__ __forceinline__ bool grouped_find_tile(const GemmArgs& p, const int by, TilesOf tiles_of, int& slot, int& tile) {
   constexpr int NTHREADS = NWAVES * 64;
@@ -894,7 +903,7 @@ __device__ __forceinline__ bool grouped_find_tile(const GemmArgs& p, const int b
   for (int z0 = 0; z0 < p.num_active; z0 += NTHREADS) {
     const int z = z0 + tid;
     int t = 0;
-    if (z < p.num_active) t = tiles_of((int)(p.offsets[z + 1] - p.offsets[z]));
+    if (z < p.num_active) t = tiles_of(grouped_slot_count(p, z));
     int incl = t;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
@@ -951,7 +960,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
     return rows <= p.small_rows ? (rows > 0 ? 1 : 0) : (rows + BM - 1) / BM;
   }, slot, tile);
   if (!found) return;
-  const int64_t slot_begin = p.offsets[slot], row_end = p.offsets[slot + 1];
+  int64_t slot_begin, row_end;
+  grouped_slot_rows(p, slot, slot_begin, row_end);
   const int64_t rest_begin = slot_begin + grouped_head_rows(p, (int)(row_end - slot_begin));
   const int64_t row_begin = rest_begin + (int64_t)tile * BM;
   const bool small = row_end - row_begin <= p.small_rows;  // also the last tile of a longer slot, when few rows are left for it
@@ -989,7 +999,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_k
     __syncthreads();
     int big = 0, mid = 0, tiny = 0;
     for (int z = threadIdx.x; z < p.num_active; z += NWAVES * 64) {
-      const int rows = (int)(p.offsets[z + 1] - p.offsets[z]);
+      const int rows = grouped_slot_count(p, z);
       const int head = grouped_head_rows(p, rows), rest = rows - head;
       big += head / BM;
       if (rest > p.small_rows) mid += (rest + 127) / 128;
@@ -1017,7 +1027,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_k
     const int by = t / ncol, bx = t - by * ncol;
     int slot, tile;
     if (!grouped_find_tile<NWAVES>(p, by, [&](int rows_total) { return grouped_head_rows(p, rows_total) / BM; }, slot, tile)) return;
-    const int64_t row_begin = (int64_t)p.offsets[slot] + (int64_t)tile * BM;
+    int64_t slot_begin, slot_end;
+    grouped_slot_rows(p, slot, slot_begin, slot_end);
+    const int64_t row_begin = slot_begin + (int64_t)tile * BM;  // (a full tile of the slot: row_begin + BM <= slot_end <= M)
     const int n0 = bx * BN;
     const int e = p.expert_ids[slot];
     if (e < 0) {
@@ -1074,10 +1086,9 @@ static int launch_grouped_large(const GemmArgs& p, dim3 grid, hipStream_t stream
 
 // The persistent kernel takes matmuls of whole 256 x 256 tiles with 16-byte aligned bf16 rows of C, one launch,
 // no K split, and operands whose byte offsets fit 31 bits (a tile's position rides in the copies' scalar offset).
-// MAXFP8_PERSIST=0 switches it off (A/B runs).
+// (The tuning switch `persist` turns it off for A/B runs.)
 static bool persist_shape(int64_t M, int64_t N, int variant) {
-  const char* e = getenv("MAXFP8_PERSIST");
-  if (e && atoi(e) == 0) return false;
+  if (!tuning().persist) return false;
   return variant == 1 && M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0;
 }
 static bool persist_ok(const GemmArgs& p, bool blockscale, dim3 grid) {
@@ -1150,11 +1161,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
       const int64_t m = i / p.N;
       const int64_t n = i - m * p.N;
       if constexpr (!BLOCKSCALE) {
-        const float a_s = p.a_scales[m * p.a_scale_stride];
+        const float a_s = scale_at(p.a_scales, m * p.a_scale_stride, p.scales_dtype);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float r = v[j] * a_s;
-          v[j] = r * p.b_scales[(n + j) * p.b_scale_stride];
+          v[j] = r * scale_at(p.b_scales, (n + j) * p.b_scale_stride, p.scales_dtype);
         }
       }
       if (p.c_dtype == MAXFP8_BF16)
@@ -1168,8 +1179,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs p) {
       const int64_t n = (i + j) - m * p.N;
       float r = v[j];
       if constexpr (!BLOCKSCALE) {
-        r = r * p.a_scales[m * p.a_scale_stride];
-        r = r * p.b_scales[n * p.b_scale_stride];
+        r = r * scale_at(p.a_scales, m * p.a_scale_stride, p.scales_dtype);
+        r = r * scale_at(p.b_scales, n * p.b_scale_stride, p.scales_dtype);
       }
       if (p.c_dtype == MAXFP8_BF16) reinterpret_cast<uint16_t*>(p.c)[m * p.ldc + n] = (uint16_t)f32_to_bf16_bits(r);
       else reinterpret_cast<float*>(p.c)[m * p.ldc + n] = r;
@@ -1192,19 +1203,14 @@ static const TileShape kShapes[4] = {
     {128, 128, 256, 0.74f, 0.66f, 9.0f},    // 4 waves, 3 stages, one block per CU: problems of at most one round of such tiles
 };
 
-// MAXFP8_TILE=1/2/3 forces a shape (for tuning runs); anything else lets the cost model pick.
-static int tile_override() {
-  const char* e = getenv("MAXFP8_TILE");
-  const int v = e ? atoi(e) : 0;
-  return (v >= 1 && v <= 4) ? v : 0;
-}
+// the tuning switch `tile` forces a shape (tuning runs and tests); 0 lets the cost model pick
+static int tile_override() { return tuning().tile; }
 
 // Split-K: when the tiles of a matmul cover only part of the chip, K is cut into `splits` shares
 // (each at least 4 slabs) until the grid fills the resident-block slots.  Needs
 // splits * M * N * 4 bytes of workspace; without workspace the matmul runs unsplit.
 static int pick_splits(int64_t tiles, int slots, int nslab) {
-  const char* e = getenv("MAXFP8_SPLITK");
-  int splits = e ? atoi(e) : 0;
+  int splits = tuning().splitk;
   if (splits <= 0) {
     splits = 1;
     if (tiles * 2 <= slots) splits = (int)(slots / tiles);
@@ -1301,22 +1307,20 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
     const int sp = pick_splits(tiles, t.slots, nslab);
     if (sp > 1 && (size_t)sp * M * N * 4 <= workspace_bytes) plan.splits = sp;
   }
-  if (free_choice && batch == 1 && !kv_on && plan.splits == 1 && !getenv("MAXFP8_ONE_REGION"))
+  if (free_choice && batch == 1 && !kv_on && plan.splits == 1 && !tuning().one_region)
     plan.two = pick_two_regions(M, N, nslab, blockscale, region_cost(M, N, nslab, t, blockscale));
   return plan;
 }
 
 // make_plan tries every cut of every pair of shapes: microseconds of host time, as much as a small matmul
-// takes on the GPU.  Plans are kept in a small table, keyed by everything make_plan reads (the tuning
-// switches of the environment included, since tests and tuning runs flip them between calls).
+// takes on the GPU.  Plans are kept in a small table, keyed by everything make_plan reads (the generation
+// of the tuning switches included, since tests and tuning runs reload them between calls).
 static TiledPlan cached_plan(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, size_t workspace_bytes,
                              int64_t batch, bool kv_on) {
   struct Entry { int64_t M, N, K, batch; size_t ws; int flags; bool valid; TiledPlan plan; };
   static Entry table[128];
   static std::mutex mu;
-  const char* sk = getenv("MAXFP8_SPLITK");
-  const int flags = (blockscale ? 1 : 0) | (has_workspace ? 2 : 0) | (kv_on ? 4 : 0) | (getenv("MAXFP8_ONE_REGION") ? 8 : 0) |
-                    (tile_override() << 4) | ((sk ? atoi(sk) & 0xff : 0) << 8);
+  const int flags = (blockscale ? 1 : 0) | (has_workspace ? 2 : 0) | (kv_on ? 4 : 0) | (int)(tuning().generation << 3);
   const uint64_t h = ((uint64_t)M * 0x9e3779b97f4a7c15ull) ^ ((uint64_t)N * 0xc2b2ae3d27d4eb4full) ^ ((uint64_t)K * 0x165667b19e3779f9ull) ^
                      ((uint64_t)batch << 7) ^ (uint64_t)flags;
   Entry& e = table[(h >> 32) % 128];
@@ -1357,18 +1361,21 @@ int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_
     GemmArgs r1 = p, r2 = p;
     r1.splits = r2.splits = 1;
     const int64_t esz = p.c_dtype == MAXFP8_BF16 ? 2 : 4;
+    const int64_t ssz = p.scales_dtype == MAXFP8_F32 ? 4 : 2;  // (row / tensor scales; block scales are f32)
     if (two.axis == 1) {  // columns [0, cut) and [cut, N): weight rows, their scales, C columns
       r1.N = (int)two.cut;
       r2.N = p.N - (int)two.cut;
       r2.b = p.b + two.cut * p.ldb;
       r2.c = reinterpret_cast<uint8_t*>(p.c) + two.cut * esz;
-      r2.b_scales = blockscale ? p.b_scales + (two.cut / 128) * p.b_scales_ld : p.b_scales + two.cut * p.b_scale_stride;
+      r2.b_scales = blockscale ? p.b_scales + (two.cut / 128) * p.b_scales_ld
+                               : reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(p.b_scales) + two.cut * p.b_scale_stride * ssz);
     } else {              // rows [0, cut) and [cut, M): activation rows, their scales, C rows
       r1.M = (int)two.cut;
       r2.M = p.M - (int)two.cut;
       r2.a = p.a + two.cut * p.lda;
       r2.c = reinterpret_cast<uint8_t*>(p.c) + two.cut * p.ldc * esz;
-      r2.a_scales = blockscale ? p.a_scales + two.cut : p.a_scales + two.cut * p.a_scale_stride;
+      r2.a_scales = blockscale ? p.a_scales + two.cut
+                               : reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(p.a_scales) + two.cut * p.a_scale_stride * ssz);
     }
     const TileShape &ta = kShapes[two.v1 - 1], &tb = kShapes[two.v2 - 1];
     const dim3 g1((unsigned)(ceil_div(r1.M, ta.bm) * ceil_div(r1.N, ta.bn)), 1, 1);
@@ -1441,23 +1448,20 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int6
   // be any) hand their full 256-row tiles to a launch with 256 x 256 tiles; everything else --
   // their last rows, the other slots -- runs in 128 x 128 tiles, and in 32 x 128 tiles with a
   // third LDS stage where at most 32 rows are left.
-  // MAXFP8_TILE=2: 256-row tiles in one launch; 3: no small tiles; 4: no large-tile launch (tuning runs)
+  // tuning switch `tile` = 2: 256-row tiles in one launch; 3: no small tiles; 4: no large-tile launch
   const int tune = tile_override();
   const bool big = tune == 2;
   const int bm = big ? 256 : 128;
   p.small_rows = tune == 3 ? 0 : (big ? 64 : 32);
   p.big_rows = 0;
   p.big_bm = 256;
-  const int big_rows = getenv("MAXFP8_BIG_ROWS") ? atoi(getenv("MAXFP8_BIG_ROWS")) : 1024;
+  const int big_rows = tuning().big_rows;
   // The large-tile launch goes down a second stream, as a fixed set of blocks, so that its tiles (bound by the matrix
   // pipe) and the other launch's (mostly bound by HBM) share the chip instead of taking turns; the caller's stream
-  // waits for both.  MAXFP8_GROUPED_OVERLAP=0 keeps the two launches in line on the caller's stream.
+  // waits for both.  (The tuning switch `grouped_overlap` = 0 keeps the two launches in line on the caller's stream.)
   SideStream* side = nullptr;
   const bool large = !big && tune != 4 && max_tokens >= big_rows && T / 256 <= 65535;
-  if (large) {
-    const char* ov = getenv("MAXFP8_GROUPED_OVERLAP");
-    if (!(ov && atoi(ov) == 0)) side = side_stream();
-  }
+  if (large && tuning().grouped_overlap) side = side_stream();
   std::unique_lock<std::mutex> side_lock;
   if (large) {
     p.big_rows = big_rows;
@@ -1470,9 +1474,8 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int6
       side_lock = std::unique_lock<std::mutex>(side->mu);  // one fork / join at a time per device
       if (hipEventRecord(side->fork, stream) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
         MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "grouped matmul: cannot order the second stream behind the caller's: %s", hipGetErrorString(hipGetLastError()));
-      const char* sb = getenv("MAXFP8_GROUPED_SHARE");
       pl.big_tile_rows = (int)(T / 256);
-      pl.share_bias = sb ? (float)atof(sb) : 0.5f;  // (measured: the model overrates the other launch's need of CUs)
+      pl.share_bias = tuning().grouped_share;  // (0.5 measured: the model overrates the other launch's need of CUs)
       const int64_t pairs = (int64_t)lgrid.x * lgrid.y;
       const int cus = compute_units();
       lgrid = dim3((unsigned)(pairs < cus ? pairs : cus));

@@ -126,20 +126,38 @@ int moe_create_indices_dispatch(uint32_t* token_expert_order, uint32_t* expert_s
 }
 
 // ---- fused SiLU(gate) * up --------------------------------------------------------------------
-// a / b from the hardware reciprocal and one correction step: the correctly rounded quotient
-// except for rare double roundings, at a third of the instructions of the IEEE sequence (the
-// kernels below are bound by these divisions, not by memory, when they use that sequence)
-__device__ __forceinline__ float fast_div(float a, float b, float rcp_b) {
-  const float q = a * rcp_b;
+// a / b, correctly rounded (the IEEE quotient), at well under the cost of the IEEE sequence on the common path:
+// the hardware reciprocal and one correction step give a candidate q; its residual a - q * b is exact whenever q
+// is within an ulp of the quotient (and large otherwise), so
+//     residual == 0                        q is the exact quotient
+//     |residual| < ulp(q) / 2 * |b|        q is the one float nearest to a / b
+// accept q, and everything else -- ties, powers of two (whose lower neighbour is half an ulp away), tiny or huge
+// operands where the products above could underflow -- takes the IEEE division.  The slow path is a wave-uniform
+// branch: it is skipped unless some lane of the wave needs it.  (Checked against the IEEE quotient on 2e8 random
+// operand pairs with the reciprocal off by -1, 0 and +1 ulp: no difference.)
+__device__ __forceinline__ float exact_div(float a, float b, float rcp_b) {
+  float q = a * rcp_b;
   const float err = fmaf(-q, b, a);
-  return err == 0.0f ? q : fmaf(err, rcp_b, q);  // (keeps the sign of a zero quotient)
+  q = err == 0.0f ? q : fmaf(err, rcp_b, q);  // (keeps the sign of a zero quotient)
+  const float res = fmaf(-q, b, a);
+  const uint32_t qb = __float_as_uint(q), qe = qb & 0x7f800000u;
+  const uint32_t ae = __float_as_uint(a) & 0x7f800000u, be = __float_as_uint(b) & 0x7f800000u;
+  const float half_ulp_b = __uint_as_float(qe - (24u << 23)) * fabsf(b);
+  // (exponents between 2^-63 and 2^63: neither the residual nor the bound can underflow or overflow)
+  const bool b_ok = be >= (64u << 23) && be <= (190u << 23);
+  const bool aq_ok = ae >= (64u << 23) && qe >= (64u << 23) && qe <= (190u << 23);
+  const bool ok = b_ok && (a == 0.0f || (aq_ok && (res == 0.0f || ((qb & 0x007fffffu) != 0u && fabsf(res) < half_ulp_b))));
+  if (__builtin_amdgcn_ballot_w64(!ok) != 0ull) {
+    if (!ok) q = a / b;
+  }
+  return q;
 }
 
 __device__ __forceinline__ float silu_mul(float gate, float up) {
   // gate / (1 + exp(-gate)) * up, every step rounded to f32 (ep_comm.mojo:4494-4497)
   const float d = 1.0f + expf(-gate);
-  // d = inf (gate < -88): gate / inf = -0; the correction step would produce NaN there
-  const float sig = d > 3.0e38f ? -0.0f : fast_div(gate, d, __builtin_amdgcn_rcpf(d));
+  // d = inf (gate < -88): gate / inf = -0, written out (a residual against inf is NaN)
+  const float sig = d > 3.0e38f ? -0.0f : exact_div(gate, d, __builtin_amdgcn_rcpf(d));
   return sig * up;
 }
 
@@ -149,12 +167,15 @@ template <bool QUANT>
 __global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__ out, float* __restrict__ scales,
                                                               const uint16_t* __restrict__ in,
                                                               const uint32_t* __restrict__ row_offsets, int num_offsets,
-                                                              int inter, int64_t in_stride, int64_t out_stride,
-                                                              int64_t scales_ld) {
-  const uint32_t rows = row_offsets[num_offsets - 1];
+                                                              int64_t max_rows, int inter, int64_t in_stride,
+                                                              int64_t out_stride, int64_t scales_ld) {
+  // (the buffers hold max_rows rows: an offset beyond that -- a stale or damaged routing tensor -- must not
+  // turn into accesses outside them)
+  const uint32_t rows_dev = row_offsets[num_offsets - 1];
+  const int64_t rows = (int64_t)rows_dev < max_rows ? (int64_t)rows_dev : max_rows;
   const int groups = inter >> 7;
   const int tid = threadIdx.x, sub = tid & 15;
-  const int64_t total = (int64_t)rows * groups;
+  const int64_t total = rows * groups;
   for (int64_t item = (int64_t)blockIdx.x * 16 + (tid >> 4); item < total; item += (int64_t)gridDim.x * 16) {
     const int64_t m = item / groups;
     const int g = (int)(item - m * groups);
@@ -183,7 +204,7 @@ __global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__
       const float rs = __builtin_amdgcn_rcpf(scale);
       float q[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) q[j] = clamp448(fast_div(f[j], scale, rs));
+      for (int j = 0; j < 8; ++j) q[j] = clamp448(exact_div(f[j], scale, rs));
       int lo = 0, hi = 0;
       lo = cvt_pk_e4m3fn(q[0], q[1], lo, false);
       lo = cvt_pk_e4m3fn(q[2], q[3], lo, true);
@@ -205,10 +226,10 @@ int fused_silu_dispatch(void* out, float* scales, const void* in, const uint32_t
   const unsigned blocks = (unsigned)(ceil_div(items, 16) < 8192 ? ceil_div(items, 16) : 8192);
   if (quant)
     hipLaunchKernelGGL(fused_silu_bf16_kernel<true>, dim3(blocks), dim3(256), 0, stream, out, scales, (const uint16_t*)in,
-                       row_offsets, (int)num_offsets, (int)inter, in_stride, out_stride, scales_ld);
+                       row_offsets, (int)num_offsets, max_rows, (int)inter, in_stride, out_stride, scales_ld);
   else
     hipLaunchKernelGGL(fused_silu_bf16_kernel<false>, dim3(blocks), dim3(256), 0, stream, out, scales, (const uint16_t*)in,
-                       row_offsets, (int)num_offsets, (int)inter, in_stride, out_stride, scales_ld);
+                       row_offsets, (int)num_offsets, max_rows, (int)inter, in_stride, out_stride, scales_ld);
   return launch_status(quant ? "fused_silu_quantized" : "fused_silu");
 }
 

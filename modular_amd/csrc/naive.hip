@@ -19,8 +19,9 @@ __device__ __forceinline__ void store_out(void* c, int c_dtype, int64_t idx, flo
 }
 
 __device__ __forceinline__ float load_scale(const void* s, int dtype, int64_t idx) {
-  return dtype == MAXFP8_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(s)[idx])
-                              : reinterpret_cast<const float*>(s)[idx];
+  if (dtype == MAXFP8_BF16) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(s)[idx]);
+  if (dtype == MAXFP8_F16) return (float)reinterpret_cast<const _Float16*>(s)[idx];
+  return reinterpret_cast<const float*>(s)[idx];
 }
 
 __device__ __forceinline__ float blockwise_dot(const uint8_t* ar, const uint8_t* br, const float* a_scales,
@@ -74,10 +75,12 @@ __global__ __launch_bounds__(256) void naive_rowwise_kernel(
 
 __global__ __launch_bounds__(256) void naive_grouped_kernel(
     void* c, const uint8_t* a, const uint8_t* b, const float* a_scales, const float* b_scales,
-    const uint32_t* offsets, const int32_t* expert_ids, int64_t N, int64_t K, int64_t a_scales_ld,
+    const uint32_t* offsets, const int32_t* expert_ids, int64_t T, int64_t N, int64_t K, int64_t a_scales_ld,
     int c_dtype) {
   const int z = blockIdx.z;
-  const int64_t r0 = offsets[z], r1 = offsets[z + 1];
+  // (held inside the T rows the buffers have, whatever the routing tensor says)
+  const int64_t o0 = offsets[z], o1 = offsets[z + 1];
+  const int64_t r0 = o0 < T ? o0 : T, r1 = o1 < T ? o1 : T;
   const int64_t n = (int64_t)blockIdx.x * 16 + (threadIdx.x & 15);
   const int64_t ml = (int64_t)blockIdx.y * 16 + (threadIdx.x >> 4);
   if (n >= N || ml >= r1 - r0) return;
@@ -118,7 +121,7 @@ int naive_rowwise_dispatch(void* c, const void* a, const void* b, const void* a_
 }
 
 int naive_grouped_dispatch(void* c, const void* a, const void* b, const void* a_scales, const void* b_scales,
-                           const uint32_t* offsets, const int32_t* expert_ids, int64_t N, int64_t K,
+                           const uint32_t* offsets, const int32_t* expert_ids, int64_t T, int64_t N, int64_t K,
                            int64_t max_tokens, int64_t num_active, int64_t a_scales_ld, int c_dtype,
                            hipStream_t stream) {
   const int64_t gy = ceil_div(max_tokens, 16);
@@ -127,7 +130,7 @@ int naive_grouped_dispatch(void* c, const void* a, const void* b, const void* a_
                 (long long)max_tokens, (long long)num_active);
   hipLaunchKernelGGL(naive_grouped_kernel, dim3((unsigned)ceil_div(N, 16), (unsigned)gy, (unsigned)num_active),
                      dim3(256), 0, stream, c, (const uint8_t*)a, (const uint8_t*)b, (const float*)a_scales,
-                     (const float*)b_scales, offsets, expert_ids, N, K, a_scales_ld, c_dtype);
+                     (const float*)b_scales, offsets, expert_ids, T, N, K, a_scales_ld, c_dtype);
   return launch_status("naive_grouped");
 }
 

@@ -1,0 +1,35 @@
+// Tuning switches of the kernel selection, read from the environment ONCE per process (at the first
+// matmul) and kept as an immutable snapshot: no launch path calls getenv.  Tuning runs and tests that
+// flip a switch between calls re-read the environment through maxfp8_tuning_reload().
+//
+//   MAXFP8_TILE=1..4           force a tile shape of the tiled matmul (grouped: 2 = 256-row tiles in one
+//                              launch, 3 = no small tiles, 4 = no large-tile launch)
+//   MAXFP8_SPLITK=n            force the K split of the tiled matmul
+//   MAXFP8_ONE_REGION=1        never cut a matmul into two regions
+//   MAXFP8_PERSIST=0           per-tile kernels instead of the persistent one
+//   MAXFP8_STREAMK=0           no (tile, slab range) work units for matmuls of few tiles
+//   MAXFP8_BIG_ROWS=n          grouped: slots with at least n rows use the large-tile launch (1024)
+//   MAXFP8_GROUPED_OVERLAP=0   grouped: the two launches in line on the caller's stream
+//   MAXFP8_GROUPED_SHARE=x     grouped: scales the share estimate of the large-tile launch (0.5)
+//   MAXFP8_SKINNY=<ntw>4<KB>   force a shape of the weight-streaming kernel (e.g. 1408, 2416)
+#pragma once
+
+namespace maxfp8 {
+
+struct Tuning {
+  int tile = 0;
+  int splitk = 0;
+  bool one_region = false;
+  bool persist = true;
+  bool streamk = true;
+  int big_rows = 1024;
+  bool grouped_overlap = true;
+  float grouped_share = 0.5f;
+  int skinny = 0;
+  unsigned generation = 0;  // counts the reloads: part of the key of every cache that depends on the switches
+};
+
+const Tuning& tuning();
+void tuning_reload();
+
+}  // namespace maxfp8

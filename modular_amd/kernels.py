@@ -329,8 +329,8 @@ def dynamic_scaled_matmul(
             f"{a_scales.dtype}, {b_scales.dtype}")
     if a.dtype != _FP8:
         raise TypeError(f"a and b must be float8_e4m3fn, got {a.dtype}")
-    if a_scales.dtype not in (torch.float32, torch.bfloat16):
-        raise TypeError(f"scales dtype {a_scales.dtype} is not float32 or bfloat16")
+    if a_scales.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise TypeError(f"scales dtype {a_scales.dtype} is not float32, bfloat16 or float16")
     if out_type not in (torch.bfloat16, torch.float32):
         raise TypeError(f"out_type {out_type} is not bfloat16 or float32")
     if gin == _lib.GRAN_COLWISE and a_scales.shape[1] < a.shape[0]:

@@ -39,16 +39,30 @@ class Linear(torch.nn.Module):
         self.register_buffer("weight", torch.zeros((out_dim, in_dim), dtype=torch.uint8, device=device)
                              .view(torch.float8_e4m3fn))
         shape = infer_weight_scale_shape(out_dim, in_dim, quant_config)
-        self.register_buffer("weight_scale", torch.ones(shape, dtype=quant_config.weight_scale.dtype, device=device))
-        # static quantisation: the pre-computed input scale is a scalar kept on the CPU (linear.py:176-184)
-        self.input_scale = None
-        if quant_config.input_scale.origin == ScaleOrigin.STATIC:
-            self.input_scale = torch.ones((), dtype=quant_config.input_scale.dtype)
+        # Scalars that the static per-tensor ops take from the HOST stay on the CPU wherever the module goes: the
+        # pre-computed input scale and, with it, a per-tensor weight scale (the reference keeps its scale weights
+        # on the CPU, linear.py:176-205).  Both are entries of the state dict, so a checkpoint's `input_scale` /
+        # `weight_scale` load like any other tensor.  Per-row and block scales live beside the weight on the GPU.
+        static = quant_config.input_scale.origin == ScaleOrigin.STATIC
+        self._host_scalars = (("input_scale",) if static else ()) + (("weight_scale",) if static and shape == () else ())
+        scale_dev = "cpu" if "weight_scale" in self._host_scalars else device
+        self.register_buffer("weight_scale", torch.ones(shape, dtype=quant_config.weight_scale.dtype, device=scale_dev))
+        if static:
+            self.register_buffer("input_scale", torch.ones((), dtype=quant_config.input_scale.dtype, device="cpu"))
+        else:
+            self.input_scale = None
         if has_bias:
             self.register_buffer("bias", torch.zeros((out_dim,), dtype=quant_config.bias_dtype or bias_dtype,
                                                      device=device))
         else:
             self.bias = None
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to(device), .cuda(), .half() ... leave the host scalars where and what they are
+        keep = {name: self._buffers[name] for name in self._host_scalars}
+        out = super()._apply(fn, *args, **kwargs)
+        self._buffers.update(keep)
+        return out
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         lead = x.shape[:-1]
@@ -66,11 +80,18 @@ class MLP(torch.nn.Module):
     Like the reference, the gate and up projections run as ONE matmul over their concatenated
     weights when the quantisation allows it (`QuantConfig.can_use_fused_mlp`, linear.py:1029-1035);
     here the two weights ARE one buffer (`gate_up_weight`, with `gate_proj.weight` / `up_proj.weight`
-    views of its halves), so nothing is concatenated per call.  For dynamic block scaling with SiLU the
-    activation, the product with `up` and the quantisation of the result for `down_proj` are one
-    kernel (`fused_silu_quantized`): four launches for the whole block, no bf16 intermediate between
-    the activation and the second matmul.  Every other case (bias, another activation, a clamp,
-    static or per-tensor scales) takes the reference's unfused route through the three `Linear`s.
+    views of its halves), so nothing is concatenated per call.  With SiLU and no bias the activation
+    and the product with `up` are one kernel (`fused_silu`) whose bf16 result `down_proj` quantises
+    like any other input: the reference's arithmetic, five launches for the whole block.
+
+    `fuse_activation_quant=True` (dynamic block scaling only) also folds the quantisation for
+    `down_proj` into that kernel (`fused_silu_quantized`: four launches, no bf16 intermediate).
+    That kernel is the expert-parallel MoE quantiser (ep_comm.mojo:4505-4624), whose recipe is not
+    the one `down_proj` applies -- scale = max(amax, 1e-4) / 448 without the upper bound of 1200,
+    a division instead of a multiplication by the reciprocal, the f32 product instead of its bf16
+    rounding -- so the fp8 codes it hands to the second matmul can differ by a step from the
+    reference's: opt in where that is acceptable.  Every other case (bias, another activation, a
+    clamp, static or per-tensor scales) takes the unfused route through the three `Linear`s.
     """
 
     _ACTIVATIONS = {
@@ -83,7 +104,8 @@ class MLP(torch.nn.Module):
     }
 
     def __init__(self, hidden_dim: int, feed_forward_length: int, quant_config: QuantConfig, device=None,
-                 has_bias: bool = False, activation_function: str = "silu", swiglu_limit: float = 0.0) -> None:
+                 has_bias: bool = False, activation_function: str = "silu", swiglu_limit: float = 0.0,
+                 fuse_activation_quant: bool = False) -> None:
         super().__init__()
         if activation_function not in self._ACTIVATIONS:
             raise ValueError(f"Unsupported activation function: {activation_function}. "
@@ -92,6 +114,8 @@ class MLP(torch.nn.Module):
         self.quant_config = quant_config
         self.activation_function = activation_function
         self.swiglu_limit = swiglu_limit
+        self.fuse_activation_quant = fuse_activation_quant
+        self._row_offsets: dict[tuple, torch.Tensor] = {}  # [0, rows] per (rows, device): built once, on the device
         self.gate_proj = Linear(hidden_dim, feed_forward_length, quant_config, device=device, has_bias=has_bias)
         self.up_proj = Linear(hidden_dim, feed_forward_length, quant_config, device=device, has_bias=has_bias)
         self.down_proj = Linear(feed_forward_length, hidden_dim, quant_config, device=device, has_bias=has_bias)
@@ -123,16 +147,32 @@ class MLP(torch.nn.Module):
             self._tie_halves()
         return out
 
+    def _silu_kernel(self) -> bool:
+        """silu(gate) * up as one kernel on the stacked [rows, 2 * F] result of the one matmul"""
+        return (self._one_matmul and self.activation_function == "silu" and self.swiglu_limit == 0
+                and self.gate_proj.bias is None and self.feed_forward_length % 8 == 0)
+
     def _fused(self) -> bool:
         cfg = self.quant_config
-        return (self._one_matmul and cfg.input_scale.is_block and cfg.weight_scale.is_block
-                and cfg.input_scale.block_size == (1, 128) and self.activation_function == "silu"
-                and self.swiglu_limit == 0 and self.gate_proj.bias is None and self.down_proj.bias is None
+        return (self.fuse_activation_quant and self._silu_kernel() and cfg.input_scale.is_block and cfg.weight_scale.is_block
+                and cfg.input_scale.block_size == (1, 128) and self.down_proj.bias is None
                 and self.feed_forward_length % 128 == 0)
+
+    def _all_rows(self, rows: int, device: torch.device) -> torch.Tensor:
+        """The row_offsets operand of the silu kernels for a dense block: [0, rows] (uint32, on the device).  Kept
+        per row count, so that a call neither copies from the host nor breaks a HIP graph capture."""
+        key = (rows, device)
+        t = self._row_offsets.get(key)
+        if t is None:
+            if len(self._row_offsets) >= 64:
+                self._row_offsets.clear()
+            t = torch.tensor([0, rows], dtype=torch.int64).to(torch.uint32).to(device)
+            self._row_offsets[key] = t
+        return t
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         from .kernels import dynamic_scaled_matmul, quantize_dynamic_scaled_float8
-        from .moe_kernels import fused_silu_quantized
+        from .moe_kernels import fused_silu, fused_silu_quantized
 
         cfg = self.quant_config
         lead = x.shape[:-1]
@@ -142,11 +182,14 @@ class MLP(torch.nn.Module):
             xq, xs = quantize_dynamic_scaled_float8(x2, cfg.input_scale, cfg.weight_scale, scales_type=torch.float32)
             gate_up = dynamic_scaled_matmul(xq, self.gate_up_weight, xs, self.gate_up_weight_scale, cfg.input_scale,
                                             cfg.weight_scale, out_type=torch.bfloat16)
-            all_rows = torch.tensor([0, rows], dtype=torch.int64).to(torch.uint32).to(x2.device)
-            hq, hs = fused_silu_quantized(gate_up, all_rows, cfg)
+            hq, hs = fused_silu_quantized(gate_up, self._all_rows(rows, x2.device), cfg)
             y = dynamic_scaled_matmul(hq, self.down_proj.weight, hs, self.down_proj.weight_scale, cfg.input_scale,
                                       cfg.weight_scale, out_type=torch.bfloat16)
             return y.reshape(*lead, self.hidden_dim)
+        if self._silu_kernel():
+            both = quantized_matmul(x2, self.gate_up_weight, self.gate_up_weight_scale, None, cfg)
+            hidden = fused_silu(both, self._all_rows(x2.shape[0], x2.device))
+            return self.down_proj(hidden).reshape(*lead, self.hidden_dim)
         act = self._ACTIVATIONS[self.activation_function]
         if self._one_matmul and self.gate_proj.bias is None:
             both = quantized_matmul(x2, self.gate_up_weight, self.gate_up_weight_scale, None, cfg)

@@ -1,13 +1,16 @@
 """FP8 dispatch of a quantised linear, mirroring `quantized_matmul` /
 `_matmul_float8` (max/python/max/nn/quant_ops.py:516-592, 336-481): the static
-per-tensor branch and the dynamic tensor / per-row / block branches.
+per-tensor branch and the dynamic tensor / per-row / block branches; and of the
+quantised grouped matmul of the MoE layers, `quantized_grouped_matmul`
+(quant_ops.py:880-1007, FP8 formats).
 """
 from __future__ import annotations
 
 import torch
 
-from .kernels import (dynamic_scaled_matmul, fused_qkv_ragged_matmul_scaled_float8, matmul_static_scaled_float8,
-                      quantize_dynamic_scaled_float8, quantize_static_scaled_float8,
+from .kernels import (dynamic_scaled_matmul, fused_qkv_ragged_matmul_scaled_float8,
+                      grouped_dynamic_scaled_fp8_matmul, grouped_matmul_rowwise_dynamic_scaled_fp8,
+                      matmul_static_scaled_float8, quantize_dynamic_scaled_float8, quantize_static_scaled_float8,
                       quantize_tensor_dynamic_scaled_float8)
 from .kv_cache import KVCacheParams, PagedCacheValues
 from .quant_config import InputScaleSpec, QuantConfig, QuantFormat, ScaleGranularity, WeightScaleSpec
@@ -112,3 +115,67 @@ def quantized_fused_qkv_matmul(
     return fused_qkv_ragged_matmul_scaled_float8(kv_params, input=xq, input_scale=x_scales.to(x.device).float(),
                                                  weight_scale=weight_scale.to(x.device).float(), quant_config=quant_config,
                                                  **common)
+
+
+# ---- grouped (MoE) entry point ---------------------------------------------------------------
+# The reference keeps stacked FP8 expert weights in storage layout [E, in, out] = [E, K, N] and
+# transposes them to [E, N, K] in the graph (quant_ops.py:941-944), where the transposition of a
+# constant weight is folded away at compile time.  The eager equivalent: a storage tensor is
+# transposed once and the K-innermost copy is kept for as long as the storage tensor stays as it is
+# (same memory, same shape, no in-place write since).
+_K_INNERMOST: dict[tuple, tuple[torch.Tensor, torch.Tensor]] = {}
+_K_INNERMOST_MAX = 16
+
+
+def _k_innermost(t: torch.Tensor) -> torch.Tensor:
+    """t.transpose(1, 2) as a contiguous tensor, made once per storage tensor."""
+    key = (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t.dtype, t.device, t._version)
+    hit = _K_INNERMOST.get(key)
+    if hit is not None and hit[0] is t:
+        return hit[1]
+    # (fp8 has no copy kernel of its own in every torch build: move the bytes)
+    tt = t.view(torch.uint8).transpose(1, 2).contiguous().view(t.dtype) if t.element_size() == 1 else t.transpose(1, 2).contiguous()
+    if len(_K_INNERMOST) >= _K_INNERMOST_MAX:
+        _K_INNERMOST.pop(next(iter(_K_INNERMOST)))
+    _K_INNERMOST[key] = (t, tt)
+    return tt
+
+
+def quantized_grouped_matmul(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    weight_scale: torch.Tensor,
+    expert_start_indices: torch.Tensor,
+    expert_ids: torch.Tensor,
+    usage_stats: torch.Tensor,
+    quant_config: QuantConfig,
+) -> torch.Tensor:
+    """Single entry point of the quantised grouped matmuls of a MoE layer (quant_ops.py:880-1007),
+    FP8 formats: x [T, K] bf16 with its rows sorted by expert; weight in STORAGE layout [E, K, N]
+    e4m3fn; weight_scale in storage layout -- [E, K/128, N/128] for block scaling, [E, N, 1] for
+    per-channel scaling; usage_stats = [most rows on one expert, active experts] (device or CPU: the
+    op takes them as host scalars, so a device tensor is copied, which waits for the GPU).
+
+    Block scaling: both are transposed to the K-innermost orientation of the kernel, x is quantised
+    in 1 x block groups with scales of the weight scales' dtype, then the grouped block-scaled matmul.
+    Per-channel weight scales with per-token activation scales (no block size): the weight scales
+    are used as they are, the [1, T] scales of the quantiser become the kernel's [T, 1]."""
+    if quant_config.format not in (QuantFormat.COMPRESSED_TENSORS_FP8, QuantFormat.FBGEMM_FP8, QuantFormat.BLOCKSCALED_FP8):
+        raise ValueError(f"Unsupported quantization format for grouped matmul: {quant_config.format}")
+    if weight.dim() != 3:
+        raise ValueError(f"expected weight of rank 3 but got {weight.dim()}")
+    weight_t = _k_innermost(weight)
+    stats_host = usage_stats.cpu()
+    if quant_config.weight_scale.is_rowwise and quant_config.input_scale.block_size is None:
+        x_fp8, x_scales = quantize_dynamic_scaled_float8(x, quant_config.input_scale, quant_config.weight_scale,
+                                                         out_type=weight.dtype, scales_type=torch.float32)
+        return grouped_matmul_rowwise_dynamic_scaled_fp8(x_fp8, weight_t, x_scales.transpose(0, 1), weight_scale,
+                                                         expert_start_indices, expert_ids, stats_host)
+    assert quant_config.input_scale.block_size is not None
+    input_block_size = quant_config.input_scale.block_size[1]
+    scale_t = _k_innermost(weight_scale)
+    x_fp8, x_scales = quantize_dynamic_scaled_float8(x, quant_config.input_scale, quant_config.weight_scale,
+                                                     group_size_or_per_token=input_block_size, out_type=weight.dtype,
+                                                     scales_type=quant_config.weight_scale.dtype)
+    return grouped_dynamic_scaled_fp8_matmul(x_fp8, weight_t, x_scales, scale_t, expert_start_indices, expert_ids,
+                                             stats_host, quant_config.input_scale, quant_config.weight_scale)

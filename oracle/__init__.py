@@ -308,18 +308,20 @@ def matmul_blockwise(a: np.ndarray, b: np.ndarray, a_scales: np.ndarray, b_scale
 
 def matmul_rowwise(a: np.ndarray, b: np.ndarray, a_scales: np.ndarray, b_scales: np.ndarray,
                    *, c_dtype: int = F32, tensor_scales: bool = False,
-                   threads: int = 1) -> np.ndarray:
-    """a_scales [1, M] (or [1,1]), b_scales [N, 1] (or [1,1]); f32."""
+                   threads: int = 1, scales_dtype: int = F32) -> np.ndarray:
+    """a_scales [1, M] (or [1,1]), b_scales [N, 1] (or [1,1]): float32 arrays, or with
+    scales_dtype BF16 / F16 uint16 bit patterns / float16 values that the oracle widens."""
     a = np.ascontiguousarray(a, dtype=np.uint8)
     b = np.ascontiguousarray(b, dtype=np.uint8)
-    a_scales = np.ascontiguousarray(a_scales, dtype=np.float32)
-    b_scales = np.ascontiguousarray(b_scales, dtype=np.float32)
+    sdt = {F32: np.float32, BF16: np.uint16, F16: np.float16}[scales_dtype]
+    a_scales = np.ascontiguousarray(a_scales, dtype=sdt)
+    b_scales = np.ascontiguousarray(b_scales, dtype=sdt)
     M, K = a.shape
     N = b.shape[0]
     c = np.zeros((M, N), dtype=np.float32 if c_dtype == F32 else np.uint16)
     st = 0 if tensor_scales else 1
     rc = lib().orc_matmul_rowwise(_p(c), _p(a), _p(b), _p(a_scales), _p(b_scales),
-                                  M, N, K, K, K, N, st, st, c_dtype, F32, threads)
+                                  M, N, K, K, K, N, st, st, c_dtype, scales_dtype, threads)
     if rc:
         raise ValueError(f"oracle rowwise matmul failed: {rc}")
     return c

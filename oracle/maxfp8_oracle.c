@@ -369,9 +369,12 @@ static inline void store_c(void* c, int c_dtype, int64_t idx, float v) {
   else ((float*)c)[idx] = v;
 }
 
+/* A scale of dtype f32, bf16 or f16, widened to f32 as the reference's epilogue does
+ * (fp8_quantization.mojo:1218-1240: load, cast to the accumulator's dtype, multiply). */
 static inline float load_scale(const void* s, int dtype, int64_t idx) {
-  return dtype == ORC_BF16 ? bf16_to_f32(((const uint16_t*)s)[idx])
-                           : ((const float*)s)[idx];
+  if (dtype == ORC_BF16) return bf16_to_f32(((const uint16_t*)s)[idx]);
+  if (dtype == ORC_F16) return f16_to_f32(((const uint16_t*)s)[idx]);
+  return ((const float*)s)[idx];
 }
 
 /*

@@ -9,7 +9,7 @@ import torch
 import modular_amd as mx
 import oracle
 from modular_amd import synth
-from util import F32_BUDGET, assert_rel, f32_np, fp8_bytes, fp8_from_bytes, u32_np
+from util import F32_BUDGET, assert_rel, bf16_bits, f32_np, fp8_bytes, fp8_from_bytes, u32_np
 
 pytestmark = pytest.mark.gpu
 BLK = mx.blockwise_fp8_config()
@@ -113,33 +113,44 @@ def test_grouped_zero_edges_and_untouched_rows(dev):
         assert np.array_equal(two[:10], full[:10]) and np.all(np.isnan(two[10:]))
 
 
-def test_moe_config_sampled(dev):
-    # 256 experts, top-8 of 4096 tokens with Zipf(1.1) popularity; down projection K=2048, N=7168.
-    E, Kd, Nd = 256, 2048, 7168
+@pytest.mark.parametrize("proj,Kd,Nd", [("gate_up", 7168, 4096), ("down", 2048, 7168)])
+def test_moe_config_sampled(dev, proj, Kd, Nd):
+    # 256 experts, top-8 of 4096 tokens with Zipf(1.1) popularity; both expert matmuls of the DeepSeek-V3 layer
+    # (gate_up: hidden 7168 -> 2 * 2048; down: 2048 -> 7168) at full size, 32768 routed rows.
+    E = 256
     off, ids, counts, stats = synth.moe_routing(4096, E, 8, seed=0, device=dev)
     T = int(counts.sum())
     assert T == 32768
-    x = synth.activations(T, Kd, seed=0, outlier_frac=0.0, device=dev)
+    x = synth.activations(T, Kd, seed=0, outlier_frac=0.01 if proj == "gate_up" else 0.0, device=dev)
     q, sa = mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32)
+    del x
     w = torch.empty((E, Nd, Kd), dtype=torch.float8_e4m3fn, device=dev)
     sb = torch.empty((E, Nd // 128, Kd // 128), dtype=torch.float32, device=dev)
-    for e0 in range(0, E, 32):
-        wq, ws = synth.quantize_weight_block(synth.weights_f32(32 * Nd, Kd, seed=100 + e0, device=dev).reshape(32, Nd, Kd))
-        w[e0:e0 + 32], sb[e0:e0 + 32] = wq, ws
+    for e0 in range(0, E, 16):
+        wq, ws = synth.quantize_weight_block(synth.weights_f32(16 * Nd, Kd, seed=100 + e0, device=dev).reshape(16, Nd, Kd))
+        w[e0:e0 + 16], sb[e0:e0 + 16] = wq, ws
     c = mx.grouped_dynamic_scaled_fp8_matmul(q, w, sa, sb, off, ids, stats, BLK.input_scale, BLK.weight_scale)
     torch.cuda.synchronize()
     assert bool(torch.isfinite(c.float()).all())
     offs = u32_np(off).astype(np.int64)
     order = np.argsort(-counts.numpy())
-    for e in list(order[:2]) + list(order[-3:]) + [17, 128]:   # biggest, smallest and two arbitrary experts
+    # the two biggest experts, the three smallest, two of medium size (a few 128-row tiles) and two arbitrary ones
+    mid = [int(e) for e in order if 129 <= counts[e] <= 1023][:2]
+    for e in list(order[:2]) + list(order[-3:]) + mid + [17, 128]:
         r0, r1 = offs[e], offs[e + 1]
         if r1 == r0:
             continue
-        rows = torch.arange(r0, r1, max(1, (r1 - r0) // 8), device=dev)[:8]
+        # rows spread over the slot, its last row included (the slot's ragged last tile)
+        rows = torch.unique(torch.cat([torch.arange(r0, r1, max(1, (r1 - r0) // 8), device=dev)[:8], torch.tensor([r1 - 1], device=dev)]))
         refc = mx.dynamic_scaled_matmul(q[rows].contiguous(), w[e], sa[:, rows].contiguous(), sb[e], BLK.input_scale,
                                         BLK.weight_scale, out_type=torch.float32, algo="naive")
         torch.cuda.synchronize()
-        assert_rel(f32_np(c[rows]), f32_np(refc), TOL, f"expert {e} rows {r0}:{r1}")
+        assert_rel(f32_np(c[rows]), f32_np(refc), TOL, f"{proj}: expert {e} rows {r0}:{r1}", natural_scale=True)
+    # one row of the biggest expert against the CPU oracle itself
+    e = int(order[0])
+    r = int(offs[e])
+    cpu = oracle.matmul_blockwise(fp8_bytes(q[r:r + 1]), fp8_bytes(w[e]), f32_np(sa[:, r:r + 1]), f32_np(sb[e]), threads=NT)
+    assert_rel(f32_np(c[r:r + 1]), cpu, TOL, f"{proj}: row {r} against the CPU oracle", natural_scale=True)
 
 
 def test_random_groupings_are_exact(dev):
@@ -175,3 +186,99 @@ def test_random_groupings_are_exact(dev):
         got = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=out)
         want = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=out, algo="naive")
         assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, N {N}, K {K}, {out}"
+
+
+# ---- the layer above the op: quantized_grouped_matmul and Fp8Strategy -----------------------------------
+
+def test_quantized_grouped_matmul_from_the_storage_layout(dev):
+    """quant_ops.py:880-1007: bf16 rows sorted by expert, weights and block scales in STORAGE layout [E, K, N] /
+    [E, K/128, N/128].  The entry point transposes both to the kernel's orientation, quantises x in 1 x 128 groups and
+    runs the grouped matmul: against the oracle's quantiser + grouped matmul on the K-innermost operands."""
+    from modular_amd import quant_ops
+    counts, ids, E, N, K = [20, 1500, 300, 28], [0, 3, 2, 4], 5, 256, 512
+    T = sum(counts)
+    x = synth.activations(T, K, seed=3)
+    w_nk, s_nk = synth.quantize_weight_block(synth.weights_f32(E * N, K, seed=4).reshape(E, N, K))   # kernel orientation
+    w_store = w_nk.view(torch.uint8).transpose(1, 2).contiguous().view(torch.float8_e4m3fn)            # [E, K, N]
+    s_store = s_nk.transpose(1, 2).contiguous()                                                         # [E, K/128, N/128]
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32)
+    ids_t = torch.tensor(ids + [-1] * (E - len(ids)), dtype=torch.int32)
+    stats = torch.tensor([max(counts), len(counts)], dtype=torch.int64).to(torch.uint32)
+    wd, sd = w_store.to(dev), s_store.to(dev)
+    y = quant_ops.quantized_grouped_matmul(x.to(dev), wd, sd, off.to(dev), ids_t.to(dev), stats.to(dev), BLK)
+    torch.cuda.synchronize()
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (T, N)
+    q, sa = oracle.quantize_dynamic_scaled_fp8(bf16_bits(x), 128, threads=NT)
+    want = oracle.grouped_matmul(q, fp8_bytes(w_nk), sa, s_nk.numpy(), u32_np(off), ids_t.numpy(), max(counts), len(counts), threads=NT)
+    assert_rel(f32_np(y), want, TOL, "quantized_grouped_matmul", natural_scale=True)
+    # the K-innermost copy is made once per storage tensor, and again after an in-place write
+    n_cached = len(quant_ops._K_INNERMOST)
+    y2 = quant_ops.quantized_grouped_matmul(x.to(dev), wd, sd, off.to(dev), ids_t.to(dev), stats, BLK)
+    assert len(quant_ops._K_INNERMOST) == n_cached and torch.equal(y, y2)
+    wd.view(torch.uint8)[3].zero_()   # expert 3 serves slot 1
+    y3 = quant_ops.quantized_grouped_matmul(x.to(dev), wd, sd, off.to(dev), ids_t.to(dev), stats, BLK)
+    assert len(quant_ops._K_INNERMOST) == n_cached + 1
+    lo = counts[0] + counts[1]
+    assert torch.equal(y3[:counts[0]], y[:counts[0]]) and torch.equal(y3[lo:], y[lo:]) and not y3[counts[0]:lo].float().any()
+
+
+def test_quantized_grouped_matmul_per_channel_layout(dev):
+    """The compressed-tensors FP8-dynamic layout (quant_ops.py:945-981): per-channel weight scales [E, N, 1] used as
+    they are, per-token activation scales [1, T] handed to the kernel as [T, 1]."""
+    from modular_amd import quant_ops
+    ROWCFG = mx.rowwise_fp8_config()
+    counts, ids, E, N, K = [40, 0, 130, 1], [2, 1, 3, 0], 4, 384, 512
+    T = sum(counts)
+    x = synth.activations(T, K, seed=5, outlier_frac=0.0)
+    w_nk, s_nk = synth.quantize_weight_rowwise(synth.weights_f32(E * N, K, seed=6))
+    w_nk, s_nk = w_nk.reshape(E, N, K), s_nk.reshape(E, N, 1)
+    w_store = w_nk.view(torch.uint8).transpose(1, 2).contiguous().view(torch.float8_e4m3fn)
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32)
+    ids_t = torch.tensor(ids, dtype=torch.int32)
+    stats = torch.tensor([max(counts), len(counts)], dtype=torch.int64).to(torch.uint32)
+    y = quant_ops.quantized_grouped_matmul(x.to(dev), w_store.to(dev), s_nk.to(dev), off.to(dev), ids_t.to(dev), stats, ROWCFG)
+    torch.cuda.synchronize()
+    q, sa = oracle.quantize_dynamic_scaled_fp8(bf16_bits(x), K, threads=NT)          # [1, T]
+    want = oracle.grouped_matmul_rowwise(q, fp8_bytes(w_nk), sa.reshape(T, 1), s_nk.numpy(), u32_np(off), ids_t.numpy(), len(counts), threads=NT)
+    assert_rel(f32_np(y), want, TOL, "quantized_grouped_matmul, per-channel", natural_scale=True)
+
+
+def test_fp8_strategy_methods(dev):
+    """moe/quant_strategy.py:114-215: quantize / grouped_quantize / grouped_matmul / prepare_weight_scales /
+    fused_silu_quantize do what the ops they forward to do."""
+    counts, ids, E, N, K = [7, 0, 129, 0, 128], [2, 1, 0, 3, 4], 5, 256, 384
+    T = sum(counts)
+    st = mx.Fp8Strategy(BLK, torch.float8_e4m3fn)
+    x = synth.activations(T, K, seed=7).to(dev)
+    xq, xs = st.quantize(x, 128)
+    q0, s0 = mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32, group_size_or_per_token=128)
+    assert torch.equal(xq.view(torch.uint8), q0.view(torch.uint8)) and torch.equal(xs[:, :T], s0[:, :T]) and xs.dtype == torch.float32
+    g2 = st.grouped_quantize(x, 128, None, None, None, None)
+    assert torch.equal(g2[0].view(torch.uint8), xq.view(torch.uint8))
+    w, sw = synth.quantize_weight_block(synth.weights_f32(E * N, K, seed=8).reshape(E, N, K))
+    a, b = st.prepare_weight_scales(sw, sw, dev)
+    assert a is sw and b is sw
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32).to(dev)
+    ids_t = torch.tensor(ids, dtype=torch.int32, device=dev)
+    stats = torch.tensor([max(counts), len(counts)], dtype=torch.int64).to(torch.uint32).to(dev)   # on the device: copied to the host inside
+    inputs = (xq, xs, off, ids_t, stats)
+    y = st.grouped_matmul(w.to(dev), sw.to(dev), expert_inputs=inputs)
+    want = mx.grouped_dynamic_scaled_fp8_matmul(xq, w.to(dev), xs, sw.to(dev), off, ids_t, stats.cpu(), BLK.input_scale, BLK.weight_scale)
+    assert torch.equal(y, want)
+    hq, hs = st.fused_silu_quantize(y, expert_inputs=inputs)
+    wq_, ws_ = mx.fused_silu_quantized(y, off, BLK)
+    assert torch.equal(hq.view(torch.uint8), wq_.view(torch.uint8)) and torch.equal(hs, ws_)
+    with pytest.raises(AssertionError):
+        st.fused_silu_quantize(y, expert_inputs=inputs, clamp_activation=True)
+
+
+@pytest.mark.parametrize("algo", ["auto", "naive"])
+def test_offsets_beyond_the_rows_are_held_to_the_buffers(dev, algo):
+    """expert_start_indices is read on the device.  Entries beyond T (a stale or damaged routing tensor) are held
+    to T: the slot ends with the buffers, no row outside them is read or written."""
+    counts, ids, E, N, K = [10, 30], [1, 0], 2, 256, 256
+    a, b, sa, sb, off, ids_t = make(counts, ids, E, N, K, seed=9)
+    good = run(a, b, sa, sb, off, ids_t, 40, 2, dev, algo=algo)
+    wild = torch.tensor([0, 10, 1 << 30], dtype=torch.int64).to(torch.uint32)
+    got = run(a, b, sa, sb, wild, ids_t, 40, 2, dev, algo=algo)
+    assert torch.equal(good, got)

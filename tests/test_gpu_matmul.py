@@ -115,10 +115,10 @@ def test_mfma_rowwise_exact(dev, algo, M):
 
 @pytest.mark.parametrize("sel", ["1408", "1416", "2408", "2416", "4432"])
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (8, 200, 1040), (16, 272, 640), (33, 100, 512), (64, 336, 1152)])
-def test_every_decode_shape_is_exact(dev, monkeypatch, sel, M, N, K):
+def test_every_decode_shape_is_exact(dev, tune, sel, M, N, K):
     """The decode kernel's shapes (weight rows per block, bytes in flight per wave) forced one by one, on ragged N and
     K: exact on integer data in both scale modes, so the choice between them cannot change a result."""
-    monkeypatch.setenv("MAXFP8_SKINNY", sel)
+    tune(MAXFP8_SKINNY=sel)
     a, b, sa, sb, want = exact_case(M, N, K, seed=M + N + K)
     got = f32_np(mm(a, b, sa, sb, BLK, dev, algo="skinny")).astype(np.float64)
     assert np.array_equal(got, want), f"block mode, shape {sel}: {np.argwhere(got != want)[:4].tolist()}"
@@ -261,42 +261,102 @@ def test_empty(dev):
 
 
 # ---- configuration-sized problems, checked on sampled rows by the naive kernel ----------------
+# Every (K, N) of the benchmark configurations at the M values named there; rows are sampled because the
+# scalar-order kernel (bit-identical to the CPU oracle, tested above) needs a second per 24 rows at these sizes.
 
-@pytest.mark.parametrize("M,K,N", [
-    (2048, 4096, 6144),     # Llama-3.1-8B QKV
-    (128, 14336, 4096),     # Llama-3.1-8B down, M = 128
-    (1024, 7168, 1536),     # DeepSeek-V3 q_a
-    (256, 7168, 576),       # DeepSeek-V3 kv_a (N not a multiple of 128)
-    (4096, 512, 32768),     # DeepSeek-V3 kv_b
-    (16, 4096, 28672),      # Llama-3.1-8B gate_up, decode-like
-])
-def test_config_shapes_blockwise(dev, M, K, N):
+LLAMA8B = {"qkv": (4096, 6144), "gate_up": (4096, 28672), "down": (14336, 4096), "o_proj": (4096, 4096)}
+DSV3 = {"q_a": (7168, 1536), "q_b": (1536, 24576), "kv_a": (7168, 576), "kv_b": (512, 32768), "o_proj": (16384, 7168)}
+CONFIG_CELLS = ([("single_linear", 64, 4096, 4096)]
+                + [(f"llama8b_{n}", M, K, N) for n, (K, N) in LLAMA8B.items() for M in (1, 16, 128, 2048)]
+                + [(f"dsv3_{n}", M, K, N) for n, (K, N) in DSV3.items() for M in (256, 1024, 4096)])
+
+_operands = {}
+
+
+def config_operands(K, N, dev):
+    """weights of one (K, N) cell, quantised once and shared by the cell's M values"""
+    if (K, N) not in _operands:
+        _operands.clear()
+        _operands[(K, N)] = synth.quantize_weight_block(synth.weights_f32(N, K, seed=1, device=dev))
+    return _operands[(K, N)]
+
+
+@pytest.mark.parametrize("name,M,K,N", CONFIG_CELLS, ids=[f"{c[0]}_m{c[1]}" for c in CONFIG_CELLS])
+def test_config_shapes_blockwise(dev, name, M, K, N):
     x = synth.activations(M, K, seed=0, device=dev)
-    w, sb = synth.quantize_weight_block(synth.weights_f32(N, K, seed=1, device=dev))
+    w, sb = config_operands(K, N, dev)
     q, sa = mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32)
     c = mx.dynamic_scaled_matmul(q, w, sa, sb, BLK.input_scale, BLK.weight_scale)
-    rows = torch.arange(0, M, max(1, M // 24), device=dev)[:24]
+    # 24 rows spread over the matrix, the last one included (the last tile row, where partial tiles live)
+    rows = torch.unique(torch.cat([torch.arange(0, M, max(1, M // 23), device=dev)[:23], torch.tensor([M - 1], device=dev)]))
     ref = mx.dynamic_scaled_matmul(q[rows].contiguous(), w, sa[:, rows].contiguous(), sb, BLK.input_scale,
                                    BLK.weight_scale, out_type=torch.float32, algo="naive")
     torch.cuda.synchronize()
-    assert_rel(f32_np(c[rows]), f32_np(ref), TOL, f"config {M}x{N}x{K}")
+    fig = assert_rel(f32_np(c[rows]), f32_np(ref), TOL, f"config {name} {M}x{N}x{K}", natural_scale=True)
+    print(f"[parity] {name} M={M}: rel err {fig['rel_err']:.2e} (floor 2^-4 rms), {fig['rel_err_strict_floor']:.2e} "
+          f"(floor 2^-8 rms), |err| <= {fig['err_over_rms']:.2e} rms, reference-style excess {fig['reference_style_excess']:.2f}")
     # one row against the CPU oracle itself
     r0 = int(rows[-1])
     cpu = oracle.matmul_blockwise(fp8_bytes(q[r0:r0 + 1]), fp8_bytes(w), f32_np(sa[:, r0:r0 + 1]), f32_np(sb), threads=NT)
     assert np.array_equal(f32_np(ref[-1:]), cpu)
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 8192, 10240), (8, 8192, 10240), (4, 28672, 8192), (2, 8192, 57344)])
-def test_config_shapes_decode_rowwise(dev, M, K, N):
+DECODE70B = {"qkv": (8192, 10240), "gate_up": (8192, 57344), "down": (28672, 8192)}
+DECODE_CELLS = [(n, M, K, N) for n, (K, N) in DECODE70B.items() for M in (1, 2, 4, 8)]
+
+
+@pytest.mark.parametrize("name,M,K,N", DECODE_CELLS, ids=[f"{c[0]}_m{c[1]}" for c in DECODE_CELLS])
+def test_config_shapes_decode_rowwise(dev, name, M, K, N):
     x = synth.activations(M, K, seed=0, outlier_frac=0.0, device=dev)
-    w, sb = synth.quantize_weight_rowwise(synth.weights_f32(N, K, seed=1, device=dev))
+    if ("row", K, N) not in _operands:
+        _operands.clear()
+        _operands[("row", K, N)] = synth.quantize_weight_rowwise(synth.weights_f32(N, K, seed=1, device=dev))
+    w, sb = _operands[("row", K, N)]
     q, sa = mx.quantize_dynamic_scaled_float8(x, ROW.input_scale, ROW.weight_scale, scales_type=torch.float32)
     assert tuple(sa.shape) == (1, M)
     c = mx.dynamic_scaled_matmul(q, w, sa, sb, ROW.input_scale, ROW.weight_scale)
     cols = torch.arange(0, N, 37, device=dev)
     ref = oracle.matmul_rowwise(fp8_bytes(q), fp8_bytes(w[cols]), f32_np(sa), f32_np(sb[cols]), threads=NT)
     torch.cuda.synchronize()
-    assert_rel(f32_np(c[:, cols]), ref, TOL, f"decode {M}x{N}x{K}")
+    assert_rel(f32_np(c[:, cols]), ref, TOL, f"decode {name} {M}x{N}x{K}", natural_scale=True)
     # linearity in the activation scale: doubling a_s doubles C exactly (power of two)
     c2 = mx.dynamic_scaled_matmul(q, w, sa * 2, sb, ROW.input_scale, ROW.weight_scale)
     assert torch.equal(c2.float(), c.float() * 2)
+    _ = name
+
+
+# ---- per-token / per-channel scales in bf16 and f16 ----------------------------------------------
+
+@pytest.mark.parametrize("algo,M,N,K", [("tiled", 300, 1040, 1024), ("tiled", 2048, 512, 512), ("tiled", 1024, 1024, 256),
+                                        ("skinny", 8, 1000, 2048), ("skinny", 40, 512, 256), ("auto", 96, 2304, 16384)])
+@pytest.mark.parametrize("sdt", [torch.bfloat16, torch.float16])
+def test_rowwise_scales_in_bf16_and_f16(dev, algo, M, N, K, sdt):
+    """The reference's matmul takes its scales in bf16, f16 or f32 (fp8_quantization.mojo:996-1018; its Python
+    wrapper even defaults to bf16) and widens them when the epilogue loads them (:1218-1240).  Every kernel does
+    the same: the result equals the f32-scales result on the widened values bit for bit, whatever the kernel, and
+    meets the oracle reading the 16-bit scales itself."""
+    a, b = synth.random_fp8((M, K), M), synth.random_fp8((N, K), N)
+    sa = synth.random_scales((1, M), 3, lo=0.01, hi=0.1).to(sdt)
+    sb = synth.random_scales((N, 1), 4, lo=0.001, hi=0.01).to(sdt)
+    odt = oracle.BF16 if sdt == torch.bfloat16 else oracle.F16
+    bits = (lambda t: bf16_bits(t)) if sdt == torch.bfloat16 else (lambda t: t.numpy())
+    ref = oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), bits(sa), bits(sb), threads=NT, scales_dtype=odt)
+    assert np.array_equal(ref, oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), sa.float().numpy(), sb.float().numpy(), threads=NT))
+    from modular_amd import _lib
+    assert "naive" not in _lib.matmul_describe(M, N, K, False, True)
+    for out in (torch.float32, torch.bfloat16):
+        c = mm(a, b, sa, sb, ROW, dev, out=out, algo=algo)
+        assert_rel(f32_np(c), ref, TOL, f"{sdt} scales {algo} {M}x{N}x{K} {out}", F32_BUDGET if out == torch.float32 else None)
+        assert torch.equal(c, mm(a, b, sa.float(), sb.float(), ROW, dev, out=out, algo=algo))
+    # the scalar kernel reads them too (it is the oracle's twin)
+    assert np.array_equal(f32_np(mm(a, b, sa, sb, ROW, dev, algo="naive")), ref)
+
+
+def test_tensor_scales_in_bf16(dev):
+    cfg = QuantConfig(InputScaleSpec(ScaleGranularity.TENSOR, ScaleOrigin.DYNAMIC, torch.bfloat16),
+                      WeightScaleSpec(ScaleGranularity.TENSOR, torch.bfloat16))
+    a, b = synth.random_fp8((200, 512), 1), synth.random_fp8((272, 512), 2)
+    sa, sb = torch.tensor([[0.031]]).to(torch.bfloat16), torch.tensor([[0.0047]]).to(torch.bfloat16)
+    ref = oracle.matmul_rowwise(fp8_bytes(a), fp8_bytes(b), sa.float().numpy(), sb.float().numpy(), tensor_scales=True)
+    for algo in ("naive", "tiled"):
+        assert_rel(f32_np(mm(a, b, sa, sb, cfg, dev, algo=algo)), ref, TOL, algo, F32_BUDGET)

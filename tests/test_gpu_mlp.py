@@ -1,7 +1,8 @@
 """The FP8 gated MLP block (`MLP`, mirroring max/python/max/nn/linear.py:865-1095) on the GPU.
 
-Block-scaled with SiLU it is four of this package's kernels: quantise, one matmul over the stacked gate / up
-weights, silu(gate) * up fused with the quantisation for the second matmul, and the down matmul.  Each stage
+Block-scaled with SiLU it is this package's kernels only: quantise, one matmul over the stacked gate / up
+weights, silu(gate) * up (by default rounded to bf16 and quantised by `down_proj` like any input; with
+`fuse_activation_quant=True` fused with that quantisation), and the down matmul.  Each stage
 is checked against the CPU oracle ON THE GPU'S OWN INPUT of that stage (end to end, two correct runs differ
 by more than a matmul's tolerance: a bf16 flip in gate_up moves the second quantiser's scales), the block
 against float64 arithmetic on the dequantised weights, and the other routes (per-token scales, bias, clamp,
@@ -34,7 +35,7 @@ def make_block_mlp(hidden, ffl, dev, **kw):
 
 @pytest.mark.parametrize("M,hidden,ffl", [(64, 512, 1024), (300, 1024, 3584), (2048, 512, 2048), (1, 256, 512)])
 def test_block_scaled_mlp_stage_by_stage(dev, M, hidden, ffl):
-    mlp, parts = make_block_mlp(hidden, ffl, dev)
+    mlp, parts = make_block_mlp(hidden, ffl, dev, fuse_activation_quant=True)
     assert mlp._fused()
     # the projections' weights are the halves of one buffer: nothing is concatenated per call
     assert mlp.gate_proj.weight.data_ptr() == mlp.gate_up_weight.data_ptr()
@@ -76,6 +77,35 @@ def test_block_scaled_mlp_stage_by_stage(dev, M, hidden, ffl):
     full = (torch.nn.functional.silu(xd @ deq("gate_proj").t()) * (xd @ deq("up_proj").t())) @ deq("down_proj").t()
     err = (y.reshape(M, hidden).double().cpu() - full).norm() / full.norm()
     assert err < 0.06, f"relative error {err:.3f} against float64 on dequantised weights"
+
+
+@pytest.mark.parametrize("M,hidden,ffl", [(48, 512, 1024), (257, 1024, 3584)])
+def test_block_scaled_mlp_default_route_quantises_like_a_linear(dev, M, hidden, ffl):
+    """Without the opt-in the activations that reach the second matmul are what the reference's block hands it:
+    silu(gate) * up rounded to bf16, quantised by down_proj's own rule (upper bound 1200, multiplication by the
+    guarded reciprocal).  The fp8 bytes and scales are those of the oracle's quantiser on that bf16 tensor."""
+    mlp, parts = make_block_mlp(hidden, ffl, dev)
+    assert not mlp._fused() and mlp._silu_kernel()
+    x = synth.activations(M, hidden, seed=8).to(dev)
+    y = mlp(x)
+    both = mx.quantized_matmul(x, mlp.gate_up_weight, mlp.gate_up_weight_scale, None, BLK)
+    rows = torch.tensor([0, M], dtype=torch.int64).to(torch.uint32).to(dev)
+    hidden_act = mx.fused_silu(both, rows)
+    assert torch.equal(y, mlp.down_proj(hidden_act)), "the block is its stages"
+    # the stage in front of the second quantiser against the oracle: equal but for the last bit of exp
+    want_h = oracle.fused_silu(bf16_bits(both), M, quantize=False, threads=NT)
+    assert (bf16_bits(hidden_act) != want_h).mean() <= 5e-3
+    # what down_proj quantises: bit-exact with the oracle's quantize_dynamic_scaled_fp8 on the same bf16 input
+    hq, hs = mx.quantize_dynamic_scaled_float8(hidden_act, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32)
+    want_q, want_s = oracle.quantize_dynamic_scaled_fp8(bf16_bits(hidden_act), 128, threads=NT)
+    assert np.array_equal(fp8_bytes(hq), want_q) and np.array_equal(f32_np(hs)[:, :M], want_s)
+    # ... and the three-Linear route: the same block up to the stacked matmul's summation order and the single
+    # rounding of silu(gate) * up
+    want = mlp.down_proj(torch.nn.functional.silu(mlp.gate_proj(x)) * mlp.up_proj(x))
+    torch.cuda.synchronize()
+    assert_rel(f32_np(y), f32_np(want), 2e-2, "default route against the three linears")
+    # calling twice reuses the [0, rows] operand: no host tensor is built per call
+    assert len(mlp._row_offsets) == 1 and mlp(x) is not None and len(mlp._row_offsets) == 1
 
 
 @pytest.mark.parametrize("kw", [dict(has_bias=True), dict(activation_function="gelu"), dict(swiglu_limit=0.5)])

@@ -116,3 +116,54 @@ def test_fused_silu_feeds_the_down_projection(dev):
     act = g / (1 + torch.exp(-g)) * u
     ref = torch.cat([act[e * rows_per:(e + 1) * rows_per] @ w[e].T for e in range(E)])
     assert float((y - ref).abs().max()) <= 0.08 * float(ref.abs().max())
+
+
+def _exact_exp_input(max_rows, I, seed):
+    """gate values whose exp is fixed by f32 arithmetic alone, so that nothing of the op depends on an exp's last
+    bit: gate >= 17 gives 1 + exp(-gate) == 1 (exp(-17) < 2^-24) and silu(gate) = gate; gate <= -104 gives
+    exp(-gate) = inf and silu(gate) = -0.  The product gate * up of two bf16 values is exact in f32."""
+    gen = torch.Generator().manual_seed(seed)
+    gate = (17.0 + 60.0 * torch.rand((max_rows, I), generator=gen)).to(torch.bfloat16)
+    dead = torch.rand((max_rows, I), generator=gen) < 0.05
+    gate[dead] = torch.tensor(-120.0, dtype=torch.bfloat16)
+    up = (torch.randn((max_rows, I), generator=gen) * torch.exp(3.0 * torch.randn((max_rows, 1), generator=gen))).to(torch.bfloat16)
+    up[1, :128] = 0                                           # amax under the 1e-4 floor
+    up[2, :128] = up[2, :128] * 1e-5
+    return torch.cat([gate, up], dim=1), gate, up
+
+
+@pytest.mark.parametrize("max_rows,rows,I", [(64, 64, 2048), (1000, 913, 512), (4096, 4096, 2048)])
+def test_fused_silu_quantized_is_exact_where_exp_is(dev, max_rows, rows, I):
+    """On inputs whose exp is exact the op is byte work, and the kernel's division has to be the IEEE one:
+    scales and every fp8 byte equal the oracle's, and equal clamp(v / scale) worked out here from the exact
+    products v = silu(gate) * up with numpy's f32 division (ep_comm.mojo:4505-4624: value / scale, not value * (1 / scale))."""
+    x, gate, up = _exact_exp_input(max_rows, I, seed=rows + I)
+    off = torch.tensor([0, rows], dtype=torch.int64).to(torch.uint32)
+    q, s = mx.fused_silu_quantized(x.to(dev), off.to(dev), mx.blockwise_fp8_config())
+    torch.cuda.synchronize()
+    got_q, got_s = fp8_bytes(q)[:rows], s.cpu().numpy()[:, :rows]
+    # the oracle
+    want_q, want_s = oracle.fused_silu(_bits(x), rows, quantize=True, threads=NT)
+    assert np.array_equal(got_s, want_s[:, :rows]), "scales"
+    bad = np.argwhere(got_q != want_q[:rows])
+    assert bad.size == 0, f"{len(bad)} bytes differ from the oracle, first at {bad[:4].tolist()}"
+    # ... and the closed form
+    g, u = gate[:rows].float().numpy(), up[:rows].float().numpy()
+    v = np.where(g > 0, g, np.float32(-0.0)) * u                      # exact: 8 x 8 significant bits
+    amax = np.abs(v).reshape(rows, I // 128, 128).max(axis=2)
+    scale = np.maximum(amax, np.float32(1e-4)) / np.float32(448.0)
+    assert np.array_equal(got_s, scale.T)
+    quot = np.clip(v / np.repeat(scale, 128, axis=1), -448.0, 448.0).astype(np.float32)
+    assert np.array_equal(got_q, oracle.e4m3fn_encode(quot))
+
+
+def test_fused_silu_ignores_offsets_beyond_its_buffers(dev):
+    """row_offsets[-1] is read on the device; a value beyond max_rows (a stale routing tensor) is held to max_rows
+    instead of becoming accesses outside the buffers."""
+    max_rows, I = 24, 256
+    x, _, _ = _exact_exp_input(max_rows, I, seed=3)
+    xd = x.to(dev)
+    ok = mx.fused_silu(xd, torch.tensor([0, max_rows], dtype=torch.int64).to(torch.uint32).to(dev))
+    wild = mx.fused_silu(xd, torch.tensor([0, 1 << 30], dtype=torch.int64).to(torch.uint32).to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(ok, wild)

@@ -97,9 +97,34 @@ def test_linear_with_static_input_scale(dev):
     w = synth.weights_f32(N, K, seed=10)
     w_scale = float(w.abs().max()) / 448.0
     lin.weight.copy_((w / w_scale).clamp(-448, 448).to(torch.float8_e4m3fn).to(dev))
-    lin.weight_scale = torch.tensor(w_scale)
-    lin.input_scale = torch.tensor(float(x.float().abs().max()) / 448.0)
+    lin.weight_scale.fill_(w_scale)
+    lin.input_scale.fill_(float(x.float().abs().max()) / 448.0)
     y = lin(x.to(dev).reshape(4, 5, K))
     ref = (x.float() @ w.T).reshape(4, 5, N)
     assert tuple(y.shape) == (4, 5, N)
     assert float((y.float().cpu() - ref).abs().max()) <= 0.06 * float(ref.abs().max())
+
+
+def test_static_linear_loads_its_scales_from_a_state_dict(dev):
+    """A checkpoint's `weight`, `weight_scale` and `input_scale` go in through load_state_dict and the layer runs:
+    the two scalars stay on the CPU (the static ops take them from the host) wherever the module is moved."""
+    M, K, N = 24, 512, 256
+    x = synth.activations(M, K, seed=11, outlier_frac=0.0)
+    w = synth.weights_f32(N, K, seed=12)
+    w_scale = float(w.abs().max()) / 448.0
+    in_scale = float(x.float().abs().max()) / 448.0
+    state = {"weight": (w / w_scale).clamp(-448, 448).to(torch.float8_e4m3fn),
+             "weight_scale": torch.tensor(w_scale), "input_scale": torch.tensor(in_scale)}
+    lin = mx.Linear(K, N, _static_cfg(ScaleGranularity.TENSOR), device=dev)
+    assert set(lin.state_dict()) == {"weight", "weight_scale", "input_scale"}
+    lin.load_state_dict(state, strict=True)
+    lin = lin.to(dev)
+    assert lin.weight.is_cuda and lin.weight_scale.device.type == "cpu" and lin.input_scale.device.type == "cpu"
+    assert float(lin.input_scale) == float(torch.tensor(in_scale)) and float(lin.weight_scale) == float(torch.tensor(w_scale))
+    y = lin(x.to(dev))
+    ref = x.float() @ w.T
+    assert float((y.float().cpu() - ref).abs().max()) <= 0.06 * float(ref.abs().max())
+    # the same numbers as the op called by hand
+    want = mx.matmul_float8(x.to(dev), state["weight"].to(dev), state["weight_scale"], state["input_scale"],
+                            _static_cfg(ScaleGranularity.TENSOR))
+    assert torch.equal(y, want)

@@ -21,8 +21,8 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("tile", ["1", "2", "3", "4"])
 @pytest.mark.parametrize("M,N,K", [(300, 392, 1040), (257, 100, 512), (64, 129, 384), (513, 520, 256)])
-def test_each_tile_shape_exact(dev, monkeypatch, tile, M, N, K):
-    monkeypatch.setenv("MAXFP8_TILE", tile)
+def test_each_tile_shape_exact(dev, tune, tile, M, N, K):
+    tune(MAXFP8_TILE=tile)
     a, b, sa, sb, want = exact_case(M, N, K, seed=M + N + K)
     got = f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled")).astype(np.float64)
     bad = np.argwhere(got != want)
@@ -32,8 +32,8 @@ def test_each_tile_shape_exact(dev, monkeypatch, tile, M, N, K):
 
 
 @pytest.mark.parametrize("tile", ["1", "2", "3"])
-def test_each_tile_shape_rowwise(dev, monkeypatch, tile):
-    monkeypatch.setenv("MAXFP8_TILE", tile)
+def test_each_tile_shape_rowwise(dev, tune, tile):
+    tune(MAXFP8_TILE=tile)
     M, N, K = 300, 1044, 1024
     a, b = synth.random_fp8((M, K), M), synth.random_fp8((N, K), N)
     sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
@@ -45,9 +45,9 @@ def test_each_tile_shape_rowwise(dev, monkeypatch, tile):
 
 @pytest.mark.parametrize("splits", ["2", "3", "4"])
 @pytest.mark.parametrize("kind", ["block", "row"])
-def test_split_k_exact(dev, monkeypatch, splits, kind):
+def test_split_k_exact(dev, tune, splits, kind):
     # forced split counts (at most one per 4 slabs); the shares are uneven (17 slabs)
-    monkeypatch.setenv("MAXFP8_SPLITK", splits)
+    tune(MAXFP8_SPLITK=splits)
     M, N, K = 130, 264, 17 * 128
     if kind == "block":
         a, b, sa, sb, want = exact_case(M, N, K, seed=int(splits))
@@ -131,8 +131,8 @@ GROUPED = [
 @pytest.mark.parametrize("tile", ["0", "2", "3", "4"])
 @pytest.mark.parametrize("counts,ids,E,N,K", GROUPED)
 @pytest.mark.parametrize("out", [torch.float32, torch.bfloat16])
-def test_grouped_tile_kinds(dev, monkeypatch, tile, counts, ids, E, N, K, out):
-    monkeypatch.setenv("MAXFP8_TILE", tile)
+def test_grouped_tile_kinds(dev, tune, tile, counts, ids, E, N, K, out):
+    tune(MAXFP8_TILE=tile)
     args = make_grouped(counts, ids, E, N, K, seed=sum(counts) + N)
     c = run_grouped(*args, max(counts), len(counts), dev, out=out, algo="tiled")
     assert_rel(f32_np(c), ref_grouped(*args, max(counts), len(counts)), TOL, f"grouped {counts} tile {tile}",
@@ -200,8 +200,8 @@ PERSIST_SHAPES = [(512, 512, 256), (4096, 8192, 256), (2560, 7680, 384), (8192, 
 
 @pytest.mark.parametrize("M,N,K", PERSIST_SHAPES)
 @pytest.mark.parametrize("kind", ["block", "row"])
-def test_persistent_kernel_equals_per_tile_kernel(dev, monkeypatch, M, N, K, kind):
-    monkeypatch.setenv("MAXFP8_TILE", "1")
+def test_persistent_kernel_equals_per_tile_kernel(dev, tune, M, N, K, kind):
+    tune(MAXFP8_TILE="1")
     if kind == "block":
         a, b, sa, sb = make_block(M, N, K, seed=M + K)
         cfg = BLK
@@ -215,7 +215,7 @@ def test_persistent_kernel_equals_per_tile_kernel(dev, monkeypatch, M, N, K, kin
                                            algo="tiled")
     got = run()
     again = run()  # a second launch on the same stream: same bits
-    monkeypatch.setenv("MAXFP8_PERSIST", "0")
+    tune(MAXFP8_PERSIST="0")
     want = run()
     torch.cuda.synchronize()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
@@ -223,35 +223,35 @@ def test_persistent_kernel_equals_per_tile_kernel(dev, monkeypatch, M, N, K, kin
 
 
 @pytest.mark.parametrize("M,N,K", [(512, 768, 384), (2560, 7680, 144)])
-def test_persistent_kernel_exact(dev, monkeypatch, M, N, K):
-    monkeypatch.setenv("MAXFP8_TILE", "1")
+def test_persistent_kernel_exact(dev, tune, M, N, K):
+    tune(MAXFP8_TILE="1")
     a, b, sa, sb, want = exact_case(M, N, K, seed=M + N + K)
     cb = mm(a, b, sa, sb, BLK, dev, out=torch.bfloat16, algo="tiled")
     assert torch.equal(cb.cpu(), torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16))
 
 
-def test_persistent_kernel_leaves_other_outputs_alone(dev, monkeypatch):
+def test_persistent_kernel_leaves_other_outputs_alone(dev, tune):
     # f32 output, rows of C that are not 16-byte aligned and partial tiles stay with the per-tile kernel
-    monkeypatch.setenv("MAXFP8_TILE", "1")
+    tune(MAXFP8_TILE="1")
     a, b, sa, sb, want = exact_case(512, 520, 256, seed=9)
     assert np.array_equal(f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled")).astype(np.float64), want)
     a, b, sa, sb, want = exact_case(512, 512, 256, seed=10)
     assert np.array_equal(f32_np(mm(a, b, sa, sb, BLK, dev, algo="tiled")).astype(np.float64), want)
 
 
-def test_persistent_kernel_many_tiles_per_block_repeated(dev, monkeypatch):
+def test_persistent_kernel_many_tiles_per_block_repeated(dev, tune):
     # short K, sixteen tiles per block: the stores of one tile are still in flight when the next tile's first slab
     # is waited for.  Twelve launches with fresh activations, each compared with the per-tile kernel.
-    monkeypatch.setenv("MAXFP8_TILE", "1")
+    tune(MAXFP8_TILE="1")
     M, N, K = 8192, 32768, 256
     b = synth.random_fp8((N, K), 77).to(dev)
     sb = synth.random_scales((N // 128, K // 128), 78).to(dev)
     sa = synth.random_scales((K // 128, M), 79).to(dev)
     for seed in range(12):
         a = synth.random_fp8((M, K), 100 + seed).to(dev)
-        monkeypatch.setenv("MAXFP8_PERSIST", "1")
+        tune(MAXFP8_PERSIST="1")
         got = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
-        monkeypatch.setenv("MAXFP8_PERSIST", "0")
+        tune(MAXFP8_PERSIST="0")
         want = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
         torch.cuda.synchronize()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"launch {seed}"

@@ -61,6 +61,25 @@ def test_c_abi_argument_errors_need_no_gpu():
                                               4, 1, 0, 0, 0, None, 0, None) == _lib.ERR_DTYPE
 
 
+def test_row_strides_beyond_the_tile_offsets_are_refused():
+    """The MFMA kernels address a tile through 32-bit offsets with the top bit as the out-of-range mark: a strided
+    view whose 256 rows span 2^31 bytes must not reach them (it would read zeros for rows that exist)."""
+    L = _lib.lib()
+    big = (1 << 23) + 16          # 256 * big >= 2^31
+    for algo in (_lib.ALGO_TILED, _lib.ALGO_SKINNY):
+        for lda, ldb in ((big, 128), (128, big)):
+            st = L.maxfp8_matmul_dynamic_scaled_fp8(16, 16, 16, 16, 16, 4, 8, 128, lda, ldb, 8, 2, 1, -1, -1, -1,
+                                                    4, 1, 0, 2, algo, None, 0, None)
+            assert st == _lib.ERR_ALIGN and "2^31" in _lib.last_error()
+    # block scaling: the scales of all slabs of a tile, ceil(K / 128) * a_scales_ld floats, share one offset range
+    st = L.maxfp8_matmul_dynamic_scaled_fp8(16, 16, 16, 16, 16, 4, 128, 128 * 1024, 128 * 1024, 128 * 1024, 128, 3, 3,
+                                            1, 128, 128, 1 << 20, 1024, 0, 2, _lib.ALGO_TILED, None, 0, None)
+    assert st == _lib.ERR_ALIGN
+    st = L.maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8(16, 16, 16, 16, 16, 16, 16, 8, 128, 1 << 23, 2, 8, 2,
+                                                            0, 2, None)
+    assert st == _lib.ERR_SHAPE and "32-bit" in _lib.last_error()
+
+
 def test_quantize_geometry_rules():
     g = kernels.quantize_output_geometry
     assert g(81, 2048, BLK.input_scale, BLK.weight_scale, -1, torch.float32) == (128, 84)   # pad to 16 bytes
@@ -198,7 +217,9 @@ def test_mlp_stacks_gate_and_up_in_one_buffer():
     import modular_amd as mx
 
     m = mx.MLP(256, 512, mx.blockwise_fp8_config())
-    assert m._one_matmul and m._fused()
+    # the one-kernel activation + quantisation is an opt-in: its recipe is not the one down_proj applies
+    assert m._one_matmul and m._silu_kernel() and not m._fused()
+    assert mx.MLP(256, 512, mx.blockwise_fp8_config(), fuse_activation_quant=True)._fused()
     assert sorted(m.state_dict()) == ["down_proj.weight", "down_proj.weight_scale", "gate_proj.weight",
                                       "gate_proj.weight_scale", "up_proj.weight", "up_proj.weight_scale"]
     new = {k: (torch.randint(0, 100, v.shape, dtype=torch.uint8).view(v.dtype) if v.dtype == torch.float8_e4m3fn
@@ -212,5 +233,46 @@ def test_mlp_stacks_gate_and_up_in_one_buffer():
     assert torch.equal(m.gate_up_weight[:512].view(torch.uint8), new["gate_proj.weight"].view(torch.uint8))
     # per-token scales stack as well; static or per-tensor scales, bias or another activation take the unfused route
     assert mx.MLP(256, 512, mx.rowwise_fp8_config())._one_matmul
-    assert not mx.MLP(256, 512, mx.blockwise_fp8_config(), has_bias=True)._fused()
-    assert not mx.MLP(256, 512, mx.blockwise_fp8_config(), activation_function="gelu")._fused()
+    assert not mx.MLP(256, 512, mx.blockwise_fp8_config(), has_bias=True, fuse_activation_quant=True)._fused()
+    assert not mx.MLP(256, 512, mx.blockwise_fp8_config(), activation_function="gelu", fuse_activation_quant=True)._fused()
+    assert not mx.MLP(256, 512, mx.rowwise_fp8_config(), fuse_activation_quant=True)._fused()
+
+
+def test_quantized_grouped_matmul_and_strategy_argument_rules():
+    """The layer above the grouped op (quant_ops.py:880-1007, moe/quant_strategy.py:114-215): format and rank
+    checks happen before anything touches the GPU, and the storage-layout transposition is made once per tensor."""
+    import dataclasses
+
+    from modular_amd import quant_ops
+
+    x = torch.zeros((4, 256), dtype=torch.bfloat16)
+    w = torch.zeros((2, 256, 128), dtype=torch.uint8).view(FP8)       # storage layout [E, K, N]
+    ws = torch.ones((2, 2, 1))
+    off = torch.tensor([0, 2, 4], dtype=torch.int64).to(torch.uint32)
+    ids = torch.tensor([0, 1], dtype=torch.int32)
+    stats = torch.tensor([2, 2], dtype=torch.int64).to(torch.uint32)
+    bad = dataclasses.replace(BLK, format="mxfp4")
+    with pytest.raises(ValueError, match="Unsupported quantization format for grouped matmul"):
+        quant_ops.quantized_grouped_matmul(x, w, ws, off, ids, stats, bad)
+    with pytest.raises(ValueError, match="rank 3"):
+        quant_ops.quantized_grouped_matmul(x, w[0], ws, off, ids, stats, BLK)
+    # [E, K, N] -> [E, N, K], contiguous, kept per storage tensor until it is written in place
+    quant_ops._K_INNERMOST.clear()
+    src = torch.arange(2 * 3 * 5, dtype=torch.uint8).reshape(2, 3, 5).view(FP8)
+    t1 = quant_ops._k_innermost(src)
+    assert tuple(t1.shape) == (2, 5, 3) and t1.is_contiguous()
+    assert torch.equal(t1.view(torch.uint8), src.view(torch.uint8).transpose(1, 2))
+    assert quant_ops._k_innermost(src) is t1
+    src.view(torch.uint8).add_(1)
+    t2 = quant_ops._k_innermost(src)
+    assert t2 is not t1 and torch.equal(t2.view(torch.uint8), src.view(torch.uint8).transpose(1, 2))
+    quant_ops._K_INNERMOST.clear()
+    # a CPU tensor never reaches a kernel
+    with pytest.raises(RuntimeError, match="GPU only"):
+        quant_ops.quantized_grouped_matmul(x, w, torch.ones((2, 2, 1)), off, ids, stats, BLK)
+    st = mx.Fp8Strategy(BLK)
+    assert st.dtype == FP8 and st.config is BLK
+    a, b = st.prepare_weight_scales(ws, off, None)
+    assert a is ws and b is off
+    with pytest.raises(RuntimeError, match="GPU only"):
+        st.quantize(x, 128)
