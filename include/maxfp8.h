@@ -180,6 +180,33 @@ int maxfp8_matmul_dynamic_scaled_fp8(
     void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * maxfp8_matmul_dynamic_scaled_fp8 for callers that cannot allocate device memory -- code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc -- and therefore cannot bring a
+ * workspace.  No counterpart in the reference (its matmul takes temporaries from the device context's
+ * caching allocator).  Same arguments without workspace / workspace_bytes, same result: the split-K
+ * partial sums go to a static device array of the library,
+ * maxfp8_matmul_noalloc_max_scratch_bytes() = 32 MiB per GPU, held from the first use of the library on
+ * that GPU until the process ends.  The call allocates and frees nothing, on the device or through any
+ * library.  A shape whose K split needs more than the array holds (splits x M x N x 4 bytes; the large-M,
+ * narrow-N shapes) is refused with MAXFP8_ERR_WORKSPACE and a message that says so: for those,
+ * maxfp8_matmul_dynamic_scaled_fp8 with workspace = NULL runs unsplit and allocates nothing either.  All calls on one GPU share that GPU's array: calls
+ * that overlap on one GPU (two streams, two threads) race on it; calls in stream order are safe, and
+ * nothing in the array needs clearing between them.
+ */
+int maxfp8_matmul_dynamic_scaled_fp8_noalloc(
+    void* c, const void* a, const void* b,
+    const void* a_scales, const void* b_scales,
+    int64_t M, int64_t N, int64_t K,
+    int64_t lda, int64_t ldb, int64_t ldc,
+    int input_granularity, int weight_granularity,
+    int64_t gm, int64_t gn, int64_t gk,
+    int64_t a_scales_ld, int64_t b_scales_ld,
+    int c_dtype, int scales_dtype, int algo, void* stream);
+
+/* Size of the static scratch array behind maxfp8_matmul_dynamic_scaled_fp8_noalloc. */
+size_t maxfp8_matmul_noalloc_max_scratch_bytes(void);
+
+/*
  * Batched blockwise-scaled FP8 matmul: C[b] = A[b] . B[b]^T for b < B in one
  * launch.  Replaces Struct_batched_matmul_dynamic_scaled_fp8.execute
  *   (max/kernels/src/graph_compiler/builtin_kernels/linalg.mojo:1041-1090)

@@ -30,6 +30,8 @@ EXPORTS = (
     "maxfp8_grouped_matmul_dynamic_scaled_fp8_scatter",
     "maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8",
     "maxfp8_matmul_dynamic_scaled_fp8",
+    "maxfp8_matmul_dynamic_scaled_fp8_noalloc",
+    "maxfp8_matmul_noalloc_max_scratch_bytes",
     "maxfp8_batched_matmul_dynamic_scaled_fp8",
     "maxfp8_matmul_workspace_bytes",
     "maxfp8_matmul_describe",
@@ -83,6 +85,10 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_matmul_dynamic_scaled_fp8.restype = ci
     L.maxfp8_matmul_dynamic_scaled_fp8.argtypes = ([vp] * 5 + [i64] * 6 + [ci, ci] + [i64] * 5 +
                                                   [ci, ci, ci, vp, ctypes.c_size_t, vp])
+    L.maxfp8_matmul_dynamic_scaled_fp8_noalloc.restype = ci
+    L.maxfp8_matmul_dynamic_scaled_fp8_noalloc.argtypes = ([vp] * 5 + [i64] * 6 + [ci, ci] + [i64] * 5 + [ci, ci, ci, vp])
+    L.maxfp8_matmul_noalloc_max_scratch_bytes.restype = ctypes.c_size_t
+    L.maxfp8_matmul_noalloc_max_scratch_bytes.argtypes = []
     L.maxfp8_batched_matmul_dynamic_scaled_fp8.restype = ci
     L.maxfp8_batched_matmul_dynamic_scaled_fp8.argtypes = [vp] * 5 + [i64] * 17 + [ci, ci, ci, vp]
     L.maxfp8_matmul_describe.restype = ci

@@ -50,6 +50,7 @@ int naive_grouped_dispatch(void*, const void*, const void*, const void*, const v
                            const int32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, hipStream_t);
 int gemm_tiled_dispatch(const GemmArgs&, bool, size_t, int64_t, hipStream_t);
 size_t gemm_tiled_workspace_bytes(int64_t, int64_t, int64_t);
+size_t gemm_tiled_plan_workspace_bytes(int64_t, int64_t, int64_t, bool);
 int gemm_tiled_describe(int64_t, int64_t, int64_t, bool, bool, char*, size_t);
 int gemm_grouped_dispatch(const GemmArgs&, bool, int64_t, int64_t, hipStream_t);
 int gemm_skinny_dispatch(const GemmArgs&, bool, int64_t, hipStream_t);
@@ -72,6 +73,36 @@ static float round_to_dtype(float v, int dtype) {
 }
 
 static bool is_aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---- the library's own scratch memory (maxfp8_matmul_dynamic_scaled_fp8_noalloc) ------------------
+// A file-scope device array: every GPU the library runs on holds its own copy, at its own address, from the
+// moment the code object is loaded there until the process ends.  In host code the array's NAME is only a handle
+// for hipGetSymbolAddress -- it is not a device address and is never passed to a kernel or a memory call.  The
+// address is looked up once per device, with that device current, and kept; kernels receive it as an argument,
+// exactly like a caller's workspace.
+constexpr size_t kScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+static void* g_scratch_ptr[64] = {};
+static std::mutex g_scratch_mu;
+
+static int scratch_of_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= 64)
+    MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "matmul (no-alloc): no current device in 0..63: %s", hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "matmul (no-alloc): cannot resolve the scratch array on device %d: %s", dev, hipGetErrorString(e));
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MAXFP8_OK;
+}
 
 // The MFMA kernels address a tile's operands with 32-bit buffer offsets whose top bit marks lanes that are out of
 // range: the rows of the tallest tile (256) times the row stride, and the activation scales of all slabs of a tile
@@ -401,6 +432,36 @@ int maxfp8_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, cons
   const BatchStrides one = {1, 0, 0, 0, 0, 0};
   return matmul_common(c, a, b, a_scales, b_scales, M, N, K, lda, ldb, ldc, input_granularity, weight_granularity, gm, gn,
                        gk, a_scales_ld, b_scales_ld, c_dtype, scales_dtype, algo, workspace, workspace_bytes, one, stream);
+}
+
+size_t maxfp8_matmul_noalloc_max_scratch_bytes(void) { return kScratchBytes; }
+
+int maxfp8_matmul_dynamic_scaled_fp8_noalloc(void* c, const void* a, const void* b, const void* a_scales,
+                                             const void* b_scales, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                             int64_t ldb, int64_t ldc, int input_granularity, int weight_granularity,
+                                             int64_t gm, int64_t gn, int64_t gk, int64_t a_scales_ld, int64_t b_scales_ld,
+                                             int c_dtype, int scales_dtype, int algo, void* stream) {
+  // The scratch of the K split this shape gets when its caller brings all the workspace
+  // maxfp8_matmul_workspace_bytes asks for: with exactly that much the planner lands on the same plan, so both
+  // entry points add the same partial sums in the same order.
+  const bool block = input_granularity == MAXFP8_GRAN_BLOCK && weight_granularity == MAXFP8_GRAN_BLOCK;
+  size_t need = 0;
+  if (M > 0 && N > 0 && K > 0 && maxfp8_matmul_workspace_bytes(M, N, K) > 0) need = gemm_tiled_plan_workspace_bytes(M, N, K, block);
+  if (need > kScratchBytes)
+    MAXFP8_FAIL(MAXFP8_ERR_WORKSPACE,
+                "matmul (no-alloc): the K split of %lld x %lld x %lld uses %zu bytes of scratch, the library's static buffer holds "
+                "%zu; call maxfp8_matmul_dynamic_scaled_fp8 with workspace = NULL (no split, no allocation) or with a workspace",
+                (long long)M, (long long)N, (long long)K, need, kScratchBytes);
+  void* ws = nullptr;
+  if (need > 0 && M > 0 && N > 0) {
+    const int rc = scratch_of_current_device(&ws);
+    if (rc != MAXFP8_OK) return rc;
+  }
+  // (Nothing in the scratch has to start at zero: every partial tile a split writes is written in full before the
+  // reduction reads it.  Its contents after the call are the last call's partial sums.)
+  const BatchStrides one = {1, 0, 0, 0, 0, 0};
+  return matmul_common(c, a, b, a_scales, b_scales, M, N, K, lda, ldb, ldc, input_granularity, weight_granularity, gm, gn,
+                       gk, a_scales_ld, b_scales_ld, c_dtype, scales_dtype, algo, ws, ws ? need : 0, one, stream);
 }
 
 int maxfp8_batched_matmul_dynamic_scaled_fp8(void* c, const void* a, const void* b, const void* a_scales,

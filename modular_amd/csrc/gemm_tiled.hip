@@ -1312,6 +1312,13 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
   return plan;
 }
 
+// The split-K scratch of the plan an unlimited workspace gets (0: that plan does not split).  A workspace of this size --
+// or of gemm_tiled_workspace_bytes, which is never smaller -- leads to this same plan.
+size_t gemm_tiled_plan_workspace_bytes(int64_t M, int64_t N, int64_t K, bool blockscale) {
+  const TiledPlan plan = make_plan(M, N, K, blockscale, true, ~(size_t)0, 1, false);
+  return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)N * 4 : 0;
+}
+
 // make_plan tries every cut of every pair of shapes: microseconds of host time, as much as a small matmul
 // takes on the GPU.  Plans are kept in a small table, keyed by everything make_plan reads (the generation
 // of the tuning switches included, since tests and tuning runs reload them between calls).

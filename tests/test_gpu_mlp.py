@@ -99,11 +99,13 @@ def test_block_scaled_mlp_default_route_quantises_like_a_linear(dev, M, hidden, 
     hq, hs = mx.quantize_dynamic_scaled_float8(hidden_act, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32)
     want_q, want_s = oracle.quantize_dynamic_scaled_fp8(bf16_bits(hidden_act), 128, threads=NT)
     assert np.array_equal(fp8_bytes(hq), want_q) and np.array_equal(f32_np(hs)[:, :M], want_s)
-    # ... and the three-Linear route: the same block up to the stacked matmul's summation order and the single
-    # rounding of silu(gate) * up
+    # ... and the three-Linear route with torch's bf16 silu and product between them: the same block up to one
+    # rounding of silu(gate) * up instead of two, which moves about one fp8 code in a hundred by a step in front of
+    # the second matmul -- fp8 quantisation noise, a per cent of the result's norm
     want = mlp.down_proj(torch.nn.functional.silu(mlp.gate_proj(x)) * mlp.up_proj(x))
     torch.cuda.synchronize()
-    assert_rel(f32_np(y), f32_np(want), 2e-2, "default route against the three linears")
+    diff = (y.double() - want.double()).norm() / want.double().norm()
+    assert float(diff) < 0.03, f"default route against the three linears: relative difference {float(diff):.3f}"
     # calling twice reuses the [0, rows] operand: no host tensor is built per call
     assert len(mlp._row_offsets) == 1 and mlp(x) is not None and len(mlp._row_offsets) == 1
 
@@ -143,7 +145,9 @@ def test_per_token_mlp_runs_gate_and_up_as_one_matmul(dev):
     y = mlp(x)
     want = mlp.down_proj(torch.nn.functional.silu(mlp.gate_proj(x)) * mlp.up_proj(x))
     torch.cuda.synchronize()
-    assert_rel(f32_np(y), f32_np(want), 2e-2, "per-token MLP")
+    # (one rounding of silu(gate) * up instead of torch's two: a few fp8 codes differ in front of down_proj)
+    diff = (y.double() - want.double()).norm() / want.double().norm()
+    assert float(diff) < 0.03, f"per-token MLP against its three linears: relative difference {float(diff):.3f}"
 
 
 def test_mlp_argument_checks(dev):
