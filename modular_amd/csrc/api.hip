@@ -125,7 +125,7 @@ static const Tuning* read_tuning(unsigned generation) {
   t->splitk = num("MAXFP8_SPLITK", 0);
   t->one_region = getenv("MAXFP8_ONE_REGION") != nullptr;
   t->persist = num("MAXFP8_PERSIST", 1) != 0;
-  t->streamk = num("MAXFP8_STREAMK", 1) != 0;
+  t->streamk = num("MAXFP8_STREAMK", 1);
   t->big_rows = num("MAXFP8_BIG_ROWS", 1024);
   t->grouped_overlap = num("MAXFP8_GROUPED_OVERLAP", 1) != 0;
   const char* sb = getenv("MAXFP8_GROUPED_SHARE");

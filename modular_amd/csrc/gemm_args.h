@@ -56,6 +56,9 @@ struct GemmArgs {
   // split-K / skinny only
   float* workspace;
   int splits;
+  // work split along K of the persistent kernel: which set of hand-over flags this launch uses, and the value a flag takes
+  int streamk_slot;
+  unsigned int streamk_seq;
   // fused QKV only
   int kv_on;
   KvStore kv;

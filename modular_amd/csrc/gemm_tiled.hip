@@ -40,6 +40,7 @@
 // caps the wave tile at 128 x 64 with two waves per SIMD.
 #include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 #include <utility>
 #include "common.h"
@@ -65,6 +66,19 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t t2_rsrc(const void* p, uint32_
 }
 __device__ __forceinline__ uint32_t t2_clamp_u32(int64_t v) {
   return v > 0xfffffff0ll ? 0xfffffff0u : (v < 0 ? 0u : (uint32_t)v);
+}
+
+// A 16-byte buffer store whose scalar offset sits in a register.  The hardware reads the four data registers of such
+// a store during the cycles AFTER it has issued, and a VALU instruction that follows at once and writes one of them
+// changes what is stored; the compiler's hazard table has this case down as free of hazards (it pads only stores whose
+// scalar offset is an immediate) and schedules the next values straight into the registers.  Seen on MI355X as a
+// tile's bf16 pairs replaced, in some lanes, by the f32 products of the rows computed next.  The wait states are tied
+// to the data registers, so that nothing that overwrites them can be scheduled between the store and the wait.
+typedef unsigned int v4u_t __attribute__((ext_vector_type(4)));
+template <int CACHE_POLICY>
+__device__ __forceinline__ void buffer_store_b128_guarded(const v4u_t v, const __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset, uint32_t soffset) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, voffset, soffset, CACHE_POLICY);
+  asm volatile("s_nop 7" ::"v"(v));
 }
 
 // One BM x BN tile of C: rows [row_begin, row_end) (at most BM of them are used) by columns
@@ -611,7 +625,28 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
 // may skip would make the count a guess.)
 //
 // Same arithmetic, in the same order, as tile_body: results are bit-equal to gemm_tiled_kernel's.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE>
+//
+// SPLIT (work split along K, "stream-K"): the work is counted in units of one slab of one tile, in
+// tile order, and block l takes the units [l * U / G, (l + 1) * U / G): the same number for every
+// block, whatever the number of tiles -- 448 tiles on 256 CUs are 1.75 tiles each instead of two
+// rounds of which the second is three quarters empty.  A tile that a block boundary cuts is begun
+// by block l - 1 (slabs 0 .. s - 1) and finished by block l (slabs s .. end).  The f32
+// accumulators travel through the workspace, so the tile's sum is formed in the same order as by
+// one block and the result stays bit-equal to the other kernels'.  A block works in the order
+//     1. the tile it begins (the LAST of its range): accumulators -> workspace slot l + 1, then flag l + 1
+//     2. its whole tiles
+//     3. the tile it finishes (the FIRST of its range): waits for flag l, accumulators <- slot l
+// so that what a block waits for is the first thing its predecessor does, and that depends on nothing:
+// no block ever waits for a block that waits (with the host's rule of at least one tile per block a tile
+// has at most two parts).  The hand-over crosses CUs and possibly XCDs, whose L2 caches are not coherent
+// with each other: partial sums and flags are written and read with the device-scope cache policy (write
+// through / miss always), the flag only after the writer's stores have completed.  Flags hold the launch's
+// sequence number, so nothing has to be cleared between launches.  The wait is bounded; a block that gives
+// up (its predecessor never ran: a hung GPU) poisons its tile with NaN instead of hanging too.
+constexpr int kStreamkSlots = 64, kStreamkMaxBlocks = 512;
+static __device__ unsigned int g_streamk_flags[kStreamkSlots * kStreamkMaxBlocks];
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE, bool SPLIT>
 __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   constexpr int NS = 2;
   constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -623,6 +658,7 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   constexpr int PER = IA + IB + (BLOCKSCALE ? 1 : 0);
   constexpr int SIDE_BYTES = 16 * WN * 2;  // a wave's side buffer: 16 rows of its part of the tile
   constexpr int NSTORE = TM * 2;           // 16-byte stores per lane and tile
+  constexpr int PARTIAL_BYTES = BM * BN * 4;  // the accumulators of a tile: one workspace slot
   static_assert(WN == 64 && BM % 64 == 0 && NWAVES % 2 == 0 && IA >= 1 && IB >= 1 && TN % 2 == 0, "tile / wave layout");
   static_assert(NSTORE < 64, "the count must fit the vmcnt field");
 
@@ -630,15 +666,50 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int lm = lane & 15, lq = lane >> 4;
+  const int nslab = (p.K + 127) / 128;
 
-  // ---- this block's tiles: every 'nb'-th tile of its XCD's contiguous run (blocks are dealt to the XCDs round-robin)
+  // ---- this block's jobs.  A job is (tile, first slab, end slab, kind): WHOLE tiles start from zero and store C;
+  // a HEAD starts from zero and hands its accumulators on; a TAIL takes them over and stores C.
+  enum { WHOLE = 0, HEAD = 1, TAIL = 2 };
+  struct Job { int tile, s0, s1, kind; };
   const int tiles_m = p.M / BM, tiles_n = p.N / BN, total = tiles_m * tiles_n;
   const int xcd = blockIdx.x & 7;
+  int njobs;
+  // persistent: every 'nb'-th tile of the XCD's contiguous run (blocks are dealt to the XCDs round-robin)
   const int run_begin = xcd * (total >> 3) + (xcd < (total & 7) ? xcd : (total & 7));
   const int run_len = (total >> 3) + (xcd < (total & 7) ? 1 : 0);
   const int nb = ((int)gridDim.x - xcd + 7) >> 3;
-  int my = blockIdx.x >> 3;
-  if (my >= run_len) return;
+  const int my = blockIdx.x >> 3;
+  // split: logical block number l = position in XCD order, so that neighbours in l share an L2 but for 7 pairs
+  const int per_xcd = (int)gridDim.x >> 3;           // (the host launches a multiple of 8 blocks)
+  const int l = xcd * per_xcd + my;
+  int t_first = 0, t_last = 0, s_first = 0, s_last_end = 0, nwhole = 0;
+  bool has_head = false, has_tail = false;
+  if constexpr (SPLIT) {
+    const int64_t U = (int64_t)total * nslab, G = gridDim.x;
+    const int64_t ub = (int64_t)l * U / G, ue = (int64_t)(l + 1) * U / G;
+    t_first = (int)(ub / nslab);
+    s_first = (int)(ub - (int64_t)t_first * nslab);
+    t_last = (int)((ue - 1) / nslab);
+    s_last_end = (int)(ue - (int64_t)t_last * nslab);
+    has_tail = s_first != 0;
+    has_head = s_last_end != nslab;
+    nwhole = t_last - t_first + 1 - (has_tail ? 1 : 0) - (has_head ? 1 : 0);
+    njobs = nwhole + (has_tail ? 1 : 0) + (has_head ? 1 : 0);
+  } else {
+    njobs = my < run_len ? (run_len - my + nb - 1) / nb : 0;
+  }
+  if (njobs <= 0) return;
+  auto get_job = [&](int k) -> Job {
+    if constexpr (SPLIT) {
+      if (has_head && k == 0) return Job{t_last, 0, s_last_end, HEAD};
+      const int w = k - (has_head ? 1 : 0);
+      if (w < nwhole) return Job{t_first + (has_tail ? 1 : 0) + w, 0, nslab, WHOLE};
+      return Job{t_first, s_first, nslab, TAIL};
+    } else {
+      return Job{run_begin + my + k * nb, 0, nslab, WHOLE};
+    }
+  };
 
   // ---- global -> LDS copy plan: as in tile_body, with the tile's position in the scalar offset
   const __amdgpu_buffer_rsrc_t a_rsrc = t2_rsrc(p.a, t2_clamp_u32((int64_t)(p.M - 1) * p.lda + p.K));
@@ -650,7 +721,6 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   const uint32_t b_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.ldb + cchunk_b * 16;
   const uint32_t a_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.lda;
   const uint32_t b_istep = (uint32_t)(NWAVES * 8) * (uint32_t)p.ldb;
-  const int nslab = (p.K + 127) / 128;
   const int s_chunk = wave % (BM / 64);
   __amdgpu_buffer_rsrc_t s_rsrc = t2_rsrc(nullptr, 0);
   uint32_t s_voff = 0, s_slab_step = 0;
@@ -711,33 +781,73 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   const uint32_t c_row_bytes = (uint32_t)p.ldc * 2u;
   const uint32_t c_lane = (uint32_t)rr * c_row_bytes + (uint32_t)cc * 16u;
 
+  // ---- hand-over of accumulators between blocks (SPLIT): slot i = PARTIAL_BYTES at workspace + i * PARTIAL_BYTES,
+  // a wave's part at wave * (PARTIAL_BYTES / NWAVES), fragment (mt, nt) as 64 lanes x 16 bytes.  Cache policy 17 =
+  // sc0 | sc1: device scope (stores go through to memory, loads do not hit a line of this XCD's L2).
+  typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+  [[maybe_unused]] const __amdgpu_buffer_rsrc_t w_rsrc =
+      SPLIT ? t2_rsrc(p.workspace, t2_clamp_u32((int64_t)gridDim.x * PARTIAL_BYTES)) : t2_rsrc(nullptr, 0);
+  [[maybe_unused]] unsigned int* const flags = g_streamk_flags + (size_t)p.streamk_slot * kStreamkMaxBlocks;
+  constexpr int kDeviceScope = 17;
+
+  Job cur = get_job(0);
   int tm, tn;
-  tile_coords(run_begin + my, tiles_m, tiles_n, tm, tn);
-  TileAt cur = tile_at(tm, tn);
+  tile_coords(cur.tile, tiles_m, tiles_n, tm, tn);
+  TileAt cur_at = tile_at(tm, tn);
 #pragma unroll
-  for (int idx = 0; idx < PER; ++idx) dma_one(cur, 0, 0, idx, 0u);
+  for (int idx = 0; idx < PER; ++idx) dma_one(cur_at, cur.s0, 0, idx, 0u);
   float bs_nxt = 1.f;
-  if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld];
+  if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld + cur.s0];
 
   int buf = 0;
   bool stored = false;  // the wave's last vector memory operations are a tile's NSTORE stores
-  while (true) {
-    const int nxt = my + nb;
-    const bool has_next = nxt < run_len;
+  for (int k = 0; k < njobs; ++k) {
+    const bool has_next = k + 1 < njobs;
+    Job nxt = cur;
     int tm2 = tm, tn2 = tn;
-    if (has_next) tile_coords(run_begin + nxt, tiles_m, tiles_n, tm2, tn2);
-    const TileAt next = tile_at(tm2, tn2);
+    if (has_next) {
+      nxt = get_job(k + 1);
+      tile_coords(nxt.tile, tiles_m, tiles_n, tm2, tn2);
+    }
+    const TileAt next_at = tile_at(tm2, tn2);
     const float* bs_row = nullptr;
     if constexpr (BLOCKSCALE) bs_row = p.b_scales + (int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld;
 
     v4f acc[TM][TN];
+    bool took_over = false;
+    if constexpr (SPLIT) {
+      if (cur.kind == TAIL) {
+        // the predecessor's first job: in practice long done.  Every lane reads the same word.
+        took_over = true;
+        bool there = false;
+        for (int spin = 0; spin < (1 << 22); ++spin) {
+          if (__hip_atomic_load(flags + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.streamk_seq) { there = true; break; }
+          __builtin_amdgcn_s_sleep(16);
+        }
+        asm volatile("" ::: "memory");
+        // (the slot's address is formed here, out of sight of the optimiser: hoisted out of the job loop, the 32
+        // fragment offsets would sit in scalar registers for the whole kernel)
+        uint32_t base = (uint32_t)l * PARTIAL_BYTES + (uint32_t)wave * (PARTIAL_BYTES / NWAVES);
+        asm volatile("" : "+s"(base));
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+          for (int j = 0; j < TN; ++j) {
+            const v4u v = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (uint32_t)lane * 16u, base + (uint32_t)(i * TN + j) * 1024u, kDeviceScope);
+            acc[i][j] = there ? v4f{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)}
+                              : v4f{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
+          }
+      }
+    }
+    if (!took_over) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
 
-    for (int slab = 0; slab < nslab; ++slab) {
-      if (slab == 0 && stored) {
+    for (int slab = cur.s0; slab < cur.s1; ++slab) {
+      if (slab == cur.s0 && stored && !took_over) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTORE) : "memory");
       } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -746,14 +856,14 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
       asm volatile("" ::: "memory");
       const float bs = bs_nxt;
       if constexpr (BLOCKSCALE) {
-        if (slab + 1 < nslab) bs_nxt = bs_row[slab + 1];
+        if (slab + 1 < cur.s1) bs_nxt = bs_row[slab + 1];
       }
       asm volatile("" ::: "memory");
-      // the copy issued during this slab: the tile's next slab, or slab 0 of the next tile
-      const bool last = slab + 1 == nslab;
+      // the copy issued during this slab: the job's next slab, or the first slab of the next job
+      const bool last = slab + 1 == cur.s1;
       const uint32_t dead = (last && !has_next) ? 0x80000000u : 0u;
-      const TileAt dat = last ? next : cur;
-      const int dma_slab = last ? 0 : slab + 1, dma_buf = buf ^ 1;
+      const TileAt dat = last ? next_at : cur_at;
+      const int dma_slab = last ? nxt.s0 : slab + 1, dma_buf = buf ^ 1;
       constexpr int SPREAD = TM >= 4 ? TM / 2 : TM;
 
       const uint8_t* sa = smem + buf * STAGE_BYTES;
@@ -808,60 +918,83 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
       }
       buf ^= 1;
     }
-    // the first weight-block scale of the next tile travels while this one is stored
-    if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn2 * BN + wn * WN) / 128) * p.b_scales_ld];
+    // the first weight-block scale of the next job travels while this one is stored
+    if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn2 * BN + wn * WN) / 128) * p.b_scales_ld + nxt.s0];
 
-    // ---- the tile leaves, 16 rows of the wave's part at a time
-    // (row scaling: every scale of the tile is loaded before the first store, so that no later wait for a
-    // load also waits for the stores in front of it)
-    float b_s[TN / 2][8], a_s_all[TM];
-    if constexpr (!BLOCKSCALE) {
+    bool handed_on = false;
+    if constexpr (SPLIT) {
+      if (cur.kind == HEAD) {
+        // ---- the accumulators go to the successor's slot; the flag follows once every wave's stores have completed
+        handed_on = true;
+        uint32_t base = (uint32_t)(l + 1) * PARTIAL_BYTES + (uint32_t)wave * (PARTIAL_BYTES / NWAVES);
+        asm volatile("" : "+s"(base));
 #pragma unroll
-      for (int q = 0; q < TN / 2; ++q)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          b_s[q][i] = scale_at(p.b_scales, (int64_t)(tn * BN + wn * WN + q * 32 + lq * 8 + i) * p.b_scale_stride, p.scales_dtype);
-#pragma unroll
-      for (int mt = 0; mt < TM; ++mt)
-        a_s_all[mt] = scale_at(p.a_scales, ((int64_t)tm * BM + wm * WM + mt * 16 + lm) * p.a_scale_stride, p.scales_dtype);
-      asm volatile("" ::: "memory");
-    }
-    // (C goes out through a buffer descriptor: one 32-bit lane offset for all of a lane's stores, the rest scalar)
-    const uint32_t c_tile = ((uint32_t)(tm * BM + wm * WM) * (uint32_t)p.ldc + (uint32_t)(tn * BN + wn * WN)) * 2u;
-#pragma unroll
-    for (int mt = 0; mt < TM; ++mt) {
-      float a_s = 1.f;
-      if constexpr (!BLOCKSCALE) a_s = a_s_all[mt];
-#pragma unroll
-      for (int q = 0; q < TN / 2; ++q) {
-        v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
-        if constexpr (!BLOCKSCALE) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
-            lo[i] = t_lo * b_s[q][i];
-            hi[i] = t_hi * b_s[q][4 + i];
+          for (int j = 0; j < TN; ++j) {
+            const v4f a4 = acc[i][j];
+            const v4u v = {__float_as_uint(a4[0]), __float_as_uint(a4[1]), __float_as_uint(a4[2]), __float_as_uint(a4[3])};
+            buffer_store_b128_guarded<kDeviceScope>(v, w_rsrc, (uint32_t)lane * 16u, base + (uint32_t)(i * TN + j) * 1024u);
           }
-        }
-        *reinterpret_cast<uint4*>(wbuf + lm * (WN * 2) + (((q * 4 + lq) ^ (lm & 7)) * 16)) =
-            make_uint4(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3]));
-      }
-      // (a wave reads back only what it wrote itself, and its LDS operations execute in order)
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int r = i * 8 + rr;
-        typedef unsigned int v4u __attribute__((ext_vector_type(4)));
-        const v4u v = *reinterpret_cast<const v4u*>(wbuf + r * (WN * 2) + ((cc ^ (r & 7)) * 16));
-                // (non-temporal: C is not read again here, and its lines should not push the operands out of L2)
-        __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, c_lane, c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes, 2);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        if (tid == 0) __hip_atomic_store(flags + l + 1, p.streamk_seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        stored = false;
       }
     }
-    stored = true;
-    if (!has_next) break;
-    my = nxt;
+    if (!handed_on) {
+      // ---- the tile leaves, 16 rows of the wave's part at a time
+      // (row scaling: every scale of the tile is loaded before the first store, so that no later wait for a
+      // load also waits for the stores in front of it)
+      float b_s[TN / 2][8], a_s_all[TM];
+      if constexpr (!BLOCKSCALE) {
+#pragma unroll
+        for (int q = 0; q < TN / 2; ++q)
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            b_s[q][i] = scale_at(p.b_scales, (int64_t)(tn * BN + wn * WN + q * 32 + lq * 8 + i) * p.b_scale_stride, p.scales_dtype);
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt)
+          a_s_all[mt] = scale_at(p.a_scales, ((int64_t)tm * BM + wm * WM + mt * 16 + lm) * p.a_scale_stride, p.scales_dtype);
+        asm volatile("" ::: "memory");
+      }
+      // (C goes out through a buffer descriptor: one 32-bit lane offset for all of a lane's stores, the rest scalar)
+      const uint32_t c_tile = ((uint32_t)(tm * BM + wm * WM) * (uint32_t)p.ldc + (uint32_t)(tn * BN + wn * WN)) * 2u;
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        float a_s = 1.f;
+        if constexpr (!BLOCKSCALE) a_s = a_s_all[mt];
+#pragma unroll
+        for (int q = 0; q < TN / 2; ++q) {
+          v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
+          if constexpr (!BLOCKSCALE) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
+              lo[i] = t_lo * b_s[q][i];
+              hi[i] = t_hi * b_s[q][4 + i];
+            }
+          }
+          // (written and read back through the same vector type: to the compiler a store through one type and a load
+          // through another need not alias, and it may then move the load in front of the store)
+          *reinterpret_cast<v4u*>(wbuf + lm * (WN * 2) + (((q * 4 + lq) ^ (lm & 7)) * 16)) =
+              v4u{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
+        }
+        // (a wave reads back only what it wrote itself, and its LDS operations execute in order)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int r = i * 8 + rr;
+          const v4u v = *reinterpret_cast<const v4u*>(wbuf + r * (WN * 2) + ((cc ^ (r & 7)) * 16));
+          // (non-temporal: C is not read again here, and its lines should not push the operands out of L2)
+          buffer_store_b128_guarded<2>(v, c_rsrc, c_lane, c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes);
+        }
+      }
+      stored = true;
+    }
+    cur = nxt;
     tm = tm2;
     tn = tn2;
-    cur = next;
+    cur_at = next_at;
   }
   // the last copies (of nothing: every lane out of range) still write zeros into the stages: they
   // must have landed before the block's LDS goes to another block
@@ -871,7 +1004,13 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_persist_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  persist_body<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE>(p, smem);
+  persist_body<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE, false>(p, smem);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_streamk_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  persist_body<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE, true>(p, smem);
 }
 
 // ---- grouped (MoE) matmul ---------------------------------------------------------------------
@@ -1124,6 +1263,28 @@ static int launch_persist(const GemmArgs& p, hipStream_t stream, const char* nam
   return launch_with_lds(gemm_persist_kernel<256, 256, 2, 4, BLOCKSCALE>, attr_done, lds, 512, p, grid, stream, name);
 }
 
+// The work-split form: blocks = the CUs in whole rounds of the 8 XCDs; one workspace slot of 256 KB per block.
+static int streamk_blocks() {
+  const int g = (compute_units() / 8) * 8;
+  return g > kStreamkMaxBlocks ? kStreamkMaxBlocks : g;
+}
+static size_t streamk_workspace_bytes() { return (size_t)streamk_blocks() * 256 * 256 * 4; }
+
+template <bool BLOCKSCALE>
+static int launch_streamk(const GemmArgs& p_in, hipStream_t stream, const char* name) {
+  static PerDeviceFlag attr_done;
+  static std::atomic<unsigned int> seq{0};
+  constexpr int lds = tile_lds_bytes<256, 256, 2, BLOCKSCALE>() + 8 * 2048;
+  GemmArgs p = p_in;
+  // every launch gets a sequence number (never 0) as its flag value and one of 64 sets of flags: launches that
+  // follow each other on a stream may reuse a set at once, and 64 matmuls of this size are never in flight together
+  unsigned int n = seq.fetch_add(1, std::memory_order_relaxed) + 1;
+  if (n == 0) n = seq.fetch_add(1, std::memory_order_relaxed) + 1;
+  p.streamk_seq = n;
+  p.streamk_slot = (int)(n % kStreamkSlots);
+  return launch_with_lds(gemm_streamk_kernel<256, 256, 2, 4, BLOCKSCALE>, attr_done, lds, 512, p, dim3((unsigned)streamk_blocks()), stream, name);
+}
+
 // Sums the split-K partial results in split order (deterministic), applies the row / tensor
 // scales where the matmul has them, converts and stores.
 template <bool BLOCKSCALE>
@@ -1246,6 +1407,8 @@ static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can
   return best + 1;
 }
 
+static bool streamk_shape(int64_t M, int64_t N, size_t workspace_bytes);
+static bool streamk_planned(int64_t M, int64_t N, int64_t K, bool blockscale);
 size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   // the largest split count any shape could choose for this problem
   size_t worst = 0;
@@ -1256,7 +1419,13 @@ size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int sp = pick_splits(tiles, t.slots, nslab);
     if (sp > 1 && (size_t)sp > worst) worst = sp;
   }
-  return worst * (size_t)M * (size_t)N * 4;
+  const size_t split_k = worst * (size_t)M * (size_t)N * 4;
+  // the work-split persistent kernel: a slot per block for the accumulators a block hands to its successor, where the
+  // planner would use it given the memory (in either scale mode: this size does not know which one is coming)
+  size_t split_work = 0;
+  if (streamk_shape(M, N, ~(size_t)0) && (streamk_planned(M, N, K, true) || streamk_planned(M, N, K, false)))
+    split_work = streamk_workspace_bytes();
+  return split_k > split_work ? split_k : split_work;
 }
 
 // cost (microseconds) of an unsplit M x N region in tiles of shape t
@@ -1292,10 +1461,19 @@ static TwoRegionPlan pick_two_regions(int64_t M, int64_t N, int nslab, bool bloc
 }
 
 // What a tiled matmul will launch: one shape (possibly with K split), or two regions.
-struct TiledPlan { int variant; int splits; TwoRegionPlan two; };
+struct TiledPlan { int variant; int splits; TwoRegionPlan two; bool streamk; };
+
+// The work-split persistent kernel takes matmuls of whole 256 x 256 tiles that are at least one tile per block (so a
+// tile has at most two parts) and not a whole number of rounds (those have nothing to gain), when the caller's
+// workspace holds a 256 KB slot per block.
+static bool streamk_shape(int64_t M, int64_t N, size_t workspace_bytes) {
+  if (!tuning().streamk || !persist_shape(M, N, 1)) return false;
+  const int64_t tiles = (M / 256) * (N / 256), g = streamk_blocks();
+  return g >= 8 && tiles >= g && tiles % g != 0 && workspace_bytes >= streamk_workspace_bytes();
+}
 static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, size_t workspace_bytes,
                            int64_t batch, bool kv_on) {
-  TiledPlan plan = {0, 1, {0, 0, 0, 0, 0.f}};
+  TiledPlan plan = {0, 1, {0, 0, 0, 0, 0.f}, false};
   const int nslab = (int)ceil_div(K, 128);
   plan.variant = tile_override();
   const bool free_choice = plan.variant == 0;
@@ -1309,13 +1487,34 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
   }
   if (free_choice && batch == 1 && !kv_on && plan.splits == 1 && !tuning().one_region)
     plan.two = pick_two_regions(M, N, nslab, blockscale, region_cost(M, N, nslab, t, blockscale));
+  // Every block the same number of slabs instead of whole rounds of tiles.  Measured (block scaling, 300 to 900 tiles,
+  // K = 384 ... 16384): 23 microseconds (the hand-over: one drain of the pipeline, 256 KB each way per block) plus
+  // 1.9 per slab -- a sixth more per slab than the persistent kernel, whose blocks of an XCD walk K in step and
+  // find each other's operands in L2, while here neighbouring blocks sit at different K offsets.  So the split only
+  // pays where whole rounds would leave most of the last round empty and K is long (300 tiles, K = 4096: 87 against
+  // 107 microseconds; 448 tiles, K = 16384: 437 against 427): it has to beat the other plan by a tenth.
+  if (has_workspace && batch == 1 && !kv_on && plan.splits == 1 && (free_choice || plan.variant == 1) &&
+      streamk_shape(M, N, workspace_bytes)) {
+    const float tiles = (float)((M / 256) * (N / 256)), g = (float)streamk_blocks();
+    const float per_slab = 1.9f * (blockscale ? 1.0f : kShapes[0].t_slab_row / kShapes[0].t_slab_block);
+    const float cost = 23.0f + tiles / g * (float)nslab * per_slab;
+    const float other = plan.two.axis ? plan.two.cost : region_cost(M, N, nslab, t, blockscale);
+    plan.streamk = tuning().streamk == 2 || cost < 0.9f * other;
+  }
   return plan;
+}
+
+static TiledPlan cached_plan(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, size_t workspace_bytes, int64_t batch, bool kv_on);
+static bool streamk_planned(int64_t M, int64_t N, int64_t K, bool blockscale) {
+  return cached_plan(M, N, K, blockscale, true, ~(size_t)0, 1, false).streamk;
 }
 
 // The split-K scratch of the plan an unlimited workspace gets (0: that plan does not split).  A workspace of this size --
 // or of gemm_tiled_workspace_bytes, which is never smaller -- leads to this same plan.
 size_t gemm_tiled_plan_workspace_bytes(int64_t M, int64_t N, int64_t K, bool blockscale) {
   const TiledPlan plan = make_plan(M, N, K, blockscale, true, ~(size_t)0, 1, false);
+  // (a plan that splits the work between blocks instead has splits == 1: without the 64 MB of slots it needs, the
+  // planner falls back to the persistent kernel, which forms the same sums)
   return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)N * 4 : 0;
 }
 
@@ -1347,7 +1546,7 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
   auto count = [](int64_t m, int64_t n, const TileShape& t) { return (long long)(ceil_div(m, t.bm) * ceil_div(n, t.bn)); };
   // (what a bf16 result with 16-byte aligned rows gets)
   auto how = [](int64_t m, int64_t n, int variant) { return persist_shape(m, n, variant) ? " persistent" : (variant == 4 ? " three-stage" : ""); };
-  if (plan.two.axis) {
+  if (plan.two.axis && !plan.streamk) {
     const TileShape &a = kShapes[plan.two.v1 - 1], &b = kShapes[plan.two.v2 - 1];
     const bool cols = plan.two.axis == 1;
     const int64_t m1 = cols ? M : plan.two.cut, n1 = cols ? plan.two.cut : N;
@@ -1356,6 +1555,8 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
                     cols ? "columns" : "rows", (long long)plan.two.cut, b.bm, b.bn, count(m2, n2, b), how(m2, n2, plan.two.v2));
   }
   const TileShape& t = kShapes[plan.variant - 1];
+  if (plan.streamk)
+    return snprintf(buf, len, "256x256 x%lld persistent, stream-K: equal shares of slabs for %d blocks", count(M, N, kShapes[0]), streamk_blocks());
   if (plan.splits > 1) return snprintf(buf, len, "%dx%d x%lld, K split %d", t.bm, t.bn, count(M, N, t), plan.splits);
   return snprintf(buf, len, "%dx%d x%lld%s", t.bm, t.bn, count(M, N, t), how(M, N, plan.variant));
 }
@@ -1363,6 +1564,12 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
 int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, int64_t batch, hipStream_t stream) {
   GemmArgs p = p_in;
   const TiledPlan plan = cached_plan(p.M, p.N, p.K, blockscale, p.workspace != nullptr, workspace_bytes, batch, p.kv_on != 0);
+  if (plan.streamk) {
+    p.splits = 1;
+    // (the plan knows the shape; whether this call's pointers and strides suit the persistent kernels is checked here)
+    if (persist_ok(p, blockscale, dim3(1, 1, 1)))
+      return blockscale ? launch_streamk<true>(p, stream, "gemm_streamk_block_256x256") : launch_streamk<false>(p, stream, "gemm_streamk_row_256x256");
+  }
   if (plan.two.axis) {
     const TwoRegionPlan& two = plan.two;
     GemmArgs r1 = p, r2 = p;

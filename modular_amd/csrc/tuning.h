@@ -7,7 +7,8 @@
 //   MAXFP8_SPLITK=n            force the K split of the tiled matmul
 //   MAXFP8_ONE_REGION=1        never cut a matmul into two regions
 //   MAXFP8_PERSIST=0           per-tile kernels instead of the persistent one
-//   MAXFP8_STREAMK=0           no (tile, slab range) work units for matmuls of few tiles
+//   MAXFP8_STREAMK=0 / 2       never / always split the work of whole-tile matmuls evenly over the blocks
+//                              (default 1: where the cost model says it pays)
 //   MAXFP8_BIG_ROWS=n          grouped: slots with at least n rows use the large-tile launch (1024)
 //   MAXFP8_GROUPED_OVERLAP=0   grouped: the two launches in line on the caller's stream
 //   MAXFP8_GROUPED_SHARE=x     grouped: scales the share estimate of the large-tile launch (0.5)
@@ -21,7 +22,7 @@ struct Tuning {
   int splitk = 0;
   bool one_region = false;
   bool persist = true;
-  bool streamk = true;
+  int streamk = 1;
   int big_rows = 1024;
   bool grouped_overlap = true;
   float grouped_share = 0.5f;

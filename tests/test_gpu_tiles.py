@@ -173,7 +173,10 @@ def test_grouped_small_tiles_exact(dev):
     (28600, 4096, 2040, "row"),
     (2048, 4096, 28672, "row"),
 ])
-def test_two_region_launch(dev, M, K, N, kind):
+def test_two_region_launch(dev, tune, M, K, N, kind):
+    # (with a workspace, shapes of whole 256 x 256 tiles now split their work between the blocks instead: that path
+    # has its own tests below; here it is switched off so that the cut is what runs)
+    tune(MAXFP8_STREAMK="0")
     assert " + " in _lib.matmul_describe(M, N, K, kind == "block"), "this shape is meant to run as two launches"
     cfg = BLK if kind == "block" else ROW
     x = synth.activations(M, K, seed=0, outlier_frac=0.0 if kind == "row" else 0.01, device=dev)
@@ -251,6 +254,81 @@ def test_persistent_kernel_many_tiles_per_block_repeated(dev, tune):
         a = synth.random_fp8((M, K), 100 + seed).to(dev)
         tune(MAXFP8_PERSIST="1")
         got = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
+        tune(MAXFP8_PERSIST="0")
+        want = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"launch {seed}"
+
+
+# ---- the persistent kernel with its work split along K ("stream-K") --------------------------------------------
+# Matmuls of at least one 256 x 256 tile per block whose tiles are not whole rounds of the chip: every block takes the
+# same number of slabs, and a tile that a block boundary cuts is begun by one block and finished by the next, its f32
+# accumulators handed over through the workspace.  The sums keep the per-tile kernel's order: bit-equal results.
+STREAMK_SHAPES = [(2560, 7680, 384), (4096, 7168, 2048), (5120, 5120, 640), (2048, 28672, 512), (4096, 7168, 16384)]
+
+
+@pytest.mark.parametrize("M,N,K", STREAMK_SHAPES)
+@pytest.mark.parametrize("kind", ["block", "row"])
+def test_stream_k_equals_per_tile_kernel(dev, tune, M, N, K, kind):
+    if kind == "row" and K > 4096:
+        pytest.skip("one long-K case is enough")
+    tune(MAXFP8_TILE="1", MAXFP8_STREAMK="2")     # 2: wherever the shape allows it, whatever the cost model says
+    assert "stream-K" in _lib.matmul_describe(M, N, K, kind == "block", True)
+    assert "stream-K" not in _lib.matmul_describe(M, N, K, kind == "block", False)   # no workspace, no hand-over
+    if kind == "block":
+        a, b, sa, sb = make_block(M, N, K, seed=M + K)
+        cfg = BLK
+    else:
+        a, b = synth.random_fp8((M, K), M), synth.random_fp8((N, K), N + 1)
+        sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+        cfg = ROW
+    ad, bd, sad, sbd = a.to(dev), b.to(dev), sa.to(dev), sb.to(dev)
+    run = lambda: mx.dynamic_scaled_matmul(ad, bd, sad, sbd, cfg.input_scale, cfg.weight_scale, out_type=torch.bfloat16,
+                                           algo="tiled")
+    got = run()
+    tune(MAXFP8_STREAMK="0")
+    assert "stream-K" not in _lib.matmul_describe(M, N, K, kind == "block", True)
+    persistent = run()
+    tune(MAXFP8_PERSIST="0")
+    per_tile = run()
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(got.float()).all())
+    assert torch.equal(got.view(torch.int16), per_tile.view(torch.int16))
+    assert torch.equal(persistent.view(torch.int16), per_tile.view(torch.int16))
+
+
+def test_stream_k_exact(dev, tune):
+    tune(MAXFP8_TILE="1", MAXFP8_STREAMK="2")
+    M, N, K = 2560, 7680, 640
+    a, b, sa, sb, want = exact_case(M, N, K, seed=M + N + K)
+    assert "stream-K" in _lib.matmul_describe(M, N, K, True, True)
+    cb = mm(a, b, sa, sb, BLK, dev, out=torch.bfloat16, algo="tiled")
+    assert torch.equal(cb.cpu(), torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16))
+
+
+def test_stream_k_repeated_launches_with_fresh_data(dev, tune):
+    """The hand-over goes through memory that other CUs (and other XCDs, whose L2 caches are not coherent with each
+    other) wrote: thirty launches in a row, each with new activations and a new workspace position, each compared with
+    the per-tile kernel.  A block that read a stale partial sum or an old flag would show here."""
+    tune(MAXFP8_TILE="1", MAXFP8_STREAMK="2")
+    M, N, K = 2560, 7680, 1024
+    b = synth.random_fp8((N, K), 77).to(dev)
+    sb = synth.random_scales((N // 128, K // 128), 78).to(dev)
+    sa = synth.random_scales((K // 128, M), 79).to(dev)
+    L = _lib.lib()
+    need = L.maxfp8_matmul_workspace_bytes(M, N, K)
+    assert need == 64 << 20
+    ws = torch.zeros((need + 4096,), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    for seed in range(30):
+        a = synth.random_fp8((M, K), 100 + seed).to(dev)
+        got = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        off = 256 * (seed % 3)      # the same slots again, and slots shifted against the last launch's
+        tune(MAXFP8_TILE="1", MAXFP8_STREAMK="2", MAXFP8_PERSIST="1")
+        st = L.maxfp8_matmul_dynamic_scaled_fp8(got.data_ptr(), a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), M, N, K,
+                                                K, K, N, _lib.GRAN_BLOCK, _lib.GRAN_BLOCK, 1, 128, 128, M, K // 128, _lib.BF16,
+                                                _lib.F32, _lib.ALGO_TILED, ws.data_ptr() + off, need, stream)
+        assert st == 0, _lib.last_error()
         tune(MAXFP8_PERSIST="0")
         want = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
         torch.cuda.synchronize()
