@@ -238,6 +238,35 @@ def run_gpu(name, steps, warmup, settle_s=None):
     return wl, ms_step, mm_avg, mm_ms[len(mm_ms) // 2], mm_ms[0]
 
 
+def read_ceiling(wl, steps):
+    """Average time of the decode matmul's read-only probe (the same grid, LDS ring and DMA instructions streaming
+    the same weight copies, nothing else) over `steps` back-to-back launches, in milliseconds."""
+    import torch
+    from modular_amd import _lib
+
+    L, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
+
+    def launch(i):
+        w = wl.w[i % wl.copies]
+        _lib.check(L.maxfp8_decode_weight_read_probe(w.data_ptr(), wl.M, wl.N, wl.K, w.stride(0), stream))
+
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_end, i = time.perf_counter() + 0.3, 0
+    while time.perf_counter() < t_end:
+        for _ in range(64):
+            launch(i)
+            i += 1
+        torch.cuda.synchronize()
+    for i in range(200):
+        launch(i)
+    first.record()
+    for i in range(steps):
+        launch(i)
+    last.record()
+    torch.cuda.synchronize()
+    return first.elapsed_time(last) / steps
+
+
 def cpu_baseline(wl, budget_s=15.0):
     """The oracle (a port of the reference's host loops) on this host's cores, on a bounded
     slice of the same workload; throughput in the metric's unit."""
@@ -383,6 +412,9 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB three times (the known-size unit that "
                          "hardware byte counters of a rocprofv3 --pmc run are scaled by)")
+    ap.add_argument("--read-ceiling", action="store_true",
+                    help="for every decode workload (M <= 16): the matmul kernel's time beside the time of its read-only "
+                         "probe (same grid and weight traffic, no arithmetic), one JSON line each")
     args = ap.parse_args()
     SETTLE_S = max(0.0, args.settle)
     if args.gpus != 1:
@@ -406,6 +438,19 @@ def main():
                   file=sys.stderr, flush=True)
             with open(os.path.join(ROOT, RESULTS_DIR, "bench_table.json"), "w") as f:
                 json.dump(rows, f, indent=1)
+            torch.cuda.empty_cache()
+        return
+    if args.read_ceiling:
+        for name in ([args.workload] if args.workload else [n for n, w in WORKLOADS.items() if w[0] == "row" and w[1] <= 16]):
+            wl, _, mm_avg, _, _ = run_gpu(name, max(args.steps, 200), args.warmup)
+            probe = read_ceiling(wl, max(args.steps, 200))
+            _, mm_bytes, _ = algorithmic(wl.kind, wl.M, wl.K, wl.N)
+            print(json.dumps({"workload": name, "M": wl.M, "K": wl.K, "N": wl.N, "weight_bytes": wl.N * wl.K,
+                              "matmul_us": round(mm_avg * 1e3, 2), "read_only_us": round(probe * 1e3, 2),
+                              "matmul_over_read_only": round(mm_avg / probe, 3),
+                              "matmul_GBps": round(mm_bytes / mm_avg / 1e6), "read_only_GBps": round(wl.N * wl.K / probe / 1e6)}),
+                  flush=True)
+            del wl
             torch.cuda.empty_cache()
         return
     if args.calibrate:

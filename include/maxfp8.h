@@ -453,6 +453,14 @@ int maxfp8_cast_e4m3fn_to_f32(float* out, const void* in_fp8, int64_t n, void* s
  * hardware byte counters. */
 int maxfp8_copy_bytes(void* dst, const void* src, int64_t n, void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: streams the weight matrix b[N, K] (row stride ldb bytes)
+ * through the decode (M <= 16) matmul's own grid, LDS ring and DMA instructions -- the shape MAXFP8_ALGO_AUTO
+ * would pick for (M, N, K) with row scaling -- and does nothing else: no activations, no MFMA, no stores.  Its
+ * time is the ceiling the weight-streaming matmul is measured against.
+ */
+int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t K, int64_t ldb, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

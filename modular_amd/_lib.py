@@ -46,6 +46,7 @@ EXPORTS = (
     "maxfp8_cast_e4m3fn_to_f32",
     "maxfp8_cast_f32_to_bf16",
     "maxfp8_copy_bytes",
+    "maxfp8_decode_weight_read_probe",
 )
 
 _lib = None
@@ -117,6 +118,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_cast_e4m3fn_to_f32.argtypes = [vp, vp, i64, vp]
     L.maxfp8_copy_bytes.restype = ci
     L.maxfp8_copy_bytes.argtypes = [vp, vp, i64, vp]
+    L.maxfp8_decode_weight_read_probe.restype = ci
+    L.maxfp8_decode_weight_read_probe.argtypes = [vp, i64, i64, i64, i64, vp]
     _lib = L
     return L
 

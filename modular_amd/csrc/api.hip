@@ -56,6 +56,7 @@ int gemm_grouped_dispatch(const GemmArgs&, bool, int64_t, int64_t, hipStream_t);
 int gemm_skinny_dispatch(const GemmArgs&, bool, int64_t, hipStream_t);
 int gemm_skinny_max_m();
 bool gemm_skinny_preferred(int64_t M, int64_t N, int64_t K);
+int gemm_skinny_read_probe(const void* b, int64_t M, int64_t N, int64_t K, int64_t ldb, hipStream_t stream);
 
 // v rounded to bf16 / f16 and widened back: how an op parameter of the input's dtype arrives
 static float round_to_dtype(float v, int dtype) {
@@ -715,6 +716,16 @@ int maxfp8_copy_bytes(void* dst, const void* src, int64_t n, void* stream) {
   if (n % 16 != 0 || !is_aligned(dst, 16) || !is_aligned(src, 16))
     MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "copy: size and pointers must be multiples of 16 bytes");
   return copy_bytes_dispatch(dst, src, n, (hipStream_t)stream);
+}
+
+int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t K, int64_t ldb, void* stream) {
+  if (!b) MAXFP8_FAIL(MAXFP8_ERR_NULL, "read probe: null pointer");
+  if (M <= 0 || M > 16 || N <= 0 || K <= 0 || ldb < K)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "read probe: needs 1 <= M <= 16, N > 0, 0 < K <= ldb (got M %lld, N %lld, K %lld, ldb %lld)",
+                (long long)M, (long long)N, (long long)K, (long long)ldb);
+  if (!is_aligned(b, 16) || K % 16 != 0 || ldb % 16 != 0) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "read probe: needs 16-byte aligned rows and K %% 16 == 0");
+  if (!offsets_fit(K, ldb, ldb, 0, false)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "read probe: rows too long for 32-bit tile offsets");
+  return gemm_skinny_read_probe(b, M, N, K, ldb, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -345,6 +345,95 @@ static int pick_ntw(const GemmArgs& p, int64_t batch, hipStream_t stream) {
   }
 }
 
+// ---- read-only probe ---------------------------------------------------------------------------
+// The weight traffic of gemm_skinny_kernel and nothing else: same grid, block size, rows per block, split of K over
+// the waves, LDS ring, ring depth, DMA instructions and wait counts as the matmul of an M <= 16 row-scaled problem, but
+// no activations, no MFMA, no reduction and no stores (one dword per slab is read back from LDS so that the ring is
+// consumed in order).  Its time is what this access pattern can reach on the memory system: the matmul is measured
+// against it.
+template <int NTW, int RING_KB, int NWAVES>
+__global__ __launch_bounds__(NWAVES * 64) void skinny_read_probe_kernel(const uint8_t* b, int N, int K, int64_t ldb, uint32_t* sink) {
+  using Cfg = SkinnyCfg<NTW, 1, false, RING_KB, NWAVES>;
+  constexpr int WAVES = Cfg::WAVES, DEPTH = Cfg::DEPTH, SLOT = Cfg::SLOT, PER = 2 * NTW;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = blockIdx.x * (16 * NTW);
+  const int cols_here = (N - n0) < 16 * NTW ? (N - n0) : 16 * NTW;
+  const __amdgpu_buffer_rsrc_t b_rsrc = sk_rsrc(b + (int64_t)n0 * ldb, sk_clamp_u32((int64_t)(cols_here - 1) * ldb + K));
+  const int nslab = (K + 127) / 128;
+  const int per_wave = (nslab + WAVES - 1) / WAVES;
+  const int s_begin = wave * per_wave;
+  const int s_end = (s_begin + per_wave) < nslab ? (s_begin + per_wave) : nslab;
+  const int cr = lane >> 3, cp = lane & 7;
+  const uint32_t w_voff = (uint32_t)cr * (uint32_t)ldb + (cp ^ cr) * 16;
+  const uint32_t w_half = 8u * (uint32_t)ldb, w_tile = 16u * (uint32_t)ldb;
+  uint8_t* ring = smem + wave * Cfg::RING;
+  uint32_t seen = 0;
+  auto issue = [&](int slab, auto d_c) {
+    constexpr int d = decltype(d_c)::value;
+    const bool live = slab < s_end;
+    const uint32_t koff = (uint32_t)(live ? slab : s_begin) * 128u;
+    const uint32_t killw = live ? 0u : 0x80000000u;
+    uint8_t* slot = ring + d * SLOT;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (sk_lds_ptr_t)(slot + t * 2048), 16, w_voff | killw, koff + t * w_tile, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (sk_lds_ptr_t)(slot + t * 2048 + 1024), 16, w_voff | killw, koff + t * w_tile + w_half, 0, 0);
+    }
+  };
+  auto consume = [&](auto d_c) {
+    constexpr int d = decltype(d_c)::value;
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * PER) : "memory");
+    seen ^= *reinterpret_cast<const uint32_t*>(ring + d * SLOT + lane * 4);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
+  auto for_each_slot = [&](auto&& f) {
+    [&]<int... D>(std::integer_sequence<int, D...>) { (f(std::integral_constant<int, D>{}), ...); }
+    (std::make_integer_sequence<int, DEPTH>{});
+  };
+  for_each_slot([&](auto d_c) { issue(s_begin + decltype(d_c)::value, d_c); });
+  for (int base = s_begin; base < s_end; base += DEPTH) {
+    for_each_slot([&](auto d_c) {
+      constexpr int d = decltype(d_c)::value;
+      consume(d_c);
+      issue(base + DEPTH + d, d_c);
+    });
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // (never true for the data the benchmark streams; keeps the reads alive)
+  if (seen == 0x9e3779b9u && sink) sink[0] = seen;
+}
+
+template <int NTW, int RING_KB, int NWAVES>
+static int launch_read_probe(const void* b, int64_t N, int64_t K, int64_t ldb, hipStream_t stream) {
+  using Cfg = SkinnyCfg<NTW, 1, false, RING_KB, NWAVES>;
+  auto kern = skinny_read_probe_kernel<NTW, RING_KB, NWAVES>;
+  static PerDeviceFlag attr;
+  bool& attr_done = attr.here();
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM);
+    if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "read probe: cannot reserve %d bytes of LDS: %s", Cfg::SMEM, hipGetErrorString(e));
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(N, 16 * NTW)), dim3(NWAVES * 64), Cfg::SMEM, stream, (const uint8_t*)b, (int)N, (int)K,
+                     ldb, (uint32_t*)nullptr);
+  return launch_status("skinny_read_probe");
+}
+
+int gemm_skinny_read_probe(const void* b, int64_t M, int64_t N, int64_t K, int64_t ldb, hipStream_t stream) {
+  int sel = tuning().skinny;
+  if (!sel) sel = skinny_shape(M, N, K);
+  switch (sel) {
+    case 1408: return launch_read_probe<1, 8, 4>(b, N, K, ldb, stream);
+    case 1416: return launch_read_probe<1, 16, 4>(b, N, K, ldb, stream);
+    case 2416: return launch_read_probe<2, 16, 4>(b, N, K, ldb, stream);
+    case 2408: return launch_read_probe<2, 8, 4>(b, N, K, ldb, stream);
+    case 4432: return launch_read_probe<4, 32, 4>(b, N, K, ldb, stream);
+    default: MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "read probe: unknown shape selector %d", sel);
+  }
+}
+
 int gemm_skinny_max_m() { return 64; }
 
 // What MAXFP8_ALGO_AUTO gives the weight-streaming kernel: every matmul of at most 32 rows (but see below), and those
