@@ -330,8 +330,12 @@ def kernels_launched(kind, M, K, N):
     if kind == "rmsq":
         return "rmsnorm_quant_row_bf16_kernel", "one launch"
     if kind == "grouped":
-        return "gemm_grouped_kernel", ("gemm_grouped_large_kernel (full 256-row tiles of experts with >= 1024 rows) + "
-                                       "gemm_grouped_kernel (the rest), side by side on two streams")
+        if os.environ.get("MAXFP8_GROUPED_PERSIST", "1") == "0":
+            return "gemm_grouped_kernel", ("gemm_grouped_large_kernel (full 256-row tiles of experts with >= 1024 rows) + "
+                                           "gemm_grouped_kernel (the rest), side by side on two streams")
+        return "gemm_grouped_persist_kernel", ("one persistent launch, a block per CU: 256 x 256 tiles of every full 256 rows, "
+                                               "256 x 128 / 128 x 256 tiles of the rests, weight-streaming rings for rests of at "
+                                               "most 32 rows; the CUs are shared out between the matrix-bound and the streaming tiles")
     from modular_amd import _lib
     plan = _lib.matmul_describe(M, N, K, kind == "block", True)
     first = plan.split(" + ")[0]

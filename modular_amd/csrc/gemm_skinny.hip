@@ -132,7 +132,10 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
     constexpr int d = decltype(d_c)::value;
     const bool live = slab < s_end;
     const int sl = live ? slab : s_begin;
-    const uint32_t koff = (uint32_t)sl * 128u;
+    // (wave-uniform by construction; said so explicitly, or the loads' scalar offsets end up in vector registers
+    // and every load in a loop over the lanes' values)
+    const uint32_t koff = __builtin_amdgcn_readfirstlane((uint32_t)sl * 128u);
+    const uint32_t koff_hi = __builtin_amdgcn_readfirstlane(koff + 64u);
     uint32_t kill0 = live ? 0u : 0x80000000u, kill1 = kill0, killw = kill0;
     if (k_tail) {
       if (koff + lq * 16 >= (uint32_t)p.K) kill0 = 0x80000000u;
@@ -142,7 +145,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       const v4i lo = sk_load16(a_rsrc, a_off[t] | kill0, koff);
-      const v4i hi = sk_load16(a_rsrc, a_off[t] | kill1, koff + 64);
+      const v4i hi = sk_load16(a_rsrc, a_off[t] | kill1, koff_hi);
       af[d][t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
     if constexpr (BLOCKSCALE) {

@@ -1181,6 +1181,340 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_k
   }
 }
 
+// ---- grouped matmul as one persistent launch ---------------------------------------------------
+// One block of 8 waves per CU takes tiles of four kinds from four counters in device memory until all are gone:
+//   L   every full 256-row tile of a slot with at least big_rows rows           256 x 256, 2 stages (matrix-pipe bound)
+//   M2  a rest of 129 ... 255 rows                                               256 x 128, 3 stages
+//   M1  a rest of small_rows + 1 ... 128 rows                                    128 x 256, 3 stages
+//   S   a rest of at most small_rows (<= 32) rows                                512 weight rows streamed through eight
+//       rings of 16 KB, one per wave, 64 rows each (HBM bound: 128 KB in flight per CU, no barrier)
+// A CU holds one kind at a time -- the L and M tiles fill its registers and LDS, the S rings its LDS -- so the chip is
+// shared out by CUs: the first blocks start with the S tiles and go on to M1, M2 and L when none are left, the others
+// take L, M2, M1, S.  How many start with S follows from the device-resident group sizes and the per-tile times below;
+// whichever kind runs out first, its blocks move on, so the estimate only has to be roughly right.  While both are busy
+// the S blocks stream weights at the rate their rings allow and the other CUs keep the matrix pipes busy, instead of
+// the two kinds taking turns on the whole chip.
+//
+// Every block builds the same four prefix tables over the slots in LDS (row tiles of each kind before slot z); a
+// claimed index is a (row tile, column tile) pair, column tiles fastest, found by bisection.  No list of tiles in
+// memory, no host synchronisation.  The result of a tile does not depend on which block computes it.
+constexpr int kGroupedCtrSlots = 64;
+constexpr int kGroupedMaxSlots = 512;   // slots (active experts) the LDS tables hold
+static __device__ unsigned int g_grouped_ctr[kGroupedCtrSlots * 32];  // per launch in flight: kind x XCD
+
+__global__ void grouped_ctr_zero_kernel(int slot) {
+  if (threadIdx.x < 32) g_grouped_ctr[slot * 32 + threadIdx.x] = 0u;
+}
+
+// One wave: C[rows of the slot, 16 * NTW weight rows from n0 + 16 * NTW * wave] over the whole of K.  The weight slabs
+// (16 * NTW rows x 128 bytes) travel by LDS-DMA through the wave's own ring of DEPTH slots, the activations (at most
+// 16 * MT rows, read by every wave of the chip that works on this slot: L1 / L2 hits) and the scales straight to
+// registers; wait counts are exact because every slot always carries PER instructions (slabs past the end are issued
+// out of range).
+template <int MT, int NTW, int DEPTH, bool BLOCKSCALE>
+__device__ __forceinline__ void grouped_stream_body(const GemmArgs& p, uint8_t* smem, const int64_t row_begin, const int rows_here,
+                                                    const int n0, const uint8_t* bptr, const float* bs_ptr) {
+  constexpr int SLOT = NTW * 2048, PER = 2 * MT + (BLOCKSCALE ? MT + 1 : 0) + 2 * NTW;
+  static_assert((DEPTH - 1) * PER < 64, "vmcnt is a 6-bit counter");
+  static_assert(!BLOCKSCALE || 128 % (16 * NTW) == 0, "a wave's weight rows must sit inside one 128-row scale block");
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lm = lane & 15, lq = lane >> 4;
+  const int nw = n0 + wave * (16 * NTW);
+  if (nw >= p.N) return;  // (wave-uniform; the body has no barrier)
+  const int wrows = (p.N - nw) < 16 * NTW ? (p.N - nw) : 16 * NTW;
+  const __amdgpu_buffer_rsrc_t b_rsrc = t2_rsrc(bptr + (int64_t)nw * p.ldb, t2_clamp_u32((int64_t)(wrows - 1) * p.ldb + p.K));
+  const __amdgpu_buffer_rsrc_t a_rsrc = t2_rsrc(p.a + row_begin * p.lda, t2_clamp_u32((int64_t)(rows_here - 1) * p.lda + p.K));
+  const int nslab = (p.K + 127) / 128;
+  const bool k_tail = (p.K & 127) != 0;
+  const int cr = lane >> 3, cp = lane & 7;
+  const int cchunk = cp ^ cr;
+  const uint32_t w_voff = (uint32_t)cr * (uint32_t)p.ldb + cchunk * 16;
+  const uint32_t w_half = 8u * (uint32_t)p.ldb, w_tile = 16u * (uint32_t)p.ldb;
+  uint32_t a_off[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) a_off[t] = (uint32_t)(t * 16 + lm) * (uint32_t)p.lda + lq * 16;
+  const uint32_t frag0 = lm * 128 + ((lq ^ (lm & 7)) << 4);
+  const uint32_t frag1 = lm * 128 + (((lq + 4) ^ (lm & 7)) << 4);
+  uint8_t* ring = smem + wave * (DEPTH * SLOT);
+
+  __amdgpu_buffer_rsrc_t as_rsrc = t2_rsrc(nullptr, 0), bs_rsrc = t2_rsrc(nullptr, 0);
+  uint32_t as_voff[MT];
+  if constexpr (BLOCKSCALE) {
+    as_rsrc = t2_rsrc(p.a_scales + row_begin, t2_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + rows_here) * 4));
+    bs_rsrc = t2_rsrc(bs_ptr + (int64_t)(nw / 128) * p.b_scales_ld, (uint32_t)nslab * 4u);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = t * 16 + lm;
+      as_voff[t] = (uint32_t)(m < rows_here ? m : rows_here - 1) * 4u;
+    }
+  }
+  v4f acc[MT][NTW];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NTW; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+  v8i af[DEPTH][MT];
+  float as_v[DEPTH][MT], bs_v[DEPTH];
+
+  auto load16 = [&](__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+  };
+  auto issue = [&](int slab, auto d_c) {
+    constexpr int d = decltype(d_c)::value;
+    const bool live = slab < nslab;
+    const int sl = live ? slab : 0;
+    // (wave-uniform by construction; said so explicitly, or the loads' scalar offsets end up in vector registers
+    // and every load in a loop over the lanes' values)
+    const uint32_t koff = __builtin_amdgcn_readfirstlane((uint32_t)sl * 128u);
+    const uint32_t koff_hi = __builtin_amdgcn_readfirstlane(koff + 64u);
+    uint32_t kill0 = live ? 0u : 0x80000000u, kill1 = kill0, killw = kill0;
+    if (k_tail) {
+      if (koff + lq * 16 >= (uint32_t)p.K) kill0 = 0x80000000u;
+      if (koff + 64 + lq * 16 >= (uint32_t)p.K) kill1 = 0x80000000u;
+      if (koff + cchunk * 16 >= (uint32_t)p.K) killw = 0x80000000u;
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const v4i lo = load16(a_rsrc, a_off[t] | kill0, koff);
+      const v4i hi = load16(a_rsrc, a_off[t] | kill1, koff_hi);
+      af[d][t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+    if constexpr (BLOCKSCALE) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        as_v[d][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(as_rsrc, as_voff[t], (uint32_t)sl * (uint32_t)p.a_scales_ld * 4u, 0));
+      bs_v[d] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bs_rsrc, 0, (uint32_t)sl * 4u, 0));
+    }
+    uint8_t* slot = ring + d * SLOT;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(slot + t * 2048), 16, w_voff | killw, koff + t * w_tile, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(slot + t * 2048 + 1024), 16, w_voff | killw, koff + t * w_tile + w_half, 0, 0);
+    }
+  };
+  auto compute = [&](auto d_c) {
+    constexpr int d = decltype(d_c)::value;
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * PER) : "memory");
+    const uint8_t* slot = ring + d * SLOT;
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt) {
+      const v4i lo = *reinterpret_cast<const v4i*>(slot + nt * 2048 + frag0);
+      const v4i hi = *reinterpret_cast<const v4i*>(slot + nt * 2048 + frag1);
+      const v8i wf = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if constexpr (BLOCKSCALE) {
+          const v4f zero = {0.f, 0.f, 0.f, 0.f};
+          const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af[d][mt], zero, 0, 0, 0, 0, 0, 0);
+          acc[mt][nt] += part * (as_v[d][mt] * bs_v[d]);
+        } else {
+          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af[d][mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
+        }
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the fragments have left LDS before the slot is refilled
+  };
+  static_for<DEPTH>([&](auto d_c) { issue(decltype(d_c)::value, d_c); });
+  for (int base = 0; base < nslab; base += DEPTH) {
+    static_for<DEPTH>([&](auto d_c) {
+      compute(d_c);
+      issue(base + DEPTH + decltype(d_c)::value, d_c);
+    });
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last issues were out of range, but they still target the ring
+
+  // lane (lm, lq) holds rows 4 * lq .. + 3 of a 16-row weight group for token lm: four consecutive columns of C
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int ml = mt * 16 + lm;
+    if (ml >= rows_here) continue;
+    const int64_t m = row_begin + ml;
+    const int64_t cm = p.c_row_index ? (int64_t)p.c_row_index[m] : m;
+    float a_s = 1.f;
+    if constexpr (!BLOCKSCALE) a_s = scale_at(p.a_scales, m * p.a_scale_stride, p.scales_dtype);
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt) {
+      const int n = nw + nt * 16 + lq * 4;
+      if (n >= p.N) continue;
+      float v[4] = {acc[mt][nt][0], acc[mt][nt][1], acc[mt][nt][2], acc[mt][nt][3]};
+      if constexpr (!BLOCKSCALE) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int nn = (n + i < p.N) ? n + i : p.N - 1;
+          const float t = v[i] * a_s;
+          v[i] = t * scale_at(bs_ptr, (int64_t)nn * p.b_scale_stride, p.scales_dtype);
+        }
+      }
+      if (p.c_dtype == MAXFP8_BF16) {
+        uint16_t* dst = reinterpret_cast<uint16_t*>(p.c) + cm * p.ldc + n;
+        if (p.c_vec_ok && n + 3 < p.N) {
+          *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < p.N) dst[i] = (uint16_t)f32_to_bf16_bits(v[i]);
+        }
+      } else {
+        float* dst = reinterpret_cast<float*>(p.c) + cm * p.ldc + n;
+        if (p.c_vec_ok && n + 3 < p.N) {
+          *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < p.N) dst[i] = v[i];
+        }
+      }
+    }
+  }
+}
+
+// LDS of the persistent grouped kernel: the largest tile body (256 x 128, 3 stages), then the four prefix tables
+template <bool BLOCKSCALE>
+constexpr int grouped_persist_table_offset() { return 3 * ((256 + 128) * 128 + (BLOCKSCALE ? 256 * 4 : 0)); }
+
+template <bool BLOCKSCALE>
+__global__ __launch_bounds__(512, 1) void gemm_grouped_persist_kernel(GemmArgs p_arg, int ctr_slot) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  constexpr int NTHREADS = 512, S_COLS = 8 * 64, TS = kGroupedMaxSlots + 1;
+  const int tid = threadIdx.x;
+  // prefix tables: row tiles of each kind in the slots before z (kinds 0 = L, 1 = M2, 2 = M1, 3 = S)
+  int* tab = reinterpret_cast<int*>(smem + grouped_persist_table_offset<BLOCKSCALE>());
+  // Everything a block keeps from tile to tile lives in LDS, and the arguments are read again from the kernel's
+  // argument segment for every tile (a handful of scalar loads): values held in scalar registers across the tile
+  // bodies would push the bodies' own loop values out of the register file.
+  __shared__ int s_rt[4], s_ncol[4], s_step, s_sfirst, s_kind, s_t, s_xcd;
+  {
+    const GemmArgs& p = p_arg;
+    const int na = p.num_active;
+    // thread z counts slot z's row tiles of each kind; a block-wide exclusive scan makes the tables
+    static_assert(kGroupedMaxSlots == NTHREADS, "one slot per thread");
+    const int lane = tid & 63, wave = tid >> 6;
+    int c[4] = {0, 0, 0, 0};
+    if (tid < na) {
+      const int rows = grouped_slot_count(p, tid);
+      const int head = grouped_head_rows(p, rows), rest = rows - head;
+      c[0] = head / 256;
+      if (rest > 256) c[1] = (rest + 255) / 256;        // (slots below big_rows keep all their rows here)
+      else if (rest > 128) c[1] = 1;
+      else if (rest > p.small_rows) c[2] = 1;
+      else if (rest > 0) c[3] = 1;
+    }
+    __shared__ int s_wsum[4][8];
+    int incl[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      incl[k] = c[k];
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl[k], o, 64);
+        if (lane >= o) incl[k] += up;
+      }
+      if (lane == 63) s_wsum[k][wave] = incl[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      int before = 0;
+      for (int w = 0; w < wave; ++w) before += s_wsum[k][w];
+      if (tid < na) tab[k * TS + tid] = before + incl[k] - c[k];
+      if (tid == NTHREADS - 1) tab[k * TS + na] = before + incl[k];  // (threads past the last slot add nothing)
+    }
+    __syncthreads();
+    if (tid == 0) {
+      const int ncol[4] = {(p.N + 255) / 256, (p.N + 127) / 128, (p.N + 255) / 256, (p.N + S_COLS - 1) / S_COLS};
+      int cnt[4];
+      for (int k = 0; k < 4; ++k) {
+        cnt[k] = tab[k * TS + na];
+        s_rt[k] = cnt[k];
+        s_ncol[k] = ncol[k];
+      }
+      // the share of the blocks that starts with the S tiles: their work / all work, in microseconds of one CU
+      const float nslab = (float)((p.K + 127) / 128);
+      const float w_mm = (float)(cnt[0] * ncol[0]) * (nslab * 1.63f + 11.4f) +
+                         (float)(cnt[1] * ncol[1] + cnt[2] * ncol[2]) * (nslab * 0.92f + 9.0f);
+      const float w_s = (float)(cnt[3] * ncol[3]) * (nslab * 2.6f + 6.0f) * p.share_bias;
+      int first_s = cnt[3] > 0 ? (int)((float)gridDim.x * w_s / (w_mm + w_s + 1e-9f) + 0.5f) : 0;
+      if (cnt[3] > 0 && first_s < 1) first_s = 1;
+      s_sfirst = (int)blockIdx.x < first_s ? 1 : 0;
+      s_step = 0;
+    }
+  }
+  typedef const __attribute__((address_space(4))) GemmArgs* kernarg_ptr_t;
+  kernarg_ptr_t pk = (kernarg_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();  // (the argument block is the first argument)
+  while (true) {
+    __syncthreads();  // every wave is done with the last tile's LDS and with the claim; the first time: the tables are there
+    if (tid == 0) {
+      // Column tile c of every kind belongs to XCD c % 8 (blocks go to the XCDs round-robin): the weight tiles an XCD
+      // works on stay in its L2 from one row tile to the next, and the eight XCDs read an activation row tile at about
+      // the same time.  One counter per kind and XCD; a block whose own XCD has nothing left of a kind helps the others
+      // before it moves on to the next kind.  `step` only grows: every (kind, XCD) pair is tried until it is empty, once.
+      unsigned int* ctr = g_grouped_ctr + ctr_slot * 32;
+      const int my_xcd = (int)(blockIdx.x & 7);
+      int kind = -1, t = 0, xcd = 0, step = s_step;
+      while (step < 32) {
+        const int k = s_sfirst ? 3 - (step >> 3) : (step >> 3);
+        const int x = (my_xcd + (step & 7)) & 7;
+        const int cols_x = x < s_ncol[k] ? (s_ncol[k] - x + 7) >> 3 : 0;
+        const int total = s_rt[k] * cols_x;
+        if (total > 0) {
+          t = (int)atomicAdd(ctr + k * 8 + x, 1u);
+          if (t < total) { kind = k; xcd = x; break; }
+        }
+        ++step;
+      }
+      s_step = step; s_kind = kind; s_t = t; s_xcd = xcd;
+    }
+    __syncthreads();
+    const int kind = s_kind, t = s_t, xcd = s_xcd;
+    if (kind < 0) break;
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+s"(pk));
+    GemmArgs p = *pk;
+#else
+    GemmArgs p = p_arg;  // (the host pass only parses this function)
+#endif
+    const int na = p.num_active;
+    const int* tb = tab + kind * TS;
+    const int cols_x = (s_ncol[kind] - xcd + 7) >> 3;
+    const int rt = t / cols_x, col = xcd + 8 * (t - rt * cols_x);
+    // the slot whose tiles hold row tile rt: the last z with tb[z] <= rt (slots without tiles of this kind repeat
+    // their successor's value and are skipped by taking the last)
+    int lo = 0, hi = na;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (tb[mid] <= rt) lo = mid; else hi = mid;
+    }
+    const int slot = lo, tile = rt - tb[lo];
+    int64_t slot_begin, slot_end;
+    grouped_slot_rows(p, slot, slot_begin, slot_end);
+    const int head = grouped_head_rows(p, (int)(slot_end - slot_begin));
+    const int64_t row_begin = kind == 0 ? slot_begin + (int64_t)tile * 256 : slot_begin + head + (int64_t)tile * 256;
+    const int64_t row_end = kind == 0 ? row_begin + 256 : slot_end;
+    const int bn = kind == 1 ? 128 : (kind == 3 ? S_COLS : 256);
+    const int n0 = col * bn;
+    const int64_t left = row_end - row_begin;
+    const int rows_here = (int)(left < 256 ? left : 256);
+    const int e = p.expert_ids[slot];
+    if (e < 0) {
+      grouped_zero_tile<NTHREADS>(p, row_begin, rows_here, n0, bn);
+      continue;
+    }
+    const uint8_t* bptr = p.b + (int64_t)e * p.b_expert_stride;
+    const float* bs_ptr = p.b_scales + (int64_t)e * p.bs_expert_stride;
+    if (kind == 0) {
+      tile_body<256, 256, 2, 4, 2, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+    } else if (kind == 1) {
+      tile_body<256, 128, 4, 2, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+    } else if (kind == 2) {
+      tile_body<128, 256, 2, 4, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+    } else {
+      if (rows_here <= 16) grouped_stream_body<1, 4, 2, BLOCKSCALE>(p, smem, row_begin, rows_here, n0, bptr, bs_ptr);
+      else grouped_stream_body<2, 4, 2, BLOCKSCALE>(p, smem, row_begin, rows_here, n0, bptr, bs_ptr);
+    }
+  }
+}
+
 template <int BM, int BN, int NS, bool BLOCKSCALE>
 constexpr int tile_lds_bytes() {
   return NS * ((BM + BN) * 128 + (BLOCKSCALE ? (BM < 64 ? 64 : BM) * 4 : 0));
@@ -1221,6 +1555,31 @@ static int launch_grouped_large(const GemmArgs& p, dim3 grid, hipStream_t stream
   static PerDeviceFlag attr_done;
   return launch_with_lds(gemm_grouped_large_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE>, attr_done,
                          tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), WAVES_M * WAVES_N * 64, p, grid, stream, name);
+}
+
+int compute_units();
+template <bool BLOCKSCALE>
+static int launch_grouped_persist(const GemmArgs& p, hipStream_t stream, const char* name) {
+  static PerDeviceFlag attr_done;
+  static std::atomic<unsigned int> seq{0};
+  constexpr int bodies = grouped_persist_table_offset<BLOCKSCALE>();  // the largest of the four tile bodies; the tables sit behind it
+  static_assert(bodies == tile_lds_bytes<256, 128, 3, BLOCKSCALE>(), "the 256 x 128 body's stages");
+  static_assert(tile_lds_bytes<256, 256, 2, BLOCKSCALE>() <= bodies && tile_lds_bytes<128, 256, 3, BLOCKSCALE>() <= bodies && 8 * 16384 <= bodies,
+                "the tables sit behind the largest tile");
+  constexpr int lds = bodies + 4 * (kGroupedMaxSlots + 1) * 4;
+  static_assert(lds + 64 <= 160 * 1024, "one block per CU");
+  // a set of counters per launch in flight (64 sets: launches that follow each other on a stream could share one)
+  const int slot = (int)(seq.fetch_add(1, std::memory_order_relaxed) % kGroupedCtrSlots);
+  hipLaunchKernelGGL(grouped_ctr_zero_kernel, dim3(1), dim3(64), 0, stream, slot);
+  auto kern = gemm_grouped_persist_kernel<BLOCKSCALE>;
+  bool& done = attr_done.here();
+  if (!done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, lds, hipGetErrorString(e));
+    done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)compute_units()), dim3(512), lds, stream, p, slot);
+  return launch_status(name);
 }
 
 // The persistent kernel takes matmuls of whole 256 x 256 tiles with 16-byte aligned bf16 rows of C, one launch,
@@ -1673,6 +2032,15 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int6
   // The large-tile launch goes down a second stream, as a fixed set of blocks, so that its tiles (bound by the matrix
   // pipe) and the other launch's (mostly bound by HBM) share the chip instead of taking turns; the caller's stream
   // waits for both.  (The tuning switch `grouped_overlap` = 0 keeps the two launches in line on the caller's stream.)
+  // One persistent launch that shares the chip out between its four kinds of tiles (the tuning switch
+  // `grouped_persist` = 0 goes back to the two launches below).
+  if (tuning().grouped_persist && !big && p.num_active <= kGroupedMaxSlots) {
+    // (every slot's full 256-row tiles are L tiles here: one kernel, no second launch to fill)
+    p.big_rows = tune != 4 ? 256 : 0;
+    p.share_bias = tuning().grouped_share * 2.0f;
+    return blockscale ? launch_grouped_persist<true>(p, stream, "gemm_grouped_persist_block")
+                      : launch_grouped_persist<false>(p, stream, "gemm_grouped_persist_row");
+  }
   SideStream* side = nullptr;
   const bool large = !big && tune != 4 && max_tokens >= big_rows && T / 256 <= 65535;
   if (large && tuning().grouped_overlap) side = side_stream();

@@ -10,8 +10,9 @@
 //   MAXFP8_STREAMK=0 / 2       never / always split the work of whole-tile matmuls evenly over the blocks
 //                              (default 1: where the cost model says it pays)
 //   MAXFP8_BIG_ROWS=n          grouped: slots with at least n rows use the large-tile launch (1024)
-//   MAXFP8_GROUPED_OVERLAP=0   grouped: the two launches in line on the caller's stream
-//   MAXFP8_GROUPED_SHARE=x     grouped: scales the share estimate of the large-tile launch (0.5)
+//   MAXFP8_GROUPED_PERSIST=0   grouped: two launches (large tiles / the rest) instead of the one persistent launch
+//   MAXFP8_GROUPED_OVERLAP=0   grouped, two launches: in line on the caller's stream
+//   MAXFP8_GROUPED_SHARE=x     grouped: scales the estimate of how much of the chip the small tiles need (0.5)
 //   MAXFP8_SKINNY=<ntw>4<KB>   force a shape of the weight-streaming kernel (e.g. 1408, 2416)
 #pragma once
 
@@ -24,6 +25,7 @@ struct Tuning {
   bool persist = true;
   int streamk = 1;
   int big_rows = 1024;
+  bool grouped_persist = true;
   bool grouped_overlap = true;
   float grouped_share = 0.5f;
   int skinny = 0;

@@ -153,10 +153,14 @@ def test_moe_config_sampled(dev, proj, Kd, Nd):
     assert_rel(f32_np(c[r:r + 1]), cpu, TOL, f"{proj}: row {r} against the CPU oracle", natural_scale=True)
 
 
-def test_random_groupings_are_exact(dev):
+@pytest.mark.parametrize("launches", ["one persistent launch", "two launches"])
+def test_random_groupings_are_exact(dev, tune, launches):
     """A seeded sweep of groupings (empty, tiny, mid-size and >= 1024-row slots side by side, skipped experts, rows
-    past the last slot, ragged and aligned N): on integer data the automatic choice -- large-tile launch, 128-row
-    tiles, 32-row tiles -- equals the scalar kernel bit for bit on every row that belongs to a slot."""
+    past the last slot, ragged and aligned N): on integer data the automatic choice -- 256-row tiles, 128-row
+    tiles, the weight-streaming form of at most 32 rows; as one persistent launch (the default) and as the two
+    launches behind MAXFP8_GROUPED_PERSIST=0 -- equals the scalar kernel bit for bit on every row that belongs
+    to a slot."""
+    tune(MAXFP8_GROUPED_PERSIST=None if launches == "one persistent launch" else "0")
     rng = np.random.default_rng(77)
     for it in range(36):
         E = int(rng.integers(1, 24))
@@ -186,6 +190,25 @@ def test_random_groupings_are_exact(dev):
         got = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=out)
         want = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=out, algo="naive")
         assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, N {N}, K {K}, {out}"
+
+
+def test_more_slots_than_the_persistent_launch_holds(dev):
+    """600 active slots: more than the persistent launch's tables hold (512), so the two-launch form runs; exact on
+    integer data like every other path."""
+    rng = np.random.default_rng(5)
+    E, N, K = 600, 128, 256
+    counts = rng.integers(0, 5, E)
+    counts[7] = 140
+    T = int(counts.sum())
+    a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (T, K)).astype(np.float32)))
+    b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (E, N, K)).astype(np.float32)))
+    sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (K // 128, -(-T // 4) * 4))).astype(np.float32))
+    sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (E, 1, K // 128))).astype(np.float32))
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32)
+    ids = torch.from_numpy(rng.permutation(E).astype(np.int32))
+    got = run(a, b, sa, sb, off, ids, int(counts.max()), E, dev)
+    want = run(a, b, sa, sb, off, ids, int(counts.max()), E, dev, algo="naive")
+    assert torch.equal(got, want)
 
 
 # ---- the layer above the op: quantized_grouped_matmul and Fp8Strategy -----------------------------------

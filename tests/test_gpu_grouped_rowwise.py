@@ -60,7 +60,9 @@ def test_minus_one_expert_empty_slots_and_spare_rows(dev):
     assert not f32_np(c)[lo:lo + counts4[2]].any(), "expert -1 must give zeros"
 
 
-def test_exact_integers_are_bit_identical(dev):
+@pytest.mark.parametrize("launches", ["one persistent launch", "two launches"])
+def test_exact_integers_are_bit_identical(dev, tune, launches):
+    tune(MAXFP8_GROUPED_PERSIST=None if launches == "one persistent launch" else "0")
     counts, ids, E, N, K = [33, 1200, 7], [1, 0, 2], 3, 256, 256
     g = torch.Generator().manual_seed(0)
     T = sum(counts)
