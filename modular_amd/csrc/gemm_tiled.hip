@@ -1544,11 +1544,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_k
 // memory, no host synchronisation.  The result of a tile does not depend on which block computes it.
 constexpr int kGroupedCtrSlots = 64;
 constexpr int kGroupedMaxSlots = 512;   // slots (active experts) the LDS tables hold
-static __device__ unsigned int g_grouped_ctr[kGroupedCtrSlots * 32];  // per launch in flight: kind x XCD
-
-__global__ void grouped_ctr_zero_kernel(int slot) {
-  if (threadIdx.x < 32) g_grouped_ctr[slot * 32 + threadIdx.x] = 0u;
-}
+// Per launch in flight: a counter per (kind, XCD) and one that counts the blocks that are done.  All zero when the
+// module is loaded; the last block of a launch to finish puts its set back to zero, so a set is clean whenever a
+// launch takes it (sets are handed out round-robin: 64 grouped matmuls are never in flight together).
+constexpr int kGroupedCtrStride = 33;
+static __device__ unsigned int g_grouped_ctr[kGroupedCtrSlots * kGroupedCtrStride];
 
 // One wave: C[rows of the slot, 16 * NTW weight rows from n0 + 16 * NTW * wave] over the whole of K.  The weight slabs
 // (16 * NTW rows x 128 bytes) travel by LDS-DMA through the wave's own ring of DEPTH slots, the activations (at most
@@ -1793,7 +1793,7 @@ __global__ __launch_bounds__(512, 1) void gemm_grouped_persist_kernel(GemmArgs p
       // works on stay in its L2 from one row tile to the next, and the eight XCDs read an activation row tile at about
       // the same time.  One counter per kind and XCD; a block whose own XCD has nothing left of a kind helps the others
       // before it moves on to the next kind.  `step` only grows: every (kind, XCD) pair is tried until it is empty, once.
-      unsigned int* ctr = g_grouped_ctr + ctr_slot * 32;
+      unsigned int* ctr = g_grouped_ctr + ctr_slot * kGroupedCtrStride;
       const int my_xcd = (int)(blockIdx.x & 7);
       int kind = -1, t = 0, xcd = 0, step = s_step;
       while (step < 32) {
@@ -1811,7 +1811,16 @@ __global__ __launch_bounds__(512, 1) void gemm_grouped_persist_kernel(GemmArgs p
     }
     __syncthreads();
     const int kind = s_kind, t = s_t, xcd = s_xcd;
-    if (kind < 0) break;
+    if (kind < 0) {
+      // nothing left for this block (nor, by then, for any block that arrives here): the last one cleans the counters
+      if (tid == 0) {
+        unsigned int* ctr = g_grouped_ctr + ctr_slot * kGroupedCtrStride;
+        if (atomicAdd(ctr + 32, 1u) == gridDim.x - 1) {
+          for (int i = 0; i < kGroupedCtrStride; ++i) atomicExch(ctr + i, 0u);
+        }
+      }
+      break;
+    }
 #if defined(__HIP_DEVICE_COMPILE__)
     asm volatile("" : "+s"(pk));
     GemmArgs p = *pk;
@@ -1914,7 +1923,6 @@ static int launch_grouped_persist(const GemmArgs& p, hipStream_t stream, const c
   static_assert(lds + 64 <= 160 * 1024, "one block per CU");
   // a set of counters per launch in flight (64 sets: launches that follow each other on a stream could share one)
   const int slot = (int)(seq.fetch_add(1, std::memory_order_relaxed) % kGroupedCtrSlots);
-  hipLaunchKernelGGL(grouped_ctr_zero_kernel, dim3(1), dim3(64), 0, stream, slot);
   auto kern = gemm_grouped_persist_kernel<BLOCKSCALE>;
   bool& done = attr_done.here();
   if (!done) {
