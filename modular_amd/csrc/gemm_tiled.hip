@@ -1858,7 +1858,9 @@ __global__ __launch_bounds__(512, 1) void gemm_grouped_persist_kernel(GemmArgs p
     if (kind == 0) {
       tile_body<256, 256, 2, 4, 2, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
     } else if (kind == 1) {
-      tile_body<256, 128, 4, 2, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+      // (a rest of at most 192 rows: three quarters of the MFMAs)
+      if (rows_here <= 192) tile_body<192, 128, 2, 4, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+      else tile_body<256, 128, 4, 2, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
     } else if (kind == 2) {
       tile_body<128, 256, 2, 4, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
     } else {
