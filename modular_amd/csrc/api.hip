@@ -131,6 +131,7 @@ static const Tuning* read_tuning(unsigned generation) {
   t->grouped_overlap = num("MAXFP8_GROUPED_OVERLAP", 1) != 0;
   t->grouped_persist = num("MAXFP8_GROUPED_PERSIST", 1) != 0;
   t->pingpong = num("MAXFP8_PINGPONG", 0) != 0;
+  t->skinny_alds = num("MAXFP8_SKINNY_ALDS", 1) != 0;
   const char* sb = getenv("MAXFP8_GROUPED_SHARE");
   t->grouped_share = sb ? (float)atof(sb) : 0.5f;
   t->skinny = num("MAXFP8_SKINNY", 0);

@@ -47,12 +47,16 @@ __device__ __forceinline__ uint32_t sk_clamp_u32(int64_t v) {
   return v > 0xfffffff0ll ? 0xfffffff0u : (v < 0 ? 0u : (uint32_t)v);
 }
 
-template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
+// ALDS: the activations of a wave's share of K are copied to LDS once, before the loop (at most kSkinnyALdsBytes per
+// wave), instead of two loads per slab and 16-token group: on a launch that is a single round of blocks those loads
+// are half of the loop's vector-memory instructions and cost 8 % of the kernel, whatever they fetch.
+constexpr int kSkinnyALdsBytes = 4096;
+template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES, bool ALDS = false>
 struct SkinnyCfg {
   static constexpr int WAVES = NWAVES;
   static constexpr int SLOT = NTW * 2048;                    // one slab of the block's rows
   // VMEM instructions a wave issues per slab, in this order: activations, scales, weight DMA
-  static constexpr int PER = 2 * MT + (BLOCKSCALE ? MT + 1 : 0) + 2 * NTW;
+  static constexpr int PER = (ALDS ? 0 : 2 * MT) + (BLOCKSCALE ? MT + 1 : 0) + 2 * NTW;
   // slabs in flight per wave: RING_KB of weights, limited by the 6-bit vmcnt counter and by the
   // registers the activation fragments of the in-flight slabs take (96)
   static constexpr int D_BYTES = RING_KB * 1024 / SLOT, D_CNT = 63 / PER + 1, D_REGS = 96 / (MT * 8);
@@ -60,13 +64,15 @@ struct SkinnyCfg {
   static constexpr int DEPTH = D_MIN < 2 ? 2 : D_MIN;
   static constexpr int RING = DEPTH * SLOT;                  // per wave
   static constexpr int RED = WAVES * MT * NTW * 4 * 64 * 4;  // reduction buffer (reuses the rings)
-  static constexpr int SMEM = WAVES * RING > RED ? WAVES * RING : RED;
+  static constexpr int RINGS = WAVES * RING > RED ? WAVES * RING : RED;
+  static constexpr int SMEM = RINGS;  // (ALDS: plus WAVES * M * the share's bytes, added at the launch)
 };
 
-template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
+template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES, bool ALDS = false>
 __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in) {
   const GemmArgs p = gridDim.y == 1 ? p_in : batch_view(p_in, blockIdx.y);
-  using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
+  using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES, ALDS>;
+  static_assert(!ALDS || MT == 1, "activations in LDS: one 16-token group");
   constexpr int WAVES = Cfg::WAVES, DEPTH = Cfg::DEPTH, SLOT = Cfg::SLOT, PER = Cfg::PER;
   static_assert((DEPTH - 1) * PER < 64, "vmcnt is a 6-bit counter");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -103,6 +109,22 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
   const uint32_t frag0 = lm * 128 + ((lq ^ (lm & 7)) << 4);
   const uint32_t frag1 = lm * 128 + (((lq + 4) ^ (lm & 7)) << 4);
   uint8_t* ring = smem + wave * Cfg::RING;
+  // ALDS: token t's bytes of this wave's share of K sit at a_lds + t * a_tok; lane (lm, lq) reads token min(lm, M - 1)
+  // (the columns of C past M are never stored, so what their lanes multiply does not matter)
+  [[maybe_unused]] const uint32_t a_tok = ((uint32_t)per_wave * 128u + 1023u) & ~1023u;  // (whole copies: 1024 bytes each)
+  [[maybe_unused]] uint8_t* a_lds = smem + Cfg::RINGS + wave * ((uint32_t)p.M * a_tok);
+  [[maybe_unused]] const uint32_t a_rd = (uint32_t)(lm < p.M ? lm : p.M - 1) * a_tok + lq * 16;
+  if constexpr (ALDS) {
+    // one instruction moves 1024 consecutive bytes of a token; bytes past K or past the share are not fetched (zeros)
+    const uint32_t share_begin = (uint32_t)s_begin * 128u, share_end = (uint32_t)(s_end > s_begin ? s_end : s_begin) * 128u;
+    const uint32_t k_end = share_end < (uint32_t)p.K ? share_end : (uint32_t)p.K;
+    for (int t = 0; t < p.M; ++t)
+      for (uint32_t piece = 0; piece < a_tok; piece += 1024u) {
+        const uint32_t k = share_begin + piece + lane * 16u;
+        const uint32_t kill = k < k_end ? 0u : 0x80000000u;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (sk_lds_ptr_t)(a_lds + t * a_tok + piece), 16, ((uint32_t)t * (uint32_t)p.lda + k) | kill, 0, 0, 0);
+      }
+  }
 
   __amdgpu_buffer_rsrc_t as_rsrc = sk_rsrc(nullptr, 0), bs_rsrc = sk_rsrc(nullptr, 0);
   uint32_t as_voff[MT];
@@ -142,11 +164,13 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
       if (koff + 64 + lq * 16 >= (uint32_t)p.K) kill1 = 0x80000000u;
       if (koff + cchunk * 16 >= (uint32_t)p.K) killw = 0x80000000u;
     }
+    if constexpr (!ALDS) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const v4i lo = sk_load16(a_rsrc, a_off[t] | kill0, koff);
-      const v4i hi = sk_load16(a_rsrc, a_off[t] | kill1, koff_hi);
-      af[d][t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      for (int t = 0; t < MT; ++t) {
+        const v4i lo = sk_load16(a_rsrc, a_off[t] | kill0, koff);
+        const v4i hi = sk_load16(a_rsrc, a_off[t] | kill1, koff_hi);
+        af[d][t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
     }
     if constexpr (BLOCKSCALE) {
 #pragma unroll
@@ -163,11 +187,18 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
                                                koff + t * w_tile + w_half, 0, 0);
     }
   };
-  auto compute = [&](auto d_c) {
+  auto compute = [&](auto d_c, [[maybe_unused]] int slab) {
     constexpr int d = decltype(d_c)::value;
     // the slot's loads are the oldest in flight: everything issued for the DEPTH-1 younger slots may stay
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * PER) : "memory");
     const uint8_t* slot = ring + d * SLOT;
+    if constexpr (ALDS) {
+      // (a slab past the share's end multiplies zeros -- its weights were not fetched -- with whatever this reads)
+      const uint32_t at = (uint32_t)(slab < s_end ? slab - s_begin : 0) * 128u;
+      const v4i lo = *reinterpret_cast<const v4i*>(a_lds + a_rd + at);
+      const v4i hi = *reinterpret_cast<const v4i*>(a_lds + a_rd + at + 64);
+      af[d][0] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
       const v4i lo = *reinterpret_cast<const v4i*>(slot + nt * 2048 + frag0);
@@ -196,7 +227,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
   for (int base = s_begin; base < s_end; base += DEPTH) {
     for_each_slot([&](auto d_c) {
       constexpr int d = decltype(d_c)::value;
-      compute(d_c);
+      compute(d_c, base + d);
       issue(base + DEPTH + d, d_c);
     });
   }
@@ -288,19 +319,35 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
   }
 }
 
-template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES>
+template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES, bool ALDS = false>
 static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream) {
-  using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
-  auto kern = gemm_skinny_kernel<NTW, MT, BLOCKSCALE, RING_KB, NWAVES>;
+  if constexpr (MT == 1 && !ALDS) {
+    // few tokens, a share of K per wave that fits, and a weight matrix small enough that the launch is about one round of
+    // blocks: the activations go to LDS once (84 MB, M = 1: 17.8 -> 17.0 us; on a 470 MB matrix, where blocks come and
+    // go, the per-slab loads cost nothing and this form measured 1 % slower).  Not for the fused QKV epilogue's build, a
+    // rare caller at these sizes, to keep the number of kernels down.
+    const int64_t per_wave = ceil_div(ceil_div(p.K, 128), NWAVES);
+    if (tuning().skinny_alds && !p.kv_on && (int64_t)p.N * p.K < ((int64_t)1 << 27) &&
+        (int64_t)p.M * ((per_wave * 128 + 1023) / 1024 * 1024) <= kSkinnyALdsBytes)
+      return launch_skinny_r<NTW, MT, BLOCKSCALE, RING_KB, NWAVES, true>(p, batch, stream);
+  }
+  using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES, ALDS>;
+  auto kern = gemm_skinny_kernel<NTW, MT, BLOCKSCALE, RING_KB, NWAVES, ALDS>;
   static PerDeviceFlag attr;
   bool& attr_done = attr.here();
+  constexpr int smem_max = Cfg::SMEM + (ALDS ? NWAVES * kSkinnyALdsBytes : 0);
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM);
-    if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "gemm_skinny: cannot reserve %d bytes of LDS: %s", Cfg::SMEM, hipGetErrorString(e));
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem_max);
+    if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "gemm_skinny: cannot reserve %d bytes of LDS: %s", smem_max, hipGetErrorString(e));
     attr_done = true;
   }
+  int smem = Cfg::SMEM;
+  if constexpr (ALDS) {
+    const int64_t per_wave = ceil_div(ceil_div(p.K, 128), NWAVES);
+    smem += NWAVES * (int)(p.M * ((per_wave * 128 + 1023) / 1024 * 1024));
+  }
   const int64_t blocks = ceil_div(p.N, 16 * NTW);
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, (unsigned)batch), dim3(NWAVES * 64), Cfg::SMEM, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, (unsigned)batch), dim3(NWAVES * 64), smem, stream, p);
   return launch_status("gemm_skinny");
 }
 

@@ -15,6 +15,7 @@
 //   MAXFP8_GROUPED_PERSIST=0   grouped: two launches (large tiles / the rest) instead of the one persistent launch
 //   MAXFP8_GROUPED_OVERLAP=0   grouped, two launches: in line on the caller's stream
 //   MAXFP8_GROUPED_SHARE=x     grouped: scales the estimate of how much of the chip the small tiles need (0.5)
+//   MAXFP8_SKINNY_ALDS=0       decode kernel: activations loaded per slab even where a wave's share of them fits LDS
 //   MAXFP8_SKINNY=<ntw>4<KB>   force a shape of the weight-streaming kernel (e.g. 1408, 2416)
 #pragma once
 
@@ -32,6 +33,7 @@ struct Tuning {
   bool grouped_overlap = true;
   float grouped_share = 0.5f;
   int skinny = 0;
+  bool skinny_alds = true;
   unsigned generation = 0;  // counts the reloads: part of the key of every cache that depends on the switches
 };
 

@@ -132,6 +132,34 @@ def test_every_decode_shape_is_exact(dev, tune, sel, M, N, K):
     assert np.array_equal(got_row, want_row), f"row mode, shape {sel}"
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 272, 128), (1, 1000, 1040), (1, 2064, 8192), (2, 520, 8192), (2, 136, 4112),
+                                   (3, 1032, 4096), (4, 264, 2048), (4, 4104, 4000)])
+def test_decode_activations_through_lds(dev, tune, M, N, K):
+    """With few tokens and a short enough share of K per wave the decode kernel copies the activations to LDS once
+    instead of loading them slab by slab.  Same operands into the same MFMAs: bit-equal to the per-slab form on
+    random data (both scale modes, K tails, ragged N), and exact on integer data."""
+    for kind in ("block", "row"):
+        if kind == "block":
+            a, b = synth.random_fp8((M, K), M + K), synth.random_fp8((N, K), N + 1)
+            kb = -(-K // 128)
+            sa, sb = synth.random_scales((kb, -(-M // 4) * 4), 3), synth.random_scales((-(-N // 128), kb), 4)
+            cfg = BLK
+        else:
+            a, b = synth.random_fp8((M, K), M + K), synth.random_fp8((N, K), N + 1)
+            sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+            cfg = ROW
+        tune(MAXFP8_SKINNY_ALDS=None)
+        got = mm(a, b, sa, sb, cfg, dev, algo="skinny")
+        again = mm(a, b, sa, sb, cfg, dev, algo="skinny")
+        tune(MAXFP8_SKINNY_ALDS="0")
+        want = mm(a, b, sa, sb, cfg, dev, algo="skinny")
+        assert torch.equal(got.view(torch.int32), want.view(torch.int32)), f"{kind} {M}x{N}x{K}"
+        assert torch.equal(again.view(torch.int32), want.view(torch.int32)), f"{kind} {M}x{N}x{K}, second launch"
+    tune(MAXFP8_SKINNY_ALDS=None)
+    ea, eb, esa, esb, want = exact_case(M, N, K, seed=M + N)
+    assert np.array_equal(f32_np(mm(ea, eb, esa, esb, BLK, dev, algo="skinny")).astype(np.float64), want)
+
+
 @pytest.mark.parametrize("M,N,K", [(3, 16400, 4096), (12, 10256, 4096), (24, 10304, 4224), (40, 12288, 4096),
                                    (64, 8192, 2048), (20, 20480, 1536), (16, 16384, 16384), (8, 16384, 16384),
                                    (5, 4090, 2048), (32, 5120, 5120)])
