@@ -81,6 +81,44 @@ __device__ __forceinline__ void buffer_store_b128_guarded(const v4u_t v, const _
   asm volatile("s_nop 7" ::"v"(v));
 }
 
+// The activation scales of a slab in LDS.  The copy puts its lanes' values at consecutive words, and a lane may fetch
+// any row: word i of the scale area gets the row that makes the TM scales a lane needs in the main loop -- rows lm,
+// lm + 16, ... of its wave's WM = 16 * TM rows -- neighbours (word wm * WM + lm * TM + mt), so that they come back in one
+// or two wide LDS reads instead of TM narrow ones.
+// (Wave tiles whose TM is not a multiple of 4 keep the rows in order: their scales would come back in reads that
+// straddle 16-byte boundaries, which measured a quarter slower than narrow reads on the 192-row tiles.)
+template <int WM>
+__device__ __forceinline__ int scale_word_row(int i) {
+  constexpr int TM = WM / 16;
+  if constexpr (TM % 4 != 0) return i;
+  const int in_wave = i % WM;
+  return (i / WM) * WM + (in_wave % TM) * 16 + in_wave / TM;
+}
+
+// byte offset, in a stage's scale area, of the first scale of lane row lm of a wave whose rows begin at wave_row0
+template <int TM>
+__device__ __forceinline__ uint32_t scale_read_offset(int wave_row0, int lm) {
+  return (uint32_t)(wave_row0 + (TM % 4 == 0 ? lm * TM : lm)) * 4u;
+}
+// a lane's TM scales: 16-byte reads of neighbouring words where TM allows, else one word per 16-row group
+template <int TM>
+struct ScaleRow { float v[TM]; __device__ __forceinline__ float operator[](int i) const { return v[i]; } };
+template <int TM>
+__device__ __forceinline__ ScaleRow<TM> read_scales(const uint8_t* at) {
+  ScaleRow<TM> out;
+  if constexpr (TM % 4 == 0) {
+#pragma unroll
+    for (int i = 0; i < TM / 4; ++i) {
+      const v4f q = *reinterpret_cast<const v4f*>(at + i * 16);
+      out.v[4 * i] = q[0]; out.v[4 * i + 1] = q[1]; out.v[4 * i + 2] = q[2]; out.v[4 * i + 3] = q[3];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) out.v[i] = *reinterpret_cast<const float*>(at + i * 64);
+  }
+  return out;
+}
+
 // One BM x BN tile of C: rows [row_begin, row_end) (at most BM of them are used) by columns
 // [n0, n0 + BN) of the weight matrix at bptr / scales at bs_ptr.  Called by every thread of a
 // block of WAVES_M * WAVES_N waves with `smem` = the block's dynamic LDS.
@@ -172,7 +210,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   uint32_t s_voff = 0, s_slab_step = 0;
   if constexpr (BLOCKSCALE) {
     s_rsrc = t2_rsrc(p.a_scales + row_begin, t2_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + rows_here) * 4));
-    const int r = s_chunk * 64 + lane;
+    const int r = scale_word_row<WM>(s_chunk * 64 + lane);
     s_voff = r < rows_here ? (uint32_t)r * 4u : 0x80000000u;
     s_slab_step = (uint32_t)p.a_scales_ld * 4u;
   }
@@ -252,7 +290,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
   }
   const float* bs_row = nullptr;
   if constexpr (BLOCKSCALE) bs_row = bs_ptr + (int64_t)((n0 + wn * WN) / 128) * p.b_scales_ld;
-  const uint32_t s_rd = (uint32_t)((BM + BN) * 128 + (wm * WM + lm) * 4);
+  const uint32_t s_rd = (uint32_t)((BM + BN) * 128) + scale_read_offset<TM>(wm * WM, lm);
 
   // NS LDS stages, one barrier per slab, DMA issued NS-1 slabs ahead.  At the top of slab j a
   // wave waits until its own DMA of slab j has landed (the younger ones may stay in flight:
@@ -288,8 +326,9 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     const uint8_t* sa = smem + buf * STAGE_BYTES;
     float s_cur[TM];
     if constexpr (BLOCKSCALE) {
-#pragma unroll
-      for (int mt = 0; mt < TM; ++mt) s_cur[mt] = *reinterpret_cast<const float*>(sa + s_rd + mt * 64) * bs;
+const ScaleRow<TM> a_sc = read_scales<TM>(sa + s_rd);
+      #pragma unroll
+      for (int mt = 0; mt < TM; ++mt) s_cur[mt] = a_sc[mt] * bs;
     }
     v8i bf[TN];
 #pragma unroll
@@ -726,7 +765,7 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   uint32_t s_voff = 0, s_slab_step = 0;
   if constexpr (BLOCKSCALE) {
     s_rsrc = t2_rsrc(p.a_scales, t2_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + p.M) * 4));
-    s_voff = (uint32_t)(s_chunk * 64 + lane) * 4u;
+    s_voff = (uint32_t)scale_word_row<WM>(s_chunk * 64 + lane) * 4u;
     s_slab_step = (uint32_t)p.a_scales_ld * 4u;
   }
   struct TileAt { uint32_t a, b, s; };  // byte offsets of a tile's activation rows, weight rows and activation scales
@@ -774,7 +813,7 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
     const v4i hi = *reinterpret_cast<const v4i*>(g + wfrag1);
     return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
-  const uint32_t s_rd = (uint32_t)((BM + BN) * 128 + (wm * WM + lm) * 4);
+  const uint32_t s_rd = (uint32_t)((BM + BN) * 128) + scale_read_offset<TM>(wm * WM, lm);
   uint8_t* wbuf = smem + NS * STAGE_BYTES + wave * SIDE_BYTES;
   const int rr = lane >> 3, cc = lane & 7;
   const __amdgpu_buffer_rsrc_t c_rsrc = t2_rsrc(p.c, t2_clamp_u32(((int64_t)(p.M - 1) * p.ldc + p.N) * 2));
@@ -869,8 +908,9 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
       const uint8_t* sa = smem + buf * STAGE_BYTES;
       float s_cur[TM];
       if constexpr (BLOCKSCALE) {
-#pragma unroll
-        for (int mt = 0; mt < TM; ++mt) s_cur[mt] = *reinterpret_cast<const float*>(sa + s_rd + mt * 64) * bs;
+const ScaleRow<TM> a_sc = read_scales<TM>(sa + s_rd);
+        #pragma unroll
+        for (int mt = 0; mt < TM; ++mt) s_cur[mt] = a_sc[mt] * bs;
       }
       v8i bf[TN];
 #pragma unroll
@@ -1079,7 +1119,7 @@ __device__ __forceinline__ void persist_pp_body(const GemmArgs& p, uint8_t* smem
   uint32_t s_voff = 0, s_slab_step = 0;
   if constexpr (BLOCKSCALE) {
     s_rsrc = t2_rsrc(p.a_scales, t2_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + p.M) * 4));
-    s_voff = (uint32_t)(s_chunk * 64 + lane) * 4u;
+    s_voff = (uint32_t)scale_word_row<WM>(s_chunk * 64 + lane) * 4u;
     s_slab_step = (uint32_t)p.a_scales_ld * 4u;
   }
   struct TileAt { uint32_t a, b, s; };
@@ -1131,7 +1171,7 @@ __device__ __forceinline__ void persist_pp_body(const GemmArgs& p, uint8_t* smem
     const v4i hi = *reinterpret_cast<const v4i*>(g + wfrag1);
     return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
-  const uint32_t s_rd = (uint32_t)((BM + BN) * 128 + (wm * WM + lm) * 4);
+  const uint32_t s_rd = (uint32_t)((BM + BN) * 128) + scale_read_offset<TM>(wm * WM, lm);
   uint8_t* wbuf = smem + NS * STAGE_BYTES + wave * SIDE_BYTES;
   const int rr = lane >> 3, cc = lane & 7;
   const __amdgpu_buffer_rsrc_t c_rsrc = t2_rsrc(p.c, t2_clamp_u32(((int64_t)(p.M - 1) * p.ldc + p.N) * 2));
@@ -1240,8 +1280,9 @@ __device__ __forceinline__ void persist_pp_body(const GemmArgs& p, uint8_t* smem
     const int slab1 = n1_same ? slab + 1 : 0;
     const uint32_t dead1 = (n1_same || has_next) ? 0u : 0x80000000u;
     if constexpr (BLOCKSCALE) {
-#pragma unroll
-      for (int mt = 0; mt < TM; ++mt) s_cur[mt] = *reinterpret_cast<const float*>(sa + s_rd + mt * 64) * bs;
+const ScaleRow<TM> a_sc = read_scales<TM>(sa + s_rd);
+      #pragma unroll
+      for (int mt = 0; mt < TM; ++mt) s_cur[mt] = a_sc[mt] * bs;
     }
 #pragma unroll
     for (int t = 0; t < TN; ++t) bf[t] = read_wfrag(sa + b_frag_base, t);
@@ -1913,10 +1954,16 @@ static int launch_grouped_large(const GemmArgs& p, dim3 grid, hipStream_t stream
 }
 
 int compute_units();
+// One numbering of the launches for both scale modes: the two instantiations below share the counter sets (and, for the
+// work-split kernel, the flags) in device memory, so a counter of their own each would hand the same set, and the same
+// flag value, to a block-scaled and a row-scaled launch.
+static unsigned int next_launch_number() {
+  static std::atomic<unsigned int> seq{0};
+  return seq.fetch_add(1, std::memory_order_relaxed);
+}
 template <bool BLOCKSCALE>
 static int launch_grouped_persist(const GemmArgs& p, hipStream_t stream, const char* name) {
   static PerDeviceFlag attr_done;
-  static std::atomic<unsigned int> seq{0};
   constexpr int bodies = grouped_persist_table_offset<BLOCKSCALE>();  // the largest of the four tile bodies; the tables sit behind it
   static_assert(bodies == tile_lds_bytes<256, 128, 3, BLOCKSCALE>(), "the 256 x 128 body's stages");
   static_assert(tile_lds_bytes<256, 256, 2, BLOCKSCALE>() <= bodies && tile_lds_bytes<128, 256, 3, BLOCKSCALE>() <= bodies && 8 * 16384 <= bodies,
@@ -1924,7 +1971,7 @@ static int launch_grouped_persist(const GemmArgs& p, hipStream_t stream, const c
   constexpr int lds = bodies + 4 * (kGroupedMaxSlots + 1) * 4;
   static_assert(lds + 64 <= 160 * 1024, "one block per CU");
   // a set of counters per launch in flight (64 sets: launches that follow each other on a stream could share one)
-  const int slot = (int)(seq.fetch_add(1, std::memory_order_relaxed) % kGroupedCtrSlots);
+  const int slot = (int)(next_launch_number() % kGroupedCtrSlots);
   auto kern = gemm_grouped_persist_kernel<BLOCKSCALE>;
   bool& done = attr_done.here();
   if (!done) {
@@ -1992,13 +2039,12 @@ static size_t streamk_workspace_bytes() { return (size_t)streamk_blocks() * 256 
 template <bool BLOCKSCALE>
 static int launch_streamk(const GemmArgs& p_in, hipStream_t stream, const char* name) {
   static PerDeviceFlag attr_done;
-  static std::atomic<unsigned int> seq{0};
   constexpr int lds = tile_lds_bytes<256, 256, 2, BLOCKSCALE>() + 8 * 2048;
   GemmArgs p = p_in;
   // every launch gets a sequence number (never 0) as its flag value and one of 64 sets of flags: launches that
   // follow each other on a stream may reuse a set at once, and 64 matmuls of this size are never in flight together
-  unsigned int n = seq.fetch_add(1, std::memory_order_relaxed) + 1;
-  if (n == 0) n = seq.fetch_add(1, std::memory_order_relaxed) + 1;
+  unsigned int n = next_launch_number() + 1;
+  if (n == 0) n = next_launch_number() + 1;
   p.streamk_seq = n;
   p.streamk_slot = (int)(n % kStreamkSlots);
   return launch_with_lds(gemm_streamk_kernel<256, 256, 2, 4, BLOCKSCALE>, attr_done, lds, 512, p, dim3((unsigned)streamk_blocks()), stream, name);

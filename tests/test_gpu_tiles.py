@@ -305,6 +305,32 @@ def test_stream_k_equals_per_tile_kernel(dev, tune, M, N, K, kind):
     assert torch.equal(persistent.view(torch.int16), per_tile.view(torch.int16))
 
 
+def test_stream_k_scale_modes_take_turns(dev, tune):
+    # Block-scaled and row-scaled launches share the hand-over flags in device memory, so they must share the numbering
+    # of the launches too: with a counter each, the n-th row-scaled launch found its flags already set by the n-th
+    # block-scaled one, and a block could take over accumulators that its predecessor had not written yet.
+    M, N, K = 2560, 7680, 384   # 3 slabs per tile, 3.5 per block: the hand-over comes early in every block
+    cases = []
+    for kind in ("block", "row"):
+        if kind == "block":
+            a, b, sa, sb = make_block(M, N, K, seed=11)
+            cfg = BLK
+        else:
+            a, b = synth.random_fp8((M, K), 5), synth.random_fp8((N, K), 6)
+            sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+            cfg = ROW
+        ops = [t.to(dev) for t in (a, b, sa, sb)]
+        cases.append((kind, cfg, ops))
+    run = lambda cfg, ops: mx.dynamic_scaled_matmul(*ops, cfg.input_scale, cfg.weight_scale, out_type=torch.bfloat16, algo="tiled")
+    tune(MAXFP8_TILE="1", MAXFP8_STREAMK="0", MAXFP8_PERSIST="0")
+    want = {kind: run(cfg, ops) for kind, cfg, ops in cases}
+    tune(MAXFP8_TILE="1", MAXFP8_STREAMK="2")
+    for it in range(40):
+        for kind, cfg, ops in cases:
+            got = run(cfg, ops)
+            assert torch.equal(got.view(torch.int16), want[kind].view(torch.int16)), f"{kind}, launch {it}"
+
+
 def test_stream_k_exact(dev, tune):
     tune(MAXFP8_TILE="1", MAXFP8_STREAMK="2")
     M, N, K = 2560, 7680, 640
