@@ -82,23 +82,24 @@ __device__ __forceinline__ void buffer_store_b128_guarded(const v4u_t v, const _
 }
 
 // The activation scales of a slab in LDS.  The copy puts its lanes' values at consecutive words, and a lane may fetch
-// any row: word i of the scale area gets the row that makes the TM scales a lane needs in the main loop -- rows lm,
-// lm + 16, ... of its wave's WM = 16 * TM rows -- neighbours (word wm * WM + lm * TM + mt), so that they come back in one
-// or two wide LDS reads instead of TM narrow ones.
+// any row: word i of the scale area gets the row that puts the TM scales a lane needs in the main loop -- rows lm,
+// lm + 16, ... of its wave's WM = 16 * TM rows -- four by four at neighbouring words (word wm * WM + (mt / 4) * 64 +
+// lm * 4 + mt % 4: the 16 lane rows of a read cover 256 consecutive bytes, every bank once), so that they come back in
+// one or two 16-byte LDS reads instead of TM narrow ones.
 // (Wave tiles whose TM is not a multiple of 4 keep the rows in order: their scales would come back in reads that
 // straddle 16-byte boundaries, which measured a quarter slower than narrow reads on the 192-row tiles.)
 template <int WM>
 __device__ __forceinline__ int scale_word_row(int i) {
   constexpr int TM = WM / 16;
   if constexpr (TM % 4 != 0) return i;
-  const int in_wave = i % WM;
-  return (i / WM) * WM + (in_wave % TM) * 16 + in_wave / TM;
+  const int in_wave = i % WM, mt = (in_wave / 64) * 4 + in_wave % 4, lm = (in_wave % 64) / 4;
+  return (i / WM) * WM + mt * 16 + lm;
 }
 
 // byte offset, in a stage's scale area, of the first scale of lane row lm of a wave whose rows begin at wave_row0
 template <int TM>
 __device__ __forceinline__ uint32_t scale_read_offset(int wave_row0, int lm) {
-  return (uint32_t)(wave_row0 + (TM % 4 == 0 ? lm * TM : lm)) * 4u;
+  return (uint32_t)(wave_row0 + (TM % 4 == 0 ? lm * 4 : lm)) * 4u;
 }
 // a lane's TM scales: 16-byte reads of neighbouring words where TM allows, else one word per 16-row group
 template <int TM>
@@ -109,7 +110,7 @@ __device__ __forceinline__ ScaleRow<TM> read_scales(const uint8_t* at) {
   if constexpr (TM % 4 == 0) {
 #pragma unroll
     for (int i = 0; i < TM / 4; ++i) {
-      const v4f q = *reinterpret_cast<const v4f*>(at + i * 16);
+      const v4f q = *reinterpret_cast<const v4f*>(at + i * 256);
       out.v[4 * i] = q[0]; out.v[4 * i + 1] = q[1]; out.v[4 * i + 2] = q[2]; out.v[4 * i + 3] = q[3];
     }
   } else {
