@@ -45,9 +45,12 @@
  * Parity unpinned (no fixture, closed form or reference test fixes them):
  *   - NaN/Inf *inputs* to the quantiser (propagation through the reference's
  *     max-reduction is not visible in its sources);
- *   - bf16 *scales* dtype: the quotient is formed in f32 and rounded once more to
- *     bf16 here; whether the reference divides in bf16 with a single rounding is
- *     not visible in its sources (its tests only use values where both agree);
+ *   - bf16 *scales* whose quotient amax / 448 is below the normal range (the quotient
+ *     is formed in f32 and rounded once more to bf16 here; in the normal range that is
+ *     the correctly rounded bf16 quotient whichever way a compiler lowers the division --
+ *     for 8-bit significands a 24-bit intermediate makes the second rounding harmless --
+ *     and tests/test_oracle_quant.py checks every such amax against exact rational
+ *     arithmetic; below it the result hangs on the denormal mode of the division);
  *   - orc_rms_norm_fused_quantize beyond the reference test's own data: the order of the
  *     sum of squares and the rsqrt are not fixed by the reference (see the function);
  *   - orc_fused_silu in the last bit of exp() (see the function).

@@ -84,6 +84,24 @@ def test_every_bf16_amax_divides_exactly(dev):
     check(xb.contiguous(), ROW, dev, -1)
 
 
+def test_every_bf16_amax_with_bf16_scales(dev):
+    # the same, scales of dtype bf16 (the reference wrapper's default, nn/kernels.py:6883): scale bits and bytes
+    vals = (np.arange(1, 0x7F80, dtype=np.uint32) << 16).view(np.float32)
+    n = vals.size
+    x = np.zeros((n, 128), dtype=np.float32)
+    x[:, 3] = vals
+    x[:, 77] = -vals * 0.37
+    pad = (-n) % 3
+    x = np.concatenate([x, np.zeros((pad, 128), dtype=np.float32)])
+    xb = torch.from_numpy(x).to(torch.bfloat16).reshape(-1, 128 * 3).contiguous()
+    M = xb.shape[0]
+    for cfg, G in ((BLK, 128), (ROW, 384)):
+        q, s = gpu_quant(xb.to(dev), cfg, scales_type=torch.bfloat16)
+        q_ref, s_ref = oracle.quantize_dynamic_scaled_fp8(bf16_bits(xb), G, scales_dtype=oracle.BF16, threads=NT)
+        assert np.array_equal(bf16_bits(s)[:, :M], s_ref), "scales differ"
+        assert np.array_equal(fp8_bytes(q), q_ref), "quantized bytes differ"
+
+
 def test_near_zero_and_zero_groups(dev):
     # test_scaled_fp8_quantization.mojo:421-512
     x = torch.full((4, 512), 1e-38, dtype=torch.float32).to(torch.bfloat16)

@@ -136,3 +136,44 @@ def test_f32_and_f16_inputs_and_bf16_scales():
     row[0, 0] = 448.0 * 2
     qb, sb = oracle.quantize_dynamic_scaled_fp8(bf16_bits(row.to(torch.bfloat16)), 128, scales_dtype=oracle.BF16)
     assert oracle.bf16_bits_to_f32(sb)[0, 0] == 2.0 and qb[0, 0] == 0x7E
+
+
+def _rne_bf16(v):
+    """Fraction -> the nearest bf16 value (ties to even) as a Fraction; normal range only."""
+    from fractions import Fraction
+    e = v.numerator.bit_length() - v.denominator.bit_length()
+    if Fraction(2) ** e > v:
+        e -= 1
+    assert Fraction(2) ** e <= v < Fraction(2) ** (e + 1) and e >= -126
+    step = Fraction(2) ** (e - 7)
+    q = v / step
+    n = q.numerator // q.denominator
+    rem = q - n
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+        n += 1
+    return n * step
+
+
+def test_bf16_scales_are_the_correctly_rounded_quotient():
+    # Scales of dtype bf16 are bf16(min(amax, ub)) / bf16(448), one division rounded to bf16 (fp8_utils.mojo:24-60 with the
+    # scales dtype as its type).  A compiler may divide in f32 and round the f32 quotient to bf16 instead: for operands of
+    # 8 significant bits the two are the same number (an intermediate of at least 2 * 8 + 2 bits makes the second rounding
+    # harmless), so exact rational arithmetic pins the value whichever way the reference's compiler lowers it.  Every
+    # positive bf16 amax whose quotient is a normal number.
+    from fractions import Fraction
+    vals = (np.arange(1, 0x7F80, dtype=np.uint32) << 16).view(np.float32)
+    vals = vals[vals >= np.float32(448.0 * 2.0 ** -126)]
+    x = np.zeros((vals.size, 128), dtype=np.float32)
+    x[:, 5] = -vals
+    x[:, 90] = vals * 0.5
+    q, sc = oracle.quantize_dynamic_scaled_fp8(oracle.bf16_bits_of(x), 128, scales_dtype=oracle.BF16)
+    got = oracle.bf16_bits_to_f32(sc)[0, :vals.size]
+    for i in range(0, vals.size, 1):
+        a = Fraction(float(vals[i]))
+        want = _rne_bf16(min(a, Fraction(1200)) / 448)
+        assert Fraction(float(got[i])) == want, (i, float(vals[i]), float(got[i]), float(want))
+    # and the bytes follow from the f32 value of that scale: x * (1 / scale), both in f32
+    s32 = got.astype(np.float32)
+    recip = np.float32(1.0) / s32
+    want_q = oracle.e4m3fn_encode((x * recip[:, None]).astype(np.float32))
+    assert np.array_equal(q, want_q)
