@@ -103,3 +103,31 @@ def test_errors(dev):
         f(a.to(dev), b.to(dev), sa.to(dev), sb.to(dev), off.to(dev), ids.to(dev).long(), stats)
     none = torch.tensor([0, 0], dtype=torch.int64).to(torch.uint32)
     assert f(a.to(dev), b.to(dev), sa.to(dev), sb.to(dev), off.to(dev), ids.to(dev), none).shape == (8, 128)
+
+
+def test_block_and_row_scaled_launches_in_flight_together(dev):
+    """Two streams, one sending block-scaled and one row-scaled grouped matmuls, both busy at the same time: the
+    launches take their tile counters from one pool in device memory, so no two launches in flight may be handed the
+    same set.  Every result equals the one the same call gives alone."""
+    import test_gpu_grouped as blk
+    counts, ids, E, N, K = [300, 1100, 2, 40, 0, 600, 31, 129], [5, 0, 2, 1, 3, 4, 6, 7], 8, 640, 1024
+    stats = torch.tensor([max(counts), len(counts)], dtype=torch.int64).to(torch.uint32)
+    ops_b = [t.to(dev) for t in blk.make(counts, ids, E, N, K, seed=21)]
+    ops_r = [t.to(dev) for t in make(counts, ids, E, N, K, seed=22)]
+    call_b = lambda: mx.grouped_dynamic_scaled_fp8_matmul(*ops_b, stats, blk.BLK.input_scale, blk.BLK.weight_scale,
+                                                          out_type=torch.bfloat16)
+    call_r = lambda: mx.grouped_matmul_rowwise_dynamic_scaled_fp8(*ops_r, stats, out_type=torch.bfloat16)
+    want_b, want_r = call_b(), call_r()
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got_b, got_r = [], []
+    for _ in range(12):
+        with torch.cuda.stream(s1):
+            got_b.append(call_b())
+        with torch.cuda.stream(s2):
+            got_r.append(call_r())
+    torch.cuda.synchronize()
+    live = sum(counts)
+    for i, (gb, gr) in enumerate(zip(got_b, got_r)):
+        assert torch.equal(gb[:live], want_b[:live]), f"block-scaled launch {i}"
+        assert torch.equal(gr[:live], want_r[:live]), f"row-scaled launch {i}"
