@@ -127,7 +127,7 @@ __device__ __forceinline__ ScaleRow<TM> read_scales(const uint8_t* at) {
 // One BM x BN tile of C: rows [row_begin, row_end) (at most BM of them are used) by columns
 // [n0, n0 + BN) of the weight matrix at bptr / scales at bs_ptr.  Called by every thread of a
 // block of WAVES_M * WAVES_N waves with `smem` = the block's dynamic LDS.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED, bool KV = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool GROUPED, bool KV = false, int B_POLICY = 0>
 __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, const int64_t row_begin, const int64_t row_end,
                                           const int n0, const uint8_t* bptr, const float* bs_ptr) {
   constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -236,7 +236,7 @@ __device__ __forceinline__ void tile_body(const GemmArgs& p, uint8_t* smem, cons
     } else if (idx < IA + IB) {
       const int i = idx - IA;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(sb + i * NWAVES * 1024), 16, b_voff | kill_b,
-                                               koff + i * b_istep, 0, 0);
+                                               koff + i * b_istep, 0, B_POLICY);
     } else if constexpr (BLOCKSCALE) {
       // 64 scales of the slab's row of the transposed scale matrix per wave; with more waves
       // than 64-row chunks the extra waves repeat a chunk (same bytes to the same place), so
@@ -636,7 +636,8 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
   tn = in_group / gsize;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool KV = false>
+// B_STREAM: the matmul is one row of tiles, so every weight byte is read once: the weight copies are marked non-temporal
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool KV = false, bool B_STREAM = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   // ---- block -> tile: XCD de-interleave, then groups of GROUP_M row tiles share weight columns
@@ -651,7 +652,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
   int tm, tn;
   tile_coords(pid, tiles_m, tiles_n, tm, tn);
   const GemmArgs q = gridDim.z == 1 ? p : batch_view(p, blockIdx.z);
-  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false, KV>(q, smem, (int64_t)tm * BM, q.M, tn * BN, q.b, q.b_scales);
+  tile_body<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, false, KV, B_STREAM ? kStreamOnce : 0>(q, smem, (int64_t)tm * BM, q.M, tn * BN, q.b,
+                                                                                              q.b_scales);
 }
 
 // ---- persistent variant ------------------------------------------------------------------------
@@ -1939,6 +1941,14 @@ static int launch_tiled(const GemmArgs& p, dim3 grid, hipStream_t stream, const 
   static PerDeviceFlag attr_done;
   // (fused QKV: 8 more bytes per tile row for the rows' cache offsets, after the 2 * BM * BN bytes of staged output)
   constexpr int stages = tile_lds_bytes<BM, BN, NS, BLOCKSCALE>(), kv = 2 * BM * BN + 8 * BM * WAVES_N;
+  if constexpr (!KV) {
+    // one row of tiles (and one matrix): every weight byte is read once
+    if (p.M <= BM && grid.z == 1) {
+      static PerDeviceFlag attr_done_stream;
+      return launch_with_lds(gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, KV, true>, attr_done_stream, stages,
+                             WAVES_M * WAVES_N * 64, p, grid, stream, name);
+    }
+  }
   return launch_with_lds(gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, NS, BLOCKSCALE, KV>, attr_done,
                          KV && kv > stages ? kv : stages, WAVES_M * WAVES_N * 64, p, grid, stream, name);
 }
