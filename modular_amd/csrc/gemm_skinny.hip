@@ -378,11 +378,13 @@ static int skinny_shape(int64_t M, int64_t N, int64_t K) {
     if (ntw == 4 && K < 4096) break;
     const int64_t blocks = ceil_div(N, 16 * ntw);
     float cost = (float)ceil_div(blocks, cus) * (float)(16 * ntw + M + 8);
-    if (ntw == 4) cost *= 1.25f;
+    if (ntw == 4) cost *= K >= 8192 ? 1.25f : 1.35f;  // (one block per CU: its start and end weigh more the shorter K is)
     if (ntw == 1 || cost < best_cost) { best = ntw; best_cost = cost; }
   }
+  // (16 KB rings for 32-row blocks -- the selector 2416 -- were ahead on the largest matrices while the chip read 6.2
+  // TB/s; with the weight copies marked non-temporal 8 KB rings are: 68.6 against 72.2 us on 57344 x 8192 at M = 1)
   if (best == 4) return 4432;
-  if (best == 2) return (M <= 16 && N >= 16384 && N * K >= ((int64_t)1 << 28)) ? 2416 : 2408;
+  if (best == 2) return 2408;
   return 1408;
 }
 
