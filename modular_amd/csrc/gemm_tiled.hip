@@ -1907,10 +1907,11 @@ __global__ __launch_bounds__(512, 1) void gemm_grouped_persist_kernel(GemmArgs p
       tile_body<256, 256, 2, 4, 2, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
     } else if (kind == 1) {
       // (a rest of at most 192 rows: three quarters of the MFMAs)
-      if (rows_here <= 192) tile_body<192, 128, 2, 4, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
-      else tile_body<256, 128, 4, 2, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+      // (a slot's rest is one row tile: its weights are read once, as the S tiles' are)
+      if (rows_here <= 192) tile_body<192, 128, 2, 4, 3, BLOCKSCALE, true, false, kStreamOnce>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+      else tile_body<256, 128, 4, 2, 3, BLOCKSCALE, true, false, kStreamOnce>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
     } else if (kind == 2) {
-      tile_body<128, 256, 2, 4, 3, BLOCKSCALE, true>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
+      tile_body<128, 256, 2, 4, 3, BLOCKSCALE, true, false, kStreamOnce>(p, smem, row_begin, row_end, n0, bptr, bs_ptr);
     } else {
       if (rows_here <= 16) grouped_stream_body<1, 4, 2, BLOCKSCALE>(p, smem, row_begin, rows_here, n0, bptr, bs_ptr);
       else grouped_stream_body<2, 4, 2, BLOCKSCALE>(p, smem, row_begin, rows_here, n0, bptr, bs_ptr);
