@@ -55,7 +55,7 @@ __device__ __forceinline__ uint32_t sk_clamp_u32(int64_t v) {
 // ALDS: the activations of a wave's share of K are copied to LDS once, before the loop (at most kSkinnyALdsBytes per
 // wave), instead of two loads per slab and 16-token group: on a launch that is a single round of blocks those loads
 // are half of the loop's vector-memory instructions and cost 8 % of the kernel, whatever they fetch.
-constexpr int kSkinnyALdsBytes = 4096;
+constexpr int kSkinnyALdsBytes = 8192;
 template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES, bool ALDS = false>
 struct SkinnyCfg {
   static constexpr int WAVES = NWAVES;
@@ -324,6 +324,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_skinny_kernel(GemmArgs p_in)
   }
 }
 
+int compute_units();
 template <int NTW, int MT, bool BLOCKSCALE, int RING_KB, int NWAVES, bool ALDS = false>
 static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream) {
   if constexpr (MT == 1 && !ALDS) {
@@ -331,9 +332,15 @@ static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream)
     // blocks: the activations go to LDS once (84 MB, M = 1: 17.8 -> 17.0 us; on a 470 MB matrix, where blocks come and
     // go, the per-slab loads cost nothing and this form measured 1 % slower).  Not for the fused QKV epilogue's build, a
     // rare caller at these sizes, to keep the number of kernels down.
+    // The extra LDS must not cost a resident block: all blocks of such a launch sit on the chip at once, and a CU's share
+    // of them has to fit its 160 KB with the activations added (10240 x 8192 at M = 2: 18.3 -> 16.6 us; at M = 4, where
+    // a CU's three blocks would need 192 KB: 18.5 -> 20.2, so that case keeps the per-slab loads).
     const int64_t per_wave = ceil_div(ceil_div(p.K, 128), NWAVES);
-    if (tuning().skinny_alds && !p.kv_on && (int64_t)p.N * p.K < ((int64_t)1 << 27) &&
-        (int64_t)p.M * ((per_wave * 128 + 1023) / 1024 * 1024) <= kSkinnyALdsBytes)
+    const int64_t a_bytes = (int64_t)p.M * ((per_wave * 128 + 1023) / 1024 * 1024);  // per wave
+    const int64_t blocks_per_cu = ceil_div(ceil_div((int64_t)p.N, 16 * NTW) * batch, (int64_t)compute_units());
+    using Plain = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES, false>;
+    if (tuning().skinny_alds && !p.kv_on && (int64_t)p.N * p.K < ((int64_t)1 << 27) && a_bytes <= kSkinnyALdsBytes &&
+        blocks_per_cu * (Plain::SMEM + NWAVES * a_bytes) <= 160 * 1024)
       return launch_skinny_r<NTW, MT, BLOCKSCALE, RING_KB, NWAVES, true>(p, batch, stream);
   }
   using Cfg = SkinnyCfg<NTW, MT, BLOCKSCALE, RING_KB, NWAVES, ALDS>;
