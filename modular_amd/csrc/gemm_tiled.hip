@@ -1836,26 +1836,44 @@ __global__ __launch_bounds__(512, 1) void gemm_grouped_persist_kernel(GemmArgs p
   kernarg_ptr_t pk = (kernarg_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();  // (the argument block is the first argument)
   while (true) {
     __syncthreads();  // every wave is done with the last tile's LDS and with the claim; the first time: the tables are there
-    if (tid == 0) {
+    if (tid < 64) {
       // Column tile c of every kind belongs to XCD c % 8 (blocks go to the XCDs round-robin): the weight tiles an XCD
       // works on stay in its L2 from one row tile to the next, and the eight XCDs read an activation row tile at about
       // the same time.  One counter per kind and XCD; a block whose own XCD has nothing left of a kind helps the others
-      // before it moves on to the next kind.  `step` only grows: every (kind, XCD) pair is tried until it is empty, once.
+      // before it moves on to the next kind.  `step` only grows: the 32 (kind, XCD) pairs come in this block's order.
+      // A claim that comes back empty costs a trip to memory (the counters are shared by the eight L2s), and by the
+      // end every pair is empty: after the first empty claim the wave reads all 32 counters at once, lane l that of
+      // pair l, and goes straight to the next pair that still had tiles -- one trip instead of one per empty pair
+      // (a launch of one L tile per CU spent 21 of its 45 us on the seven empty claims at its end).
       unsigned int* ctr = g_grouped_ctr + ctr_slot * kGroupedCtrStride;
       const int my_xcd = (int)(blockIdx.x & 7);
+      const int sfirst = s_sfirst;
+      auto pair_of = [&](int st, int& k, int& x, int& total) {
+        k = sfirst ? 3 - (st >> 3) : (st >> 3);
+        x = (my_xcd + (st & 7)) & 7;
+        const int cols_x = x < s_ncol[k] ? (s_ncol[k] - x + 7) >> 3 : 0;
+        total = s_rt[k] * cols_x;
+      };
       int kind = -1, t = 0, xcd = 0, step = s_step;
       while (step < 32) {
-        const int k = s_sfirst ? 3 - (step >> 3) : (step >> 3);
-        const int x = (my_xcd + (step & 7)) & 7;
-        const int cols_x = x < s_ncol[k] ? (s_ncol[k] - x + 7) >> 3 : 0;
-        const int total = s_rt[k] * cols_x;
+        int k, x, total;
+        pair_of(step, k, x, total);
         if (total > 0) {
-          t = (int)atomicAdd(ctr + k * 8 + x, 1u);
+          if (tid == 0) t = (int)atomicAdd(ctr + k * 8 + x, 1u);
+          t = __builtin_amdgcn_readfirstlane(t);
           if (t < total) { kind = k; xcd = x; break; }
+          int kl, xl, total_l, pair_l = tid & 31;
+          asm volatile("" : "+v"(pair_l));  // (worked out here, where it is needed: not kept in registers across the tile bodies)
+          pair_of(pair_l, kl, xl, total_l);
+          unsigned int seen = 0xffffffffu;
+          if (tid < 32 && tid > step && total_l > 0) seen = __hip_atomic_load(ctr + kl * 8 + xl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const unsigned long long open = __ballot(seen < (unsigned int)total_l);
+          step = open ? __builtin_ctzll(open) : 32;
+        } else {
+          ++step;
         }
-        ++step;
       }
-      s_step = step; s_kind = kind; s_t = t; s_xcd = xcd;
+      if (tid == 0) { s_step = step; s_kind = kind; s_t = t; s_xcd = xcd; }
     }
     __syncthreads();
     const int kind = s_kind, t = s_t, xcd = s_xcd;
