@@ -238,6 +238,55 @@ def run_gpu(name, steps, warmup, settle_s=None):
     return wl, ms_step, mm_avg, mm_ms[len(mm_ms) // 2], mm_ms[0]
 
 
+def config_cells():
+    """Every cell of BASELINE.json's configs[1..3]: name -> (kind, M, K, N)."""
+    cells = {}
+    for proj, (K, N) in (("qkv", (4096, 6144)), ("o_proj", (4096, 4096)), ("gate_up", (4096, 28672)), ("down", (14336, 4096))):
+        for M in (1, 16, 128, 2048):
+            cells[f"llama8b_{proj}_m{M}"] = ("block", M, K, N)
+    for proj, (K, N) in (("q_a", (7168, 1536)), ("q_b", (1536, 24576)), ("kv_a", (7168, 576)), ("kv_b", (512, 32768)),
+                         ("o_proj", (16384, 7168))):
+        for M in (256, 1024, 4096):
+            cells[f"dsv3_{proj}_m{M}"] = ("block", M, K, N)
+    for proj, (K, N) in (("qkv", (8192, 10240)), ("gate_up", (8192, 57344)), ("down", (28672, 8192))):
+        for M in (1, 2, 4, 8):
+            cells[f"decode70b_{proj}_m{M}"] = ("row", M, K, N)
+    return cells
+
+
+def graph_time_ms(wl, launches):
+    """Milliseconds per matmul when `launches` of them (rotating over the operand copies) replay from one HIP graph:
+    the launch-to-launch interval on the GPU with no host in between, which is what a kernel of a few microseconds
+    needs to be timed at all (a call through the Python wrappers takes longer than such a kernel runs)."""
+    import torch
+
+    quantised = [wl.quantise(c) for c in range(wl.copies)]
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(3):
+            wl.matmul(i % wl.copies, *quantised[i % wl.copies])
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(launches):
+                wl.matmul(i % wl.copies, *quantised[i % wl.copies])
+    torch.cuda.current_stream().wait_stream(side)
+    t_end = time.perf_counter() + SETTLE_S
+    while time.perf_counter() < t_end:
+        graph.replay()
+        torch.cuda.synchronize()
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    times = []
+    for _ in range(5):
+        first.record()
+        graph.replay()
+        last.record()
+        torch.cuda.synchronize()
+        times.append(first.elapsed_time(last) / launches)
+    return sorted(times)[len(times) // 2]
+
+
 def read_ceiling(wl, steps):
     """Average time of the decode matmul's read-only probe (the same grid, LDS ring and DMA instructions streaming
     the same weight copies, nothing else) over `steps` back-to-back launches, in milliseconds."""
@@ -416,6 +465,9 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB three times (the known-size unit that "
                          "hardware byte counters of a rocprofv3 --pmc run are scaled by)")
+    ap.add_argument("--cells", action="store_true",
+                    help="every cell of configs[1..3] (each projection at each M): the matmul's time per launch when 100 "
+                         "launches replay from one HIP graph, against the roof that binds it; one JSON line each")
     ap.add_argument("--read-ceiling", action="store_true",
                     help="for every decode workload (M <= 16): the matmul kernel's time beside the time of its read-only "
                          "probe (same grid and weight traffic, no arithmetic), one JSON line each")
@@ -442,6 +494,24 @@ def main():
                   file=sys.stderr, flush=True)
             with open(os.path.join(ROOT, RESULTS_DIR, "bench_table.json"), "w") as f:
                 json.dump(rows, f, indent=1)
+            torch.cuda.empty_cache()
+        return
+    if args.cells:
+        from modular_amd import _lib
+        for name, cell in config_cells().items():
+            WORKLOADS[name] = cell
+            wl = Workload(name, torch.device("cuda:0"))
+            ms = graph_time_ms(wl, 100)
+            kind, M, K, N = cell
+            flops, mm_bytes, _ = algorithmic(kind, M, K, N)
+            hbm_bound = mm_bytes / (PEAK_HBM_GBS * 1e9) > flops / (PEAK_FP8_TFLOPS * 1e12)
+            achieved = mm_bytes / (ms * 1e-3) / 1e9 if hbm_bound else flops / (ms * 1e-3) / 1e12
+            print(json.dumps({"cell": name, "scaling": kind, "M": M, "K": K, "N": N, "us_per_launch": round(ms * 1e3, 2),
+                              "bound": "hbm" if hbm_bound else "mfma", "achieved": round(achieved, 1),
+                              "unit": "GB/s" if hbm_bound else "TFLOP/s",
+                              "frac": round(achieved / (PEAK_HBM_GBS if hbm_bound else PEAK_FP8_TFLOPS), 3),
+                              "launches": _lib.matmul_describe(M, N, K, kind == "block", True)}), flush=True)
+            del wl
             torch.cuda.empty_cache()
         return
     if args.read_ceiling:

@@ -2360,10 +2360,23 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
   return snprintf(buf, len, "%dx%d x%lld%s", t.bm, t.bn, count(M, N, t), how(M, N, plan.variant));
 }
 
+// A launch recorded into a HIP graph replays with the arguments of the recording.  The work-split kernel's flag value
+// would then repeat: a replay would find the flags of the replay before it already set, and a block could take over
+// accumulators its predecessor has not written yet.  Such a launch runs as the persistent kernel instead, which forms the
+// same sums in the same order.  (The grouped kernel's counters are put back to zero by the launch itself and replay as they are.)
+static bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
 int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_bytes, int64_t batch, hipStream_t stream) {
   GemmArgs p = p_in;
   const TiledPlan plan = cached_plan(p.M, p.N, p.K, blockscale, p.workspace != nullptr, workspace_bytes, batch, p.kv_on != 0);
-  if (plan.streamk) {
+  if (plan.streamk && !stream_is_capturing(stream)) {
     p.splits = 1;
     // (the plan knows the shape; whether this call's pointers and strides suit the persistent kernels is checked here)
     if (persist_ok(p, blockscale, dim3(1, 1, 1)))

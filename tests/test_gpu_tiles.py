@@ -331,6 +331,35 @@ def test_stream_k_scale_modes_take_turns(dev, tune):
             assert torch.equal(got.view(torch.int16), want[kind].view(torch.int16)), f"{kind}, launch {it}"
 
 
+def test_stream_k_shape_recorded_into_a_graph(dev, tune):
+    # A recorded launch replays with the arguments of the recording, so the work-split kernel's flag value would repeat
+    # and a replay would find its flags already set: under stream capture such a matmul runs as the persistent kernel
+    # (the same sums in the same order).  Four replays, each on new activations, each against the eager result.
+    M, N, K = 2560, 7680, 384
+    a, b, sa, sb = make_block(M, N, K, seed=21)
+    ad, bd, sad, sbd = a.to(dev), b.to(dev), sa.to(dev), sb.to(dev)
+    run = lambda: mx.dynamic_scaled_matmul(ad, bd, sad, sbd, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
+    tune(MAXFP8_TILE="1", MAXFP8_STREAMK="2")
+    assert "stream-K" in _lib.matmul_describe(M, N, K, True, True)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            out = run()
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in range(4):
+        ad.copy_(synth.random_fp8((M, K), 100 + seed).to(dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = run()     # eager: the work-split kernel itself
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"replay {seed}"
+
+
 def test_stream_k_exact(dev, tune):
     tune(MAXFP8_TILE="1", MAXFP8_STREAMK="2")
     M, N, K = 2560, 7680, 640
