@@ -31,6 +31,22 @@ def test_create_indices(dev, n, num_experts, dtype):
         assert np.array_equal(g, w)
 
 
+@pytest.mark.parametrize("shift", [1, 2, 3])
+def test_create_indices_of_ids_that_are_not_16_byte_aligned(dev, shift):
+    # the kernels read four ids per load where the pointer allows it and one per load where it does not
+    n, num_experts = 4099, 64
+    rng = np.random.default_rng(shift)
+    ids = rng.integers(0, num_experts, n + shift).astype(np.int32)
+    view = torch.from_numpy(ids).to(dev)[shift:]
+    assert view.data_ptr() % 16 == 4 * shift
+    outs = mx.moe_create_indices(view, num_experts)
+    torch.cuda.synchronize()
+    got = [o.cpu().view(torch.int32).numpy().view(np.uint32 if o.dtype == torch.uint32 else np.int32) for o in outs]
+    want = oracle.moe_create_indices(ids[shift:], num_experts)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+
+
 def test_create_indices_config_routing_feeds_the_grouped_matmul(dev):
     # BASELINE's MoE routing, then a grouped matmul on the gathered rows: same result as on the
     # host-sorted routing
