@@ -173,39 +173,65 @@ int moe_create_indices_dispatch(uint32_t* token_expert_order, uint32_t* expert_s
 }
 
 // ---- fused SiLU(gate) * up --------------------------------------------------------------------
-// a / b, correctly rounded (the IEEE quotient), at well under the cost of the IEEE sequence on the common path:
-// the hardware reciprocal and one correction step give a candidate q; its residual a - q * b is exact whenever q
-// is within an ulp of the quotient (and large otherwise), so
-//     residual == 0                        q is the exact quotient
-//     |residual| < ulp(q) / 2 * |b|        q is the one float nearest to a / b
-// accept q, and everything else -- ties, powers of two (whose lower neighbour is half an ulp away), tiny or huge
-// operands where the products above could underflow -- takes the IEEE division.  The slow path is a wave-uniform
-// branch: it is skipped unless some lane of the wave needs it.  (Checked against the IEEE quotient on 2e8 random
-// operand pairs with the reciprocal off by -1, 0 and +1 ulp: no difference.)
-__device__ __forceinline__ float exact_div(float a, float b, float rcp_b) {
-  float q = a * rcp_b;
-  const float err = fmaf(-q, b, a);
-  q = err == 0.0f ? q : fmaf(err, rcp_b, q);  // (keeps the sign of a zero quotient)
-  const float res = fmaf(-q, b, a);
-  const uint32_t qb = __float_as_uint(q), qe = qb & 0x7f800000u;
-  const uint32_t ae = __float_as_uint(a) & 0x7f800000u, be = __float_as_uint(b) & 0x7f800000u;
-  const float half_ulp_b = __uint_as_float(qe - (24u << 23)) * fabsf(b);
-  // (exponents between 2^-63 and 2^63: neither the residual nor the bound can underflow or overflow)
-  const bool b_ok = be >= (64u << 23) && be <= (190u << 23);
-  const bool aq_ok = ae >= (64u << 23) && qe >= (64u << 23) && qe <= (190u << 23);
-  const bool ok = b_ok && (a == 0.0f || (aq_ok && (res == 0.0f || ((qb & 0x007fffffu) != 0u && fabsf(res) < half_ulp_b))));
-  if (__builtin_amdgcn_ballot_w64(!ok) != 0ull) {
-    if (!ok) q = a / b;
+// a / b, correctly rounded (the IEEE quotient), at a third of the IEEE sequence's cost on the common path.  One Newton
+// step turns the hardware's reciprocal (within an ulp) into the correctly rounded one -- unless b's mantissa is all ones --
+// and with that, a quotient estimate, its exact residual and one correction give the correctly rounded quotient
+// (Markstein's sequence) as long as no product underflows or overflows.  Everything outside those conditions takes the
+// IEEE division, in a branch the wave skips unless one of its lanes needs it.  (Checked on the CPU against the IEEE
+// quotient: the same operations and acceptance tests on 1.8e9 operand pairs -- random, bf16 numerators, divisors whose
+// mantissa is (nearly) all ones, zeros and tiny numerators, quotients of the quantiser's size -- with the reciprocal
+// off by -1, 0 and +1 ulp: no difference.)
+__device__ __forceinline__ float refined_rcp(float b) {
+  const float y0 = __builtin_amdgcn_rcpf(b);
+  return fmaf(fmaf(-b, y0, 1.0f), y0, y0);
+}
+// a / b given y = refined_rcp(b); to be trusted where div_b_ok(b) and div_q_ok(a, result)
+__device__ __forceinline__ float div_by(float a, float b, float y) {
+  const float q0 = a * y;
+  const float q = fmaf(fmaf(-b, q0, a), y, q0);
+  return a == 0.0f ? q0 : q;  // (keeps the sign of a zero quotient)
+}
+__device__ __forceinline__ bool div_b_ok(float b) {
+  return b >= 0x1p-63f && b < 0x1p64f && (__float_as_uint(b) & 0x007fffffu) != 0x007fffffu;
+}
+__device__ __forceinline__ bool div_q_ok(float a, float q) {
+  return a == 0.0f || (fabsf(a) >= 0x1p-63f && fabsf(q) >= 0x1p-63f && fabsf(q) < 0x1p64f);
+}
+// Eight quotients a[j] / b[j] (SHARED: one divisor b[0] for all) with one test for the lane and one branch for the wave
+template <bool SHARED>
+__device__ __forceinline__ void exact_div8(const float (&a)[8], const float (&b)[8], float (&q)[8]) {
+  bool ok = true;
+  float y = 0.f;
+  if constexpr (SHARED) {
+    y = refined_rcp(b[0]);
+    ok = div_b_ok(b[0]);
   }
-  return q;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if constexpr (!SHARED) {
+      y = refined_rcp(b[j]);
+      ok = ok && div_b_ok(b[j]);
+    }
+    q[j] = div_by(a[j], b[SHARED ? 0 : j], y);
+    ok = ok && div_q_ok(a[j], q[j]);
+  }
+  if (__builtin_amdgcn_ballot_w64(!ok) != 0ull) {
+    if (!ok) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q[j] = a[j] / b[SHARED ? 0 : j];
+    }
+  }
 }
 
-__device__ __forceinline__ float silu_mul(float gate, float up) {
-  // gate / (1 + exp(-gate)) * up, every step rounded to f32 (ep_comm.mojo:4494-4497)
-  const float d = 1.0f + expf(-gate);
-  // d = inf (gate < -88): gate / inf = -0, written out (a residual against inf is NaN)
-  const float sig = d > 3.0e38f ? -0.0f : exact_div(gate, d, __builtin_amdgcn_rcpf(d));
-  return sig * up;
+// gate / (1 + exp(-gate)) * up, every step rounded to f32 (ep_comm.mojo:4494-4497), for eight outputs.
+// (1 + exp(-gate) = inf, gate < -88: outside the fast division's range, and gate / inf = -0 is what the IEEE division gives)
+__device__ __forceinline__ void silu_mul8(const float (&gate)[8], const float (&up)[8], float (&f)[8]) {
+  float d[8], sig[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) d[j] = 1.0f + expf(-gate[j]);
+  exact_div8<false>(gate, d, sig);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) f[j] = sig[j] * up[j];
 }
 
 // 16 lanes own 128 consecutive outputs of one row (8 each): one 16-byte load of gate and of up
@@ -230,12 +256,15 @@ __global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__
     const uint4 gv = *reinterpret_cast<const uint4*>(src);
     const uint4 uv = *reinterpret_cast<const uint4*>(src + inter);
     const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
-    float f[8];
+    float gate[8], up[8], f[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      f[2 * j] = silu_mul(__uint_as_float(gw[j] << 16), __uint_as_float(uw[j] << 16));
-      f[2 * j + 1] = silu_mul(__uint_as_float(gw[j] & 0xffff0000u), __uint_as_float(uw[j] & 0xffff0000u));
+      gate[2 * j] = __uint_as_float(gw[j] << 16);
+      gate[2 * j + 1] = __uint_as_float(gw[j] & 0xffff0000u);
+      up[2 * j] = __uint_as_float(uw[j] << 16);
+      up[2 * j + 1] = __uint_as_float(uw[j] & 0xffff0000u);
     }
+    silu_mul8(gate, up, f);
     if constexpr (!QUANT) {
       uint32_t w[4];
 #pragma unroll
@@ -248,10 +277,11 @@ __global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__
       for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(f[j]));
       amax = row16_max(amax);
       const float scale = fmaxf(amax, 1e-4f) / 448.0f;
-      const float rs = __builtin_amdgcn_rcpf(scale);
+      const float divisor[8] = {scale, scale, scale, scale, scale, scale, scale, scale};
       float q[8];
+      exact_div8<true>(f, divisor, q);   // (one reciprocal and one test of the divisor for the lane's eight quotients)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) q[j] = clamp448(exact_div(f[j], scale, rs));
+      for (int j = 0; j < 8; ++j) q[j] = clamp448(q[j]);
       int lo = 0, hi = 0;
       lo = cvt_pk_e4m3fn(q[0], q[1], lo, false);
       lo = cvt_pk_e4m3fn(q[2], q[3], lo, true);
