@@ -488,7 +488,9 @@ int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M
   const unsigned nb = (unsigned)batch;
   const int64_t ngroups = K / G;
   const bool fast_types = in_dtype == MAXFP8_BF16 && scales_dtype == MAXFP8_F32;
-  const bool stream_in = M * K * 2 * batch >= kStreamInputBytes;
+  // (a row gather reads its source rows more than once -- the MoE layer each token's row top_k times, far apart in
+  // time -- and wants them kept in the memory-side cache)
+  const bool stream_in = M * K * 2 * batch >= kStreamInputBytes && row_index == nullptr;
   const bool vec_ok = aligned16(in) && (in_row_stride % 8 == 0) && (reinterpret_cast<uintptr_t>(out_fp8) % 8 == 0) &&
                       (out_row_stride % 8 == 0) && (in_batch_stride % 8 == 0) && (out_batch_stride % 8 == 0);
   if (fast_types && vec_ok && G == 128) {
