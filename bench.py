@@ -287,6 +287,43 @@ def graph_time_ms(wl, launches):
     return sorted(times)[len(times) // 2]
 
 
+def moe_layer_ms(steps, fuse):
+    """Milliseconds per call (host clock around `steps` calls, clocks settled) of the expert matmuls of a block-scaled FP8
+    MoE layer on BASELINE's configs[4] routing: 4096 tokens, top-8 of 256 experts (popularity ~ rank^-1.1), hidden 7168,
+    intermediate 2048 -- grouping, gathered quantise, grouped gate_up, silu(gate) * up, quantise, grouped down."""
+    import torch
+    import modular_amd as mx
+    from modular_amd import synth
+
+    dev = torch.device("cuda:0")
+    cfg = mx.blockwise_fp8_config()
+    seq, k, E, hidden, inter = 4096, 8, 256, 7168, 2048
+    x = synth.activations(seq, hidden, seed=1, device=dev)
+    g = torch.Generator().manual_seed(0)
+    perm = torch.randperm(E, generator=g)
+    rank = torch.empty(E)
+    rank[perm] = torch.arange(1, E + 1, dtype=torch.float32)
+    logits = torch.randn((seq, E), generator=g) - 1.1 * torch.log(rank)
+    router_idx = torch.topk(torch.softmax(logits, dim=-1), k, dim=-1).indices.to(torch.int32).to(dev)
+    wgu = synth.random_fp8((E, 2 * inter, hidden), 2, device=dev)
+    sgu = synth.random_scales((E, 2 * inter // 128, hidden // 128), 3, device=dev, lo=0.001, hi=0.01)
+    wd = synth.random_fp8((E, hidden, inter), 4, device=dev)
+    sd = synth.random_scales((E, hidden // 128, inter // 128), 5, device=dev, lo=0.001, hi=0.01)
+
+    def run():
+        return mx.expert_matmuls_fp8(x, router_idx, wgu, sgu, wd, sd, cfg, host_sync=False, fuse_activation_quant=fuse)
+
+    t_end = time.perf_counter() + max(SETTLE_S, 0.5)
+    while time.perf_counter() < t_end:
+        run()
+        torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
 def read_ceiling(wl, steps):
     """Average time of the decode matmul's read-only probe (the same grid, LDS ring and DMA instructions streaming
     the same weight copies, nothing else) over `steps` back-to-back launches, in milliseconds."""
@@ -468,6 +505,10 @@ def main():
     ap.add_argument("--cells", action="store_true",
                     help="every cell of configs[1..3] (each projection at each M): the matmul's time per launch when 100 "
                          "launches replay from one HIP graph, against the roof that binds it; one JSON line each")
+    ap.add_argument("--moe-layer", action="store_true",
+                    help="the expert matmuls of the FP8 MoE layer on configs[4]'s routing (grouping, gathered quantise, grouped "
+                         "gate_up, silu * up, quantise, grouped down): milliseconds per call, one JSON line for each way of the "
+                         "activation quantisation (two kernels, one kernel)")
     ap.add_argument("--read-ceiling", action="store_true",
                     help="for every decode workload (M <= 16): the matmul kernel's time beside the time of its read-only "
                          "probe (same grid and weight traffic, no arithmetic), one JSON line each")
@@ -512,6 +553,14 @@ def main():
                               "frac": round(achieved / (PEAK_HBM_GBS if hbm_bound else PEAK_FP8_TFLOPS), 3),
                               "launches": _lib.matmul_describe(M, N, K, kind == "block", True)}), flush=True)
             del wl
+            torch.cuda.empty_cache()
+        return
+    if args.moe_layer:
+        for fuse in (False, True):
+            ms = moe_layer_ms(args.steps, fuse)
+            print(json.dumps({"workload": "expert_matmuls_fp8: 4096 tokens x top-8 of 256 experts, hidden 7168, intermediate 2048",
+                              "fuse_activation_quant": fuse, "ms_per_call": round(ms, 4), "steps": args.steps,
+                              "timing": "host clock around the calls, no host synchronisation inside a call"}), flush=True)
             torch.cuda.empty_cache()
         return
     if args.read_ceiling:
