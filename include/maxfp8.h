@@ -114,6 +114,22 @@ int maxfp8_quantize_dynamic_scaled_fp8_gather(
     int in_dtype, int scales_dtype, float scale_ub, void* stream);
 
 /*
+ * The same fused input seen from the other side, for a gather whose source rows repeat: input row r
+ * is quantised once and written to the output rows dst_index[r * copies + j], j < copies (rows of
+ * out_fp8, columns of out_scales; a destination >= out_rows is skipped).  With dst_index the inverse
+ * of the gather's row_index it writes the same bytes as maxfp8_quantize_dynamic_scaled_fp8_gather:
+ * the MoE layer (max/python/max/nn/moe/moe_fp8.py:525-560) quantises each token once and stores it
+ * to its top_k sorted rows restore_token_order[token * top_k + j] instead of quantising it top_k
+ * times.  bfloat16 input, float32 scales, group_size 128, 16-byte aligned rows; anything else is an
+ * error that names the gather form.  dst_index is a device array of M * copies uint32.
+ */
+int maxfp8_quantize_dynamic_scaled_fp8_scatter(
+    void* out_fp8, void* out_scales, const void* in, const uint32_t* dst_index, int64_t copies,
+    int64_t M, int64_t K, int64_t out_rows, int64_t in_row_stride, int64_t out_row_stride,
+    int64_t group_size, int64_t scales_ld,
+    int in_dtype, int scales_dtype, float scale_ub, void* stream);
+
+/*
  * Batched dynamic activation quantisation: B independent [M, K] problems in one
  * launch.  Replaces batched_quantize_dynamic_scaled_fp8
  *   (max/kernels/src/linalg/fp8_quantization.mojo:779-954), which the MLA

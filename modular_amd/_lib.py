@@ -27,6 +27,7 @@ EXPORTS = (
     "maxfp8_quantize_dynamic_scaled_fp8",
     "maxfp8_batched_quantize_dynamic_scaled_fp8",
     "maxfp8_quantize_dynamic_scaled_fp8_gather",
+    "maxfp8_quantize_dynamic_scaled_fp8_scatter",
     "maxfp8_grouped_matmul_dynamic_scaled_fp8_scatter",
     "maxfp8_rms_norm_fused_quantize_dynamic_scaled_fp8",
     "maxfp8_matmul_dynamic_scaled_fp8",
@@ -77,6 +78,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_quantize_dynamic_scaled_fp8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, cf, vp]
     L.maxfp8_quantize_dynamic_scaled_fp8_gather.restype = ci
     L.maxfp8_quantize_dynamic_scaled_fp8_gather.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, ci, ci, cf, vp]
+    L.maxfp8_quantize_dynamic_scaled_fp8_scatter.restype = ci
+    L.maxfp8_quantize_dynamic_scaled_fp8_scatter.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, ci, ci, cf, vp]
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8_scatter.restype = ci
     L.maxfp8_grouped_matmul_dynamic_scaled_fp8_scatter.argtypes = [vp] * 8 + [i64] * 7 + [ci, ci, ci, vp]
     L.maxfp8_batched_quantize_dynamic_scaled_fp8.restype = ci

@@ -30,6 +30,8 @@ int launch_status(const char* what) {
 // kernels (defined in the other translation units)
 int quantize_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, int,
                       float, int64_t, int64_t, int64_t, int64_t, const uint32_t*, uint32_t, hipStream_t);
+int quantize_scatter_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int64_t, int64_t, float, const uint32_t*, int64_t,
+                              int64_t, hipStream_t);
 int rmsnorm_quantize_dispatch(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float,
                               float, float, hipStream_t);
 int quantize_static_dispatch(void*, const void*, int64_t, int64_t, int64_t, int64_t, int, float, hipStream_t);
@@ -210,6 +212,28 @@ int maxfp8_quantize_dynamic_scaled_fp8_gather(void* out_fp8, void* out_scales, c
   if (index_div < 1 || index_div > 0xffffffffll) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize (gather): index_div must be at least 1");
   return quantize_common(out_fp8, out_scales, in, row_index, (uint32_t)index_div, M, K, in_row_stride, out_row_stride,
                          group_size, scales_ld, in_dtype, scales_dtype, scale_ub, stream);
+}
+
+int maxfp8_quantize_dynamic_scaled_fp8_scatter(void* out_fp8, void* out_scales, const void* in, const uint32_t* dst_index,
+                                               int64_t copies, int64_t M, int64_t K, int64_t out_rows, int64_t in_row_stride,
+                                               int64_t out_row_stride, int64_t group_size, int64_t scales_ld, int in_dtype,
+                                               int scales_dtype, float scale_ub, void* stream) {
+  if (M < 0 || K < 0 || out_rows < 0 || copies < 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize (scatter): negative size M=%lld K=%lld out_rows=%lld copies=%lld", (long long)M, (long long)K,
+                (long long)out_rows, (long long)copies);
+  if (M == 0 || K == 0 || copies == 0 || out_rows == 0) return MAXFP8_OK;
+  if (in_dtype != MAXFP8_BF16 || scales_dtype != MAXFP8_F32 || group_size != 128)
+    MAXFP8_FAIL(MAXFP8_ERR_DTYPE, "quantize (scatter): takes bfloat16 input, float32 scales and groups of 128 (got dtypes %d, %d, group %lld); "
+                "the gather form takes the rest", in_dtype, scales_dtype, (long long)group_size);
+  if (in_row_stride < K || out_row_stride < K || scales_ld < out_rows)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize (scatter): strides (in %lld, out %lld, scales %lld) smaller than the extents",
+                (long long)in_row_stride, (long long)out_row_stride, (long long)scales_ld);
+  if (!out_fp8 || !out_scales || !in || !dst_index) MAXFP8_FAIL(MAXFP8_ERR_NULL, "quantize (scatter): null pointer");
+  const int rc = quantize_scatter_dispatch(out_fp8, out_scales, in, M, K, in_row_stride, out_row_stride, scales_ld, scale_ub, dst_index,
+                                           copies, out_rows, (hipStream_t)stream);
+  if (rc == -1)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "quantize (scatter): rows must be 16-byte aligned and K a multiple of 128; the gather form takes the rest");
+  return rc;
 }
 
 int maxfp8_batched_quantize_dynamic_scaled_fp8(void* out_fp8, void* out_scales, const void* in, int64_t B, int64_t M, int64_t K,

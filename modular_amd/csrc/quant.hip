@@ -102,6 +102,70 @@ __global__ __launch_bounds__(256) void quant_g128_bf16_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// The same quantisation with `copies` destinations: input row r is quantised once and written to the output rows
+// dst_index[r * copies + j], j < copies (rows of `out`, columns of `scales`).  What a row gather with repeated source
+// rows costs top_k times over -- the loads and the arithmetic -- is paid once; the stores are the gather form's.
+// A destination outside [0, out_rows) is skipped.
+template <int U>
+__global__ __launch_bounds__(256) void quant_g128_bf16_scatter_kernel(
+    uint8_t* __restrict__ out, float* __restrict__ scales, const uint16_t* __restrict__ in,
+    int M, int ngroups, int nxb, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
+    float scale_ub, const uint32_t* __restrict__ dst_index, int copies, int64_t out_rows) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int seg = lane >> 4, sl = lane & 15;
+  const int rb = blockIdx.x / nxb, xb = blockIdx.x - rb * nxb;
+  const int row = rb * 16 + wave * 4 + seg;
+  const int gbase = xb * U;
+  const bool row_ok = row < M;
+
+  uint4 v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int g = gbase + u;
+    if (row_ok && g < ngroups)
+      v[u] = *reinterpret_cast<const uint4*>(in + (int64_t)row * in_stride + (int64_t)g * 128 + sl * 8);
+    else
+      v[u] = make_uint4(0, 0, 0, 0);
+  }
+  float my_scale = 0.0f;
+  uint2 code[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(f[i]));
+    amax = row16_max(amax);
+    float scale, recip;
+    dynamic_scale_f32(amax, scale_ub, scale, recip);
+    if (sl == u) my_scale = scale;
+    int lo = 0, hi = 0;
+    lo = cvt_pk_e4m3fn(clamp448(f[0] * recip), clamp448(f[1] * recip), lo, false);
+    lo = cvt_pk_e4m3fn(clamp448(f[2] * recip), clamp448(f[3] * recip), lo, true);
+    hi = cvt_pk_e4m3fn(clamp448(f[4] * recip), clamp448(f[5] * recip), hi, false);
+    hi = cvt_pk_e4m3fn(clamp448(f[6] * recip), clamp448(f[7] * recip), hi, true);
+    code[u] = make_uint2((uint32_t)lo, (uint32_t)hi);
+  }
+  if (!row_ok) return;
+  for (int j = 0; j < copies; ++j) {
+    const int64_t dst = dst_index[(int64_t)row * copies + j];
+    if (dst >= out_rows) continue;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (gbase + u < ngroups)
+        *reinterpret_cast<uint2*>(out + dst * out_stride + (int64_t)(gbase + u) * 128 + sl * 8) = code[u];
+    }
+    if (sl < U && gbase + sl < ngroups) scales[(int64_t)(gbase + sl) * scales_ld + dst] = my_scale;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // One block (256 threads) per row, group == K.  NV 16-byte vectors per thread are
 // held in registers; K <= 256 * 8 * NV.
 template <int NV, bool STREAM>
@@ -528,6 +592,20 @@ int quantize_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M
                      out_scales, in, (int)ngroups, (int)G, in_row_stride, out_row_stride, scales_ld, in_dtype,
                      scales_dtype, scale_ub, bs, rg);
   return launch_status("quant_generic");
+}
+
+// bf16 in, f32 scales, groups of 128, 16-byte aligned rows: what the scatter form takes (-1: not this)
+int quantize_scatter_dispatch(void* out_fp8, void* out_scales, const void* in, int64_t M, int64_t K, int64_t in_row_stride,
+                              int64_t out_row_stride, int64_t scales_ld, float scale_ub, const uint32_t* dst_index,
+                              int64_t copies, int64_t out_rows, hipStream_t stream) {
+  const bool vec_ok = aligned16(in) && (in_row_stride % 8 == 0) && (reinterpret_cast<uintptr_t>(out_fp8) % 8 == 0) && (out_row_stride % 8 == 0);
+  constexpr int U = 4;
+  const int64_t ngroups = K / 128, nxb = ceil_div(ngroups, U), blocks = ceil_div(M, 16) * nxb;
+  if (!vec_ok || K % 128 != 0 || blocks >= (int64_t)1 << 31 || copies > 0x7fffffff) return -1;
+  hipLaunchKernelGGL(quant_g128_bf16_scatter_kernel<U>, dim3((unsigned)blocks), dim3(256), 0, stream, (uint8_t*)out_fp8,
+                     (float*)out_scales, (const uint16_t*)in, (int)M, (int)ngroups, (int)nxb, in_row_stride, out_row_stride,
+                     scales_ld, scale_ub, dst_index, (int)copies, out_rows);
+  return launch_status("quant_g128_bf16_scatter");
 }
 
 int rmsnorm_quantize_dispatch(void* out_fp8, void* out_scales, const void* in, const void* gamma, int64_t rows, int64_t K,

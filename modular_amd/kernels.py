@@ -76,6 +76,7 @@ def quantize_dynamic_scaled_float8(
     *,
     row_index: torch.Tensor | None = None,
     index_div: int = 1,
+    scatter_index: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """Dynamically quantize `input` [M, K] to fp8.
 
@@ -87,6 +88,12 @@ def quantize_dynamic_scaled_float8(
     quantised from `input[row_index[r] // index_div]`: the gather that the reference's
     graph compiler fuses into the op's input (builtin_kernels/quantization.mojo:1376-1390),
     e.g. `row_index=token_expert_order, index_div=top_k` in the MoE layer.
+
+    With `scatter_index` (uint32 [M * copies] on the device) the result has M * copies rows
+    and `input[r]` is quantised once and written to the rows `scatter_index[r * copies + j]`:
+    the same bytes as the gather by the inverse permutation
+    (`scatter_index=restore_token_order`), without quantising a token top_k times.  bfloat16
+    input, float32 scales and groups of 128 only.
     """
     if input.dim() != 2:
         raise ValueError("input must be rank 2 tensor")
@@ -94,6 +101,14 @@ def quantize_dynamic_scaled_float8(
         # e4m3fnuz is only ever requested on gfx94x (kernels.py:8408-8417)
         raise ValueError("out_type must be float8_e4m3fn or float8_e4m3fnuz")
     M, K = input.shape
+    if scatter_index is not None:
+        if row_index is not None:
+            raise ValueError("row_index and scatter_index exclude each other")
+        if scatter_index.dtype != torch.uint32 or scatter_index.dim() != 1:
+            raise TypeError("scatter_index must be a rank 1 uint32 tensor")
+        if M == 0 or scatter_index.shape[0] % M != 0:
+            raise ValueError(f"scatter_index must hold a whole number of destinations per input row ({M} rows)")
+        src_rows, copies, M = M, scatter_index.shape[0] // M, scatter_index.shape[0]
     if row_index is not None:
         if row_index.dtype != torch.uint32 or row_index.dim() != 1:
             raise TypeError("row_index must be a rank 1 uint32 tensor")
@@ -116,6 +131,14 @@ def quantize_dynamic_scaled_float8(
         input = input.contiguous()
     out = torch.empty((M, K), dtype=_FP8, device=input.device)
     scales = torch.empty((K // group_size, a_scales_dim1), dtype=scales_type, device=input.device)
+    if scatter_index is not None:
+        _require_gpu(scatter_index)
+        st = _lib.lib().maxfp8_quantize_dynamic_scaled_fp8_scatter(
+            out.data_ptr(), scales.data_ptr(), input.data_ptr(), scatter_index.data_ptr(), copies, src_rows, K, M,
+            input.stride(0) if src_rows > 1 else K, K,
+            group_size, a_scales_dim1, _DT[input.dtype], _DT[scales_type], float(scale_ub), _stream(input))
+        _lib.check(st)
+        return out, scales
     if row_index is not None:
         _require_gpu(row_index)
         st = _lib.lib().maxfp8_quantize_dynamic_scaled_fp8_gather(

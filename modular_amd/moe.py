@@ -2,8 +2,10 @@
 `_expert_matmuls` (max/python/max/nn/moe/moe_fp8.py:487-616, FP8 block-scaled strategy):
 
     group the (token, expert) assignments by expert      moe_create_indices
-    gather the tokens into that order and quantise       quantize_dynamic_scaled_float8(row_index=...)
-    1 x 128 (the gather rides on the quantiser's loads)
+    gather the tokens into that order and quantise       quantize_dynamic_scaled_float8(scatter_index=...)
+    1 x 128 (a token is quantised once and stored to
+    its top_k rows; other dtypes: row_index=..., the
+    gather rides on the quantiser's loads)
     gate_up = grouped matmul                             grouped_dynamic_scaled_fp8_matmul
     silu(gate) * up on the rows in use                   fused_silu
     quantise 1 x 128, down = grouped matmul that stores  grouped_dynamic_scaled_fp8_matmul(out_row_index=...)
@@ -35,12 +37,12 @@ class Fp8Strategy:
         self.dtype = dtype
 
     def quantize(self, tensor: torch.Tensor, group_size: int, *, row_index: torch.Tensor | None = None,
-                 index_div: int = 1) -> tuple[torch.Tensor, torch.Tensor]:
+                 index_div: int = 1, scatter_index: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
         """Quantizes activations to FP8 and returns (quantized, scales)."""
         return quantize_dynamic_scaled_float8(tensor, self.config.input_scale, self.config.weight_scale,
                                               group_size_or_per_token=group_size, out_type=self.dtype,
                                               scales_type=self.config.weight_scale.dtype, row_index=row_index,
-                                              index_div=index_div)
+                                              index_div=index_div, scatter_index=scatter_index)
 
     def grouped_quantize(self, tensor: torch.Tensor, group_size: int, input_scale: torch.Tensor | None,
                          expert_start: torch.Tensor, scales_offset: torch.Tensor | None,
@@ -118,8 +120,13 @@ def expert_matmuls_fp8(
         # the bounds that need no look at the GPU: every row on one expert, every expert active
         usage_stats = torch.tensor([seq_len * top_k, num_experts], dtype=torch.int64).to(torch.uint32)
 
-    # sorted row r is assignment token_order[r] = token * top_k + slot: it reads token token_order[r] // top_k
-    permuted_quant, permuted_scales = strategy.quantize(x, group, row_index=token_order, index_div=top_k)
+    # sorted row r is assignment token_order[r] = token * top_k + slot: it reads token token_order[r] // top_k.  Seen
+    # from the token: it is quantised once and stored to its top_k sorted rows restore_order[token * top_k + slot] --
+    # the same bytes, and what the kernel for bfloat16 activations, float32 scales and groups of 128 does
+    if x.dtype == torch.bfloat16 and group == 128 and quant_config.weight_scale.dtype == torch.float32 and x.stride(0) % 8 == 0:
+        permuted_quant, permuted_scales = strategy.quantize(x, group, scatter_index=restore_order)
+    else:
+        permuted_quant, permuted_scales = strategy.quantize(x, group, row_index=token_order, index_div=top_k)
     gate_up_scales, down_scales = strategy.prepare_weight_scales(gate_up_proj_scales, down_proj_scales, x.device)
     expert_inputs = (permuted_quant, permuted_scales, expert_start, expert_ids, usage_stats)
     gate_up = strategy.grouped_matmul(gate_up_proj, gate_up_scales, expert_inputs=expert_inputs)

@@ -50,6 +50,58 @@ def test_quantise_gathered_rows(dev, rows, K, R, div, group, dtype):
         assert np.array_equal(f32_np(s)[:, :R], so)
 
 
+@pytest.mark.parametrize("rows,K,copies", [(64, 512, 2), (300, 7168, 8), (1, 256, 8), (33, 384, 1), (4096, 1024, 8), (50, 128, 3)])
+def test_quantise_once_and_scatter_rows(dev, rows, K, copies):
+    # input row r, quantised once, goes to the rows scatter_index[r * copies + j]: with a permutation as the index the
+    # same bytes as the gather by its inverse, and as the oracle on the gathered rows
+    g = torch.Generator().manual_seed(rows * 3 + copies)
+    x = synth.activations(rows, K, seed=rows + K)
+    dst = torch.randperm(rows * copies, generator=g)          # assignment a = r * copies + j lands in row dst[a]
+    src = torch.empty_like(dst)
+    src[dst] = torch.arange(rows * copies)                    # row d is assignment src[d]: the gather's index
+    spec = (BLK.input_scale, BLK.weight_scale)
+    kw = dict(scales_type=torch.float32, group_size_or_per_token=128)
+    xd = x.to(dev)
+    q, s = mx.quantize_dynamic_scaled_float8(xd, *spec, scatter_index=u32(dst).to(dev), **kw)
+    q0, s0 = mx.quantize_dynamic_scaled_float8(xd, *spec, row_index=u32(src).to(dev), index_div=copies, **kw)
+    torch.cuda.synchronize()
+    R = rows * copies
+    assert q.shape == (R, K) and s.shape == s0.shape
+    assert np.array_equal(fp8_bytes(q), fp8_bytes(q0))
+    assert np.array_equal(f32_np(s)[:, :R], f32_np(s0)[:, :R])
+    qo, so = oracle.quantize_dynamic_scaled_fp8(bf16_bits(x.index_select(0, src // copies)), 128, threads=NT)
+    assert np.array_equal(fp8_bytes(q), qo)
+    assert np.array_equal(f32_np(s)[:, :R], so)
+
+
+def test_scatter_skips_destinations_outside_the_result(dev):
+    rows, K = 16, 256
+    x = synth.activations(rows, K, seed=3).to(dev)
+    dst = torch.arange(rows * 2)
+    dst[5] = 4000000000 % (1 << 32)          # far outside the 32 rows of the result
+    q, s = mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32,
+                                             group_size_or_per_token=128, scatter_index=u32(dst).to(dev))
+    q0, s0 = mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32,
+                                               group_size_or_per_token=128)
+    torch.cuda.synchronize()
+    keep = [a for a in range(rows * 2) if a != 5]
+    assert np.array_equal(fp8_bytes(q)[keep], fp8_bytes(q0)[[a // 2 for a in keep]])
+
+
+def test_scatter_argument_checks(dev):
+    x = synth.activations(8, 256, seed=1).to(dev)
+    idx = u32(torch.arange(16)).to(dev)
+    kw = dict(scales_type=torch.float32, group_size_or_per_token=128)
+    with pytest.raises(TypeError):
+        mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scatter_index=torch.arange(16).to(dev), **kw)
+    with pytest.raises(ValueError):   # not a whole number of destinations per row
+        mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scatter_index=idx[:15], **kw)
+    with pytest.raises(ValueError):
+        mx.quantize_dynamic_scaled_float8(x, BLK.input_scale, BLK.weight_scale, scatter_index=idx, row_index=idx, **kw)
+    with pytest.raises(TypeError):   # float32 input: the gather form's business
+        mx.quantize_dynamic_scaled_float8(x.float(), BLK.input_scale, BLK.weight_scale, scatter_index=idx, **kw)
+
+
 def test_gather_argument_checks(dev):
     x = synth.activations(8, 256, seed=1).to(dev)
     idx = torch.zeros(4, dtype=torch.int64)
