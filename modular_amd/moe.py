@@ -123,7 +123,8 @@ def expert_matmuls_fp8(
     # sorted row r is assignment token_order[r] = token * top_k + slot: it reads token token_order[r] // top_k.  Seen
     # from the token: it is quantised once and stored to its top_k sorted rows restore_order[token * top_k + slot] --
     # the same bytes, and what the kernel for bfloat16 activations, float32 scales and groups of 128 does
-    if x.dtype == torch.bfloat16 and group == 128 and quant_config.weight_scale.dtype == torch.float32 and x.stride(0) % 8 == 0:
+    if (x.dtype == torch.bfloat16 and group == 128 and quant_config.weight_scale.dtype == torch.float32 and
+            x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
         permuted_quant, permuted_scales = strategy.quantize(x, group, scatter_index=restore_order)
     else:
         permuted_quant, permuted_scales = strategy.quantize(x, group, row_index=token_order, index_div=top_k)
