@@ -192,6 +192,27 @@ def test_random_groupings_are_exact(dev, tune, launches):
         assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, N {N}, K {K}, {out}"
 
 
+@pytest.mark.parametrize("counts,N", [([1024] * 8, 2048), ([8] * 100, 1024), ([200] * 40, 512), ([100] * 30 + [1300] * 3, 768)])
+def test_launches_of_one_kind_of_tile_many_times(dev, counts, N):
+    """A grouping whose tiles are all of one kind (256-row tiles only; streaming tiles only; one mid-size kind) leaves
+    most (kind, XCD) counters of the persistent launch without work from the start and the others empty at the same
+    moment: the blocks' search for the next pair that still has tiles, and the counters' return to zero, decide the
+    result.  More launches than there are counter sets (64), every one equal to the scalar kernel's result."""
+    rng = np.random.default_rng(len(counts) + N)
+    E, K = len(counts), 256
+    T = sum(counts)
+    a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (T, K)).astype(np.float32)))
+    b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (E, N, K)).astype(np.float32)))
+    sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (K // 128, -(-T // 4) * 4))).astype(np.float32))
+    sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (E, -(-N // 128), K // 128))).astype(np.float32))
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32)
+    idt = torch.arange(E, dtype=torch.int32)
+    want = run(a, b, sa, sb, off, idt, max(counts), E, dev, out=torch.bfloat16, algo="naive")
+    for launch in range(70):
+        got = run(a, b, sa, sb, off, idt, max(counts), E, dev, out=torch.bfloat16)
+        assert torch.equal(got, want), f"launch {launch}"
+
+
 def test_more_slots_than_the_persistent_launch_holds(dev):
     """600 active slots: more than the persistent launch's tables hold (512), so the two-launch form runs; exact on
     integer data like every other path."""
