@@ -353,6 +353,54 @@ def read_ceiling(wl, steps):
     return first.elapsed_time(last) / steps
 
 
+MFMA_CEILING_KERNELS = {0: ("eight waves, 256 x 256 tiles (gemm_persist_kernel)", 256),
+                        5: ("four waves, 160 x 256 tiles (gemm_w4_kernel)", 160),
+                        6: ("four waves, 192 x 256 tiles (gemm_w4_kernel)", 192)}
+
+
+def mfma_ceiling(slabs=4096, reps=20, settle_s=0.5):
+    """The main loops of the dense kernels on operands that never leave the chip (maxfp8_mfma_issue_probe): one block per
+    CU runs `slabs` K slabs of one tile -- level 2: the MFMA loop alone, fragments read from LDS (row scaling: MFMA only;
+    block scaling: with the per-slab promotions); level 1: with the LDS-DMA copies, waits and barriers, operands in L2.
+    Yields one record per (kernel, scaling, level): microseconds per slab and the rate over all CUs."""
+    import torch
+    from modular_amd import _lib, synth
+
+    dev = torch.device("cuda:0")
+    L, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
+    # operands like the workloads': quantised normal data (no NaN bytes), scales of the usual size
+    a = synth.random_fp8((256, 1024), 1, std=150.0).to(dev)
+    b = synth.random_fp8((256, 1024), 2, std=150.0).to(dev)
+    a_s = synth.random_scales((8, 256), 3).to(dev)
+    b_s = synth.random_scales((2, 8), 4).to(dev)
+    c = torch.empty((256, 256), dtype=torch.bfloat16, device=dev)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for kernel, (label, rows) in MFMA_CEILING_KERNELS.items():
+        for block in (0, 1):
+            for level in (2, 1):
+                def launch(n):
+                    _lib.check(L.maxfp8_mfma_issue_probe(kernel, block, level, n, a.data_ptr(), b.data_ptr(), a_s.data_ptr(),
+                                                         b_s.data_ptr(), c.data_ptr(), stream))
+                t_end = time.perf_counter() + settle_s   # the clocks of an idle GPU take tenths of a second to settle
+                while time.perf_counter() < t_end:
+                    launch(slabs)
+                    torch.cuda.synchronize()
+                first.record()
+                for _ in range(reps):
+                    launch(slabs)
+                last.record()
+                torch.cuda.synchronize()
+                us_slab = first.elapsed_time(last) * 1e3 / reps / slabs
+                flops_slab = 2.0 * rows * 256 * 128 * cus
+                yield {"kernel": label, "scaling": "block" if block else "row",
+                       "level": "MFMA loop on LDS-resident operands" + (" + promotions" if block else "") if level == 2 else
+                                "whole loop (copies, waits, barriers), operands in L2",
+                       "us_per_slab": round(us_slab, 4), "TFLOP/s": round(flops_slab / us_slab / 1e6, 1),
+                       "frac_of_peak": round(flops_slab / us_slab / 1e6 / PEAK_FP8_TFLOPS, 3), "slabs": slabs, "launches": reps,
+                       "blocks": cus}
+
+
 def cpu_baseline(wl, budget_s=15.0):
     """The oracle (a port of the reference's host loops) on this host's cores, on a bounded
     slice of the same workload; throughput in the metric's unit."""
@@ -509,6 +557,10 @@ def main():
                     help="the expert matmuls of the FP8 MoE layer on configs[4]'s routing (grouping, gathered quantise, grouped "
                          "gate_up, silu * up, quantise, grouped down): milliseconds per call, one JSON line for each way of the "
                          "activation quantisation (two kernels, one kernel)")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="the dense kernels' main loops on operands that stay on the chip (LDS-resident: MFMA loop alone and "
+                         "with promotions; L2-resident: with copies and barriers), one JSON line each: the issue ceiling the "
+                         "dense matmuls are measured against")
     ap.add_argument("--read-ceiling", action="store_true",
                     help="for every decode workload (M <= 16): the matmul kernel's time beside the time of its read-only "
                          "probe (same grid and weight traffic, no arithmetic), one JSON line each")
@@ -562,6 +614,10 @@ def main():
                               "fuse_activation_quant": fuse, "ms_per_call": round(ms, 4), "steps": args.steps,
                               "timing": "host clock around the calls, no host synchronisation inside a call"}), flush=True)
             torch.cuda.empty_cache()
+        return
+    if args.mfma_ceiling:
+        for rec in mfma_ceiling():
+            print(json.dumps(rec), flush=True)
         return
     if args.read_ceiling:
         for name in ([args.workload] if args.workload else [n for n, w in WORKLOADS.items() if w[0] == "row" and w[1] <= 16]):

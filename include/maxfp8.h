@@ -477,6 +477,20 @@ int maxfp8_copy_bytes(void* dst, const void* src, int64_t n, void* stream);
  */
 int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t K, int64_t ldb, void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: the main loop of a dense block- or row-scaled matmul kernel
+ * (kernel 0: eight waves, 256 x 256 tiles; kernel 5 / 6: four waves, 160 x 256 / 192 x 256 tiles) run for `slabs` K slabs of 128 bytes
+ * by one block on every compute unit, all blocks on the same tile:
+ *   level 2: the MFMA loop alone (block scaling: with its promotions), fragments read from what one copy left in LDS;
+ *   level 1: the whole loop -- LDS-DMA copies, waits, barriers -- with operands that stay in L2 (slabs 0..7 of tile
+ *            (0, 0) over and over).
+ * a, b: 256 rows x 1024 bytes of e4m3fn each; a_scales: 8 x 256 floats, b_scales: 2 x 8 floats; c: 256 x 256 bf16, written
+ * once at the end with meaningless values.  The kernel's time over slabs * 256 * 256 * 128 * 2 flops per block (four waves:
+ * 160 or 192 rows) is the issue ceiling the matmul kernels are measured against.
+ */
+int maxfp8_mfma_issue_probe(int kernel, int blockscale, int level, int64_t slabs, const void* a, const void* b, const float* a_scales,
+                            const float* b_scales, void* c, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

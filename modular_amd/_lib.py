@@ -48,6 +48,7 @@ EXPORTS = (
     "maxfp8_cast_f32_to_bf16",
     "maxfp8_copy_bytes",
     "maxfp8_decode_weight_read_probe",
+    "maxfp8_mfma_issue_probe",
 )
 
 _lib = None
@@ -123,6 +124,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_copy_bytes.argtypes = [vp, vp, i64, vp]
     L.maxfp8_decode_weight_read_probe.restype = ci
     L.maxfp8_decode_weight_read_probe.argtypes = [vp, i64, i64, i64, i64, vp]
+    L.maxfp8_mfma_issue_probe.restype = ci
+    L.maxfp8_mfma_issue_probe.argtypes = [ci, ci, ci, i64, vp, vp, vp, vp, vp, vp]
     _lib = L
     return L
 

@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libmaxfp8.so")
 
-SOURCES = ["api.hip", "quant.hip", "naive.hip", "gemm_tiled.hip", "gemm_skinny.hip", "moe.hip"]
+SOURCES = ["api.hip", "quant.hip", "naive.hip", "gemm_tiled.hip", "gemm_w4.hip", "gemm_skinny.hip", "moe.hip"]
 
 # packed-fp32 VALU ops are switched off for every kernel (they are not used by hand either)
 COMMON = [
@@ -26,7 +26,9 @@ COMMON = [
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
 # the naive kernels must round every product and sum like a scalar host loop
-PER_FILE = {"naive.hip": ["-ffp-contract=off"]}
+# the four-wave kernels keep their MFMA results in ordinary VGPRs (the promotions are VALU work) and their operand
+# fragments in AGPRs: left to itself the compiler writes every MFMA result to AGPRs once a kernel uses any
+PER_FILE = {"naive.hip": ["-ffp-contract=off"], "gemm_w4.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def hipcc() -> str:

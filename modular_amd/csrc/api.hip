@@ -59,6 +59,10 @@ int gemm_skinny_dispatch(const GemmArgs&, bool, int64_t, hipStream_t);
 int gemm_skinny_max_m();
 bool gemm_skinny_preferred(int64_t M, int64_t N, int64_t K);
 int gemm_skinny_read_probe(const void* b, int64_t M, int64_t N, int64_t K, int64_t ldb, hipStream_t stream);
+int gemm_persist_probe(const GemmArgs&, bool, int, hipStream_t);
+int gemm_w4_probe(const GemmArgs&, bool, int, int, hipStream_t);
+int gemm_w4_launch(const GemmArgs&, bool, int, hipStream_t);
+bool gemm_w4_ok(const GemmArgs&, bool);
 
 // v rounded to bf16 / f16 and widened back: how an op parameter of the input's dtype arrives
 static float round_to_dtype(float v, int dtype) {
@@ -132,7 +136,8 @@ static const Tuning* read_tuning(unsigned generation) {
   t->big_rows = num("MAXFP8_BIG_ROWS", 1024);
   t->grouped_overlap = num("MAXFP8_GROUPED_OVERLAP", 1) != 0;
   t->grouped_persist = num("MAXFP8_GROUPED_PERSIST", 1) != 0;
-  t->pingpong = num("MAXFP8_PINGPONG", 0) != 0;
+  const int w4 = num("MAXFP8_W4", -1);
+  t->w4 = (w4 == 0 || w4 == 5 || w4 == 6) ? w4 : -1;
   t->skinny_alds = num("MAXFP8_SKINNY_ALDS", 1) != 0;
   const char* sb = getenv("MAXFP8_GROUPED_SHARE");
   t->grouped_share = sb ? (float)atof(sb) : 0.5f;
@@ -753,6 +758,30 @@ int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t
   if (!is_aligned(b, 16) || K % 16 != 0 || ldb % 16 != 0) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "read probe: needs 16-byte aligned rows and K %% 16 == 0");
   if (!offsets_fit(K, ldb, ldb, 0, false)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "read probe: rows too long for 32-bit tile offsets");
   return gemm_skinny_read_probe(b, M, N, K, ldb, (hipStream_t)stream);
+}
+
+int maxfp8_mfma_issue_probe(int kernel, int blockscale, int level, int64_t slabs, const void* a, const void* b, const float* a_scales,
+                            const float* b_scales, void* c, void* stream) {
+  if (!a || !b || !c || !a_scales || !b_scales) MAXFP8_FAIL(MAXFP8_ERR_NULL, "issue probe: null pointer");
+  if ((kernel != 0 && kernel != 5 && kernel != 6) || (level != 1 && level != 2) || slabs < 8 || slabs > (1 << 22) || slabs % 2 != 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "issue probe: kernel 0 / 5 / 6, level 1 / 2, an even number of slabs in [8, 2^22]");
+  if (!is_aligned(a, 16) || !is_aligned(b, 16) || !is_aligned(c, 16)) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "issue probe: 16-byte aligned buffers");
+  GemmArgs p;
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t*)a;
+  p.b = (const uint8_t*)b;
+  p.c = c;
+  p.a_scales = a_scales;
+  p.b_scales = b_scales;
+  p.M = 256; p.N = 256; p.K = (int)(slabs * 128);
+  p.lda = 1024; p.ldb = 1024; p.ldc = 256;
+  p.a_scales_ld = 256; p.b_scales_ld = 8;
+  p.a_scale_stride = 0; p.b_scale_stride = 0;  // (row mode: element 0 of each scale vector, in the epilogue)
+  p.c_dtype = MAXFP8_BF16;
+  p.scales_dtype = MAXFP8_F32;
+  p.c_vec_ok = 1; p.c_vec8_ok = 1;
+  p.splits = 1;
+  return kernel == 0 ? gemm_persist_probe(p, blockscale != 0, level, (hipStream_t)stream) : gemm_w4_probe(p, blockscale != 0, level, kernel, (hipStream_t)stream);
 }
 
 }  // extern "C"

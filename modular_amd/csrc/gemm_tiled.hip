@@ -45,45 +45,10 @@
 #include <utility>
 #include "common.h"
 #include "gemm_args.h"
+#include "gemm_device.h"
 #include "tuning.h"
 
 namespace maxfp8 {
-
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-
-// Cache policy of copies whose bytes are read once per launch (the weights of experts with few rows): non-temporal.  The
-// stream then does not displace what the memory-side cache and the L2 hold, and the chip reads 7.0 instead of 6.2 TB/s.
-constexpr int kStreamOnce = 2;
-
-// f(integral_constant<int, 0>{}) ... f(integral_constant<int, N - 1>{}): a loop whose index is a constant
-template <class F, int... I>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t t2_rsrc(const void* p, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
-}
-__device__ __forceinline__ uint32_t t2_clamp_u32(int64_t v) {
-  return v > 0xfffffff0ll ? 0xfffffff0u : (v < 0 ? 0u : (uint32_t)v);
-}
-
-// A 16-byte buffer store whose scalar offset sits in a register.  The hardware reads the four data registers of such
-// a store during the cycles AFTER it has issued, and a VALU instruction that follows at once and writes one of them
-// changes what is stored; the compiler's hazard table has this case down as free of hazards (it pads only stores whose
-// scalar offset is an immediate) and schedules the next values straight into the registers.  Seen on MI355X as a
-// tile's bf16 pairs replaced, in some lanes, by the f32 products of the rows computed next.  The wait states are tied
-// to the data registers, so that nothing that overwrites them can be scheduled between the store and the wait.
-typedef unsigned int v4u_t __attribute__((ext_vector_type(4)));
-template <int CACHE_POLICY>
-__device__ __forceinline__ void buffer_store_b128_guarded(const v4u_t v, const __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset, uint32_t soffset) {
-  __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, voffset, soffset, CACHE_POLICY);
-  asm volatile("s_nop 7" ::"v"(v));
-}
 
 // The activation scales of a slab in LDS.  The copy puts its lanes' values at consecutive words, and a lane may fetch
 // any row: word i of the scale area gets the row that puts the TM scales a lane needs in the main loop -- rows lm,
@@ -624,18 +589,6 @@ const ScaleRow<TM> a_sc = read_scales<TM>(sa + s_rd);
   }
 }
 
-// tile number -> (row tile, column tile): groups of GROUP_M row tiles share weight columns, walked column-major
-__device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  constexpr int GROUP_M = 4;
-  const int per_group = GROUP_M * tiles_n;
-  const int group = pid / per_group;
-  const int first_m = group * GROUP_M;
-  const int gsize = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-  const int in_group = pid - group * per_group;
-  tm = first_m + in_group % gsize;
-  tn = in_group / gsize;
-}
-
 // B_STREAM: the matmul is one row of tiles, so every weight byte is read once: the weight copies are marked non-temporal
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NS, bool BLOCKSCALE, bool KV = false, bool B_STREAM = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2 : 1) void gemm_tiled_kernel(GemmArgs p) {
@@ -692,8 +645,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
 constexpr int kStreamkSlots = 64, kStreamkMaxBlocks = 512;
 static __device__ unsigned int g_streamk_flags[kStreamkSlots * kStreamkMaxBlocks];
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE, bool SPLIT>
+// PROBE (measurement aid, results meaningless): 1 the same loop with every copy reading tile (0, 0) and slabs 0..7 over
+// and over, so that the operands stay in L2, one job of K / 128 slabs per block; 2 the same without copies, waits and
+// barriers -- the MFMA loop on what the prologue left in LDS.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE, bool SPLIT, int PROBE = 0>
 __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
+  static_assert(!(SPLIT && PROBE != 0), "the probe has no hand-over");
   constexpr int NS = 2;
   constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -742,6 +699,8 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
     has_head = s_last_end != nslab;
     nwhole = t_last - t_first + 1 - (has_tail ? 1 : 0) - (has_head ? 1 : 0);
     njobs = nwhole + (has_tail ? 1 : 0) + (has_head ? 1 : 0);
+  } else if constexpr (PROBE != 0) {
+    njobs = 1;
   } else {
     njobs = my < run_len ? (run_len - my + nb - 1) / nb : 0;
   }
@@ -777,9 +736,11 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   }
   struct TileAt { uint32_t a, b, s; };  // byte offsets of a tile's activation rows, weight rows and activation scales
   auto tile_at = [&](int tm, int tn) {
+    if constexpr (PROBE != 0) return TileAt{0u, 0u, 0u};
     return TileAt{(uint32_t)(tm * BM) * (uint32_t)p.lda, (uint32_t)(tn * BN) * (uint32_t)p.ldb, (uint32_t)(tm * BM) * 4u};
   };
   auto dma_one = [&](const TileAt& at, int slab, int buf, int idx, uint32_t dead) {
+    if constexpr (PROBE != 0) slab &= 7;
     const uint32_t koff = (uint32_t)slab * 128u;
     uint32_t kill = dead, kill_b = dead;
     if (koff + cchunk * 16 >= (uint32_t)p.K) kill = 0x80000000u;
@@ -839,9 +800,17 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   Job cur = get_job(0);
   int tm, tn;
   tile_coords(cur.tile, tiles_m, tiles_n, tm, tn);
+  if constexpr (PROBE != 0) tm = tn = 0;
   TileAt cur_at = tile_at(tm, tn);
 #pragma unroll
   for (int idx = 0; idx < PER; ++idx) dma_one(cur_at, cur.s0, 0, idx, 0u);
+  if constexpr (PROBE == 2) {
+#pragma unroll
+    for (int idx = 0; idx < PER; ++idx) dma_one(cur_at, 1, 1, idx, 0u);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  }
   float bs_nxt = 1.f;
   if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld + cur.s0];
 
@@ -893,16 +862,18 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
     }
 
     for (int slab = cur.s0; slab < cur.s1; ++slab) {
-      if (slab == cur.s0 && stored && !took_over) {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTORE) : "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if constexpr (PROBE != 2) {
+        if (slab == cur.s0 && stored && !took_over) {
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTORE) : "memory");
+        } else {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
       }
-      __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
       const float bs = bs_nxt;
       if constexpr (BLOCKSCALE) {
-        if (slab + 1 < cur.s1) bs_nxt = bs_row[slab + 1];
+        if (slab + 1 < cur.s1) bs_nxt = bs_row[PROBE != 0 ? ((slab + 1) & 7) : slab + 1];
       }
       asm volatile("" ::: "memory");
       // the copy issued during this slab: the job's next slab, or the first slab of the next job
@@ -959,9 +930,11 @@ const ScaleRow<TM> a_sc = read_scales<TM>(sa + s_rd);
             acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
         }
         af = af_next;
+        if constexpr (PROBE != 2) {
 #pragma unroll
-        for (int idx = 0; idx < PER; ++idx)
-          if (idx * SPREAD / PER == mt) dma_one(dat, dma_slab, dma_buf, idx, dead);
+          for (int idx = 0; idx < PER; ++idx)
+            if (idx * SPREAD / PER == mt) dma_one(dat, dma_slab, dma_buf, idx, dead);
+        }
       }
       buf ^= 1;
     }
@@ -1054,355 +1027,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_persist_kernel(
   persist_body<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE, false>(p, smem);
 }
 
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE, int PROBE>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_persist_probe_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  persist_body<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE, false, PROBE>(p, smem);
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_streamk_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   persist_body<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE, true>(p, smem);
-}
-
-// ---- persistent variant, the two halves of the block half a slab apart ------------------------
-// Same tiles, stages, fragments and sums as gemm_persist_kernel, other timing.  There every wave passes one barrier per
-// slab, reads its first fragments and multiplies; the two waves of a SIMD do that in step, so the matrix pipe idles while
-// both wait, both read, and again when the faster one is done.  Here the block's two groups of four waves (the upper and
-// the lower 128 rows of the tile; one wave of each per SIMD) run the same slab loop HALF A SLAB APART: the block passes a
-// barrier every half slab, which for one group is the start of a slab and for the other its middle, so a wave that waits
-// for the barrier or for its first fragments shares its SIMD with a wave that is in the middle of its MFMAs.
-//
-// What makes that possible with two stages: a group's 128 activation rows (and their scales) are read by that group
-// only, so the stage's copy of them is free as soon as the group has finished the slab; and a slab's weight fragments are
-// read once, at the start of the slab.  Per slab s of the block's stream (S slabs over all of its tiles):
-//   group 0, first half:   copies its activation rows, their scales and weight rows 0..127 of slab s + 1
-//   group 1, first half:   copies its activation rows and their scales of slab s + 1
-//   group 1, second half:  copies weight rows 128..255 of slab s + 2 (group 0 read slab s's weights a barrier ago,
-//                          group 1 before this half's barrier)
-// Every copy has two half slabs to land.  A wave waits for its own copies with exact counts (the weight rows of slab
-// s + 2 and a finished tile's stores may stay in flight), then the barrier publishes them.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE>
-__device__ __forceinline__ void persist_pp_body(const GemmArgs& p, uint8_t* smem) {
-  constexpr int NS = 2;
-  constexpr int NWAVES = WAVES_M * WAVES_N;
-  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-  constexpr int TM = WM / 16, TN = WN / 16, HM = TM / 2;
-  constexpr int GW = WAVES_N;                     // waves per group
-  constexpr int IA = WM / 8 / GW, IB = (BN / 2) / 8 / GW;
-  constexpr int NSC = BLOCKSCALE ? 1 : 0;
-  constexpr int SCALE_BYTES = BLOCKSCALE ? BM * 4 : 0;
-  constexpr int STAGE_BYTES = (BM + BN) * 128 + SCALE_BYTES;
-  constexpr int SIDE_BYTES = 16 * WN * 2;
-  constexpr int NSTORE = TM * 2;
-  static_assert(WAVES_M == 2 && WN == 64 && WM == 128 && TM % 2 == 0 && TN % 2 == 0 && IA >= 1 && IB >= 1, "tile / wave layout");
-  static_assert(IA + NSC + IB + NSTORE < 64, "the counts must fit the vmcnt field");
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;  // wm: the group
-  const int lm = lane & 15, lq = lane >> 4;
-  const int nslab = (p.K + 127) / 128;
-
-  // the block's tiles: every 'nb'-th tile of its XCD's contiguous run, as in persist_body
-  const int tiles_m = p.M / BM, tiles_n = p.N / BN, total = tiles_m * tiles_n;
-  const int xcd = blockIdx.x & 7;
-  const int run_begin = xcd * (total >> 3) + (xcd < (total & 7) ? xcd : (total & 7));
-  const int run_len = (total >> 3) + (xcd < (total & 7) ? 1 : 0);
-  const int nb = ((int)gridDim.x - xcd + 7) >> 3;
-  const int my = blockIdx.x >> 3;
-  const int njobs = my < run_len ? (run_len - my + nb - 1) / nb : 0;
-  if (njobs <= 0) return;
-
-  // ---- copy plan.  Row block rb (8 rows) of the activation / weight rows of a stage sits at rb * 1024; wave wn of group
-  // g moves row blocks 16 * g + 4 * i + wn, i = 0 .. 3, of either operand.
-  const __amdgpu_buffer_rsrc_t a_rsrc = t2_rsrc(p.a, t2_clamp_u32((int64_t)(p.M - 1) * p.lda + p.K));
-  const __amdgpu_buffer_rsrc_t b_rsrc = t2_rsrc(p.b, t2_clamp_u32((int64_t)(p.N - 1) * p.ldb + p.K));
-  const int cr = lane >> 3, cp = lane & 7;
-  const int cchunk = cp ^ cr;
-  const int cchunk_b = cp ^ (((wn & 1) << 2) | (cr & 3));  // (row block parity == wn parity)
-  const int rb0 = 16 * wm + wn;
-  const uint32_t a_voff = (uint32_t)(rb0 * 8 + cr) * (uint32_t)p.lda + cchunk * 16;
-  const uint32_t b_voff = (uint32_t)(rb0 * 8 + cr) * (uint32_t)p.ldb + cchunk_b * 16;
-  const uint32_t a_istep = (uint32_t)(GW * 8) * (uint32_t)p.lda;
-  const uint32_t b_istep = (uint32_t)(GW * 8) * (uint32_t)p.ldb;
-  const int s_chunk = 2 * wm + (wn & 1);             // 64 activation scales per copy: the group's two chunks, twice
-  __amdgpu_buffer_rsrc_t s_rsrc = t2_rsrc(nullptr, 0);
-  uint32_t s_voff = 0, s_slab_step = 0;
-  if constexpr (BLOCKSCALE) {
-    s_rsrc = t2_rsrc(p.a_scales, t2_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + p.M) * 4));
-    s_voff = (uint32_t)scale_word_row<WM>(s_chunk * 64 + lane) * 4u;
-    s_slab_step = (uint32_t)p.a_scales_ld * 4u;
-  }
-  struct TileAt { uint32_t a, b, s; };
-  auto tile_at = [&](int tm, int tn) {
-    return TileAt{(uint32_t)(tm * BM) * (uint32_t)p.lda, (uint32_t)(tn * BN) * (uint32_t)p.ldb, (uint32_t)(tm * BM) * 4u};
-  };
-  // one copy instruction: idx 0 .. IA-1 activation rows, IA .. IA+NSC-1 their scales, then IB weight row blocks
-  auto dma_a = [&](const TileAt& at, int slab, int buf, int i, uint32_t dead) {
-    const uint32_t koff = (uint32_t)slab * 128u;
-    const uint32_t kill = (koff + cchunk * 16 >= (uint32_t)p.K) ? 0x80000000u : dead;
-    uint8_t* dst = smem + buf * STAGE_BYTES + (rb0 + i * GW) * 1024;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)dst, 16, a_voff | kill, at.a + koff + i * a_istep, 0, 0);
-  };
-  auto dma_s = [&](const TileAt& at, int slab, int buf, uint32_t dead) {
-    if constexpr (BLOCKSCALE) {
-      uint8_t* ss = smem + buf * STAGE_BYTES + (BM + BN) * 128 + s_chunk * 256;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(s_rsrc, (lds_ptr_t)ss, 4, s_voff | dead, at.s + (uint32_t)slab * s_slab_step, 0, 0);
-    }
-  };
-  // (on == false: the other group's turn.  The instruction is issued all the same, every lane out of range, so that both
-  // groups run the same code with the same counts; its zeros go to a kilobyte of the wave's own that nothing reads.)
-  uint8_t* const dummy = smem + NS * STAGE_BYTES + NWAVES * SIDE_BYTES + wave * 1024;
-  auto dma_b = [&](const TileAt& at, int slab, int buf, int i, uint32_t dead, bool on) {
-    const uint32_t koff = (uint32_t)slab * 128u;
-    const uint32_t off = on ? dead : 0x80000000u;
-    const uint32_t kill = (koff + cchunk_b * 16 >= (uint32_t)p.K) ? 0x80000000u : off;
-    uint8_t* dst = on ? smem + buf * STAGE_BYTES + BM * 128 + (rb0 + i * GW) * 1024 : dummy;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)dst, 16, b_voff | kill, at.b + koff + i * b_istep, 0, 0);
-  };
-
-  // ---- fragment read plan: as in tile_body
-  const int sw = lm & 7;
-  const uint32_t frag0 = lm * 128 + ((lq ^ sw) << 4);
-  const uint32_t frag1 = lm * 128 + (((lq + 4) ^ sw) << 4);
-  const uint32_t a_frag_base = (uint32_t)(wm * WM) * 128;
-  const uint32_t b_frag_base = (uint32_t)(BM + wn * WN) * 128;
-  auto read_frag = [&](const uint8_t* base) -> v8i {
-    const v4i lo = *reinterpret_cast<const v4i*>(base + frag0);
-    const v4i hi = *reinterpret_cast<const v4i*>(base + frag1);
-    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-  };
-  const int wrow = 8 * (lm >> 2) + (lm & 3);
-  const int wsw = (((wrow >> 3) & 1) << 2) | (wrow & 3);
-  const uint32_t wfrag0 = wrow * 128 + ((lq ^ wsw) << 4);
-  const uint32_t wfrag1 = wrow * 128 + (((lq + 4) ^ wsw) << 4);
-  auto read_wfrag = [&](const uint8_t* base, int t) -> v8i {
-    const uint8_t* g = base + (t >> 1) * 4096 + (t & 1) * 512;
-    const v4i lo = *reinterpret_cast<const v4i*>(g + wfrag0);
-    const v4i hi = *reinterpret_cast<const v4i*>(g + wfrag1);
-    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-  };
-  const uint32_t s_rd = (uint32_t)((BM + BN) * 128) + scale_read_offset<TM>(wm * WM, lm);
-  uint8_t* wbuf = smem + NS * STAGE_BYTES + wave * SIDE_BYTES;
-  const int rr = lane >> 3, cc = lane & 7;
-  const __amdgpu_buffer_rsrc_t c_rsrc = t2_rsrc(p.c, t2_clamp_u32(((int64_t)(p.M - 1) * p.ldc + p.N) * 2));
-  const uint32_t c_row_bytes = (uint32_t)p.ldc * 2u;
-  const uint32_t c_lane = (uint32_t)rr * c_row_bytes + (uint32_t)cc * 16u;
-  typedef unsigned int v4u __attribute__((ext_vector_type(4)));
-
-  // ---- the stream: job k, slab; the tile after this one
-  int k = 0, tm, tn, tm2 = 0, tn2 = 0;
-  tile_coords(run_begin + my, tiles_m, tiles_n, tm, tn);
-  TileAt cur_at = tile_at(tm, tn), next_at = cur_at;
-  bool has_next = njobs > 1;
-  if (has_next) {
-    tile_coords(run_begin + my + nb, tiles_m, tiles_n, tm2, tn2);
-    next_at = tile_at(tm2, tn2);
-  }
-  // prologue: slab 0 (and, group 1, its weight rows of slab 1)
-#pragma unroll
-  for (int i = 0; i < IA; ++i) dma_a(cur_at, 0, 0, i, 0u);
-  dma_s(cur_at, 0, 0, 0u);
-#pragma unroll
-  for (int i = 0; i < IB; ++i) dma_b(cur_at, 0, 0, i, 0u, true);
-  {
-    const bool same = nslab > 1;
-    const uint32_t dead = (same || has_next) ? 0u : 0x80000000u;
-#pragma unroll
-    for (int i = 0; i < IB; ++i) dma_b(same ? cur_at : next_at, same ? 1 : 0, 1, i, dead, wm == 1);
-  }
-  // (the weight-block scales are read through the constant address space: scalar loads, which neither take part in the
-  // vector-memory counts below nor hold a vector register from one slab to the next)
-  typedef const __attribute__((address_space(4))) float* const_f32_ptr;
-  const_f32_ptr b_scales_c = (const_f32_ptr)p.b_scales;
-  float bs_nxt = 1.f;
-  if constexpr (BLOCKSCALE) bs_nxt = b_scales_c[(int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld];
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if (wm == 1) __builtin_amdgcn_s_barrier();  // group 0's first half of its first slab
-
-  v4f acc[TM][TN];
-  v8i bf[TN], af;
-  float s_cur[TM];
-  [[maybe_unused]] v4f part[2][TN];
-  int buf = 0, slab = 0;
-  bool stored = false;  // the wave's youngest vector memory operations are a tile's NSTORE stores
-  const_f32_ptr bs_row = b_scales_c;
-  if constexpr (BLOCKSCALE) bs_row = b_scales_c + (int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld;
-
-  // one 16-row group of the wave's part: its MFMAs, the previous group's promotions, the next group's fragment
-  auto mt_step = [&](auto mt_c, const uint8_t* sa) {
-    constexpr int mt = decltype(mt_c)::value;
-    v8i af_next = af;
-    if constexpr (mt + 1 < TM) af_next = read_frag(sa + a_frag_base + (mt + 1) * 2048);
-    if constexpr (BLOCKSCALE) {
-      const v4f zero = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int nt = 0; nt < TN; ++nt)
-        part[mt & 1][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, zero, 0, 0, 0, 0, 0, 0);
-      if constexpr (mt > 0 && mt != HM) {
-#pragma unroll
-        for (int nt = 0; nt < TN; ++nt) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
-        }
-      } else {
-        __builtin_amdgcn_sched_group_barrier(0x008, TN, 0);
-      }
-      if constexpr (mt > 0) {
-#pragma unroll
-        for (int nt = 0; nt < TN; ++nt) acc[mt - 1][nt] += part[(mt - 1) & 1][nt] * s_cur[mt - 1];
-      }
-      if constexpr (mt == TM - 1) {
-#pragma unroll
-        for (int nt = 0; nt < TN; ++nt) acc[mt][nt] += part[mt & 1][nt] * s_cur[mt];
-      }
-    } else {
-#pragma unroll
-      for (int nt = 0; nt < TN; ++nt)
-        acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
-    }
-    af = af_next;
-  };
-
-  while (true) {
-    const bool last_slab = slab + 1 == nslab;
-    // ================= first half =================
-    // the group's own copies of this slab have landed; younger: (group 1) the weight rows of the slab after, a tile's stores
-    if (stored) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IB + NSTORE) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IB) : "memory");
-    stored = false;
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    const float bs = bs_nxt;
-    if constexpr (BLOCKSCALE) {
-      if (!last_slab) bs_nxt = bs_row[slab + 1];
-    }
-    asm volatile("" ::: "memory");
-    if (slab == 0) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
-    }
-    const uint8_t* sa = smem + buf * STAGE_BYTES;
-    // what is copied during this slab: slab + 1 of the stream (and, group 1, weight rows of slab + 2)
-    const bool n1_same = !last_slab;
-    const TileAt at1 = n1_same ? cur_at : next_at;
-    const int slab1 = n1_same ? slab + 1 : 0;
-    const uint32_t dead1 = (n1_same || has_next) ? 0u : 0x80000000u;
-    if constexpr (BLOCKSCALE) {
-const ScaleRow<TM> a_sc = read_scales<TM>(sa + s_rd);
-      #pragma unroll
-      for (int mt = 0; mt < TM; ++mt) s_cur[mt] = a_sc[mt] * bs;
-    }
-#pragma unroll
-    for (int t = 0; t < TN; ++t) bf[t] = read_wfrag(sa + b_frag_base, t);
-    af = read_frag(sa + a_frag_base);
-    static_for<HM>([&](auto mt_c) {
-      constexpr int mt = decltype(mt_c)::value;
-      mt_step(mt_c, sa);
-      // the copies, a few behind each 16-row group (a wave that sends its whole share at once sits in the issue queue)
-      constexpr int NP = IA + NSC + IB;  // group 0's pieces; group 1 sends the first IA + NSC of them here
-#pragma unroll
-      for (int idx = 0; idx < NP; ++idx) {
-        if (idx * HM / NP == mt) {
-          if (idx < IA) dma_a(at1, slab1, buf ^ 1, idx, dead1);
-          else if (idx < IA + NSC) dma_s(at1, slab1, buf ^ 1, dead1);
-          else dma_b(at1, slab1, buf ^ 1, idx - IA - NSC, dead1, wm == 0);
-        }
-      }
-    });
-    // ================= second half =================
-    // group 1: its weight rows of this slab's successor (copied during the last second half) have landed: group 0 reads
-    // them after this barrier.  Younger: this slab's first-half copies.  (Group 0 has nothing to wait for here.)
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IA + NSC + IB) : "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    static_for<HM>([&](auto h_c) {
-      constexpr int mt = HM + decltype(h_c)::value;
-      mt_step(std::integral_constant<int, mt>{}, sa);
-      {
-        // group 1: weight rows 128 .. 255 of slab + 2 of the stream, into this slab's own stage: every wave has its
-        // weight fragments of this slab (group 1's waves passed the barrier above after reading theirs)
-        const bool n2_same = slab + 2 < nslab;
-        const TileAt at2 = n2_same ? cur_at : next_at;
-        const int slab2 = n2_same ? slab + 2 : slab + 2 - nslab;
-        const uint32_t dead2 = (n2_same || has_next) ? 0u : 0x80000000u;
-#pragma unroll
-        for (int i = 0; i < IB; ++i)
-          if (i * HM / IB == mt - HM) dma_b(at2, slab2, buf, i, dead2, wm == 1);
-      }
-    });
-    buf ^= 1;
-    if (!last_slab) {
-      ++slab;
-      continue;
-    }
-    // ---- the tile is complete: it leaves, 16 rows of the wave's part at a time (as in persist_body)
-    if constexpr (BLOCKSCALE) {
-      if (has_next) bs_nxt = b_scales_c[(int64_t)((tn2 * BN + wn * WN) / 128) * p.b_scales_ld];
-    }
-    {
-      float b_s[TN / 2][8], a_s_all[TM];
-      if constexpr (!BLOCKSCALE) {
-#pragma unroll
-        for (int q = 0; q < TN / 2; ++q)
-#pragma unroll
-          for (int i = 0; i < 8; ++i)
-            b_s[q][i] = scale_at(p.b_scales, (int64_t)(tn * BN + wn * WN + q * 32 + lq * 8 + i) * p.b_scale_stride, p.scales_dtype);
-#pragma unroll
-        for (int mt = 0; mt < TM; ++mt)
-          a_s_all[mt] = scale_at(p.a_scales, ((int64_t)tm * BM + wm * WM + mt * 16 + lm) * p.a_scale_stride, p.scales_dtype);
-        asm volatile("" ::: "memory");
-      }
-      const uint32_t c_tile = ((uint32_t)(tm * BM + wm * WM) * (uint32_t)p.ldc + (uint32_t)(tn * BN + wn * WN)) * 2u;
-#pragma unroll
-      for (int mt = 0; mt < TM; ++mt) {
-        float a_s = 1.f;
-        if constexpr (!BLOCKSCALE) a_s = a_s_all[mt];
-#pragma unroll
-        for (int q = 0; q < TN / 2; ++q) {
-          v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
-          if constexpr (!BLOCKSCALE) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
-              lo[i] = t_lo * b_s[q][i];
-              hi[i] = t_hi * b_s[q][4 + i];
-            }
-          }
-          *reinterpret_cast<v4u*>(wbuf + lm * (WN * 2) + (((q * 4 + lq) ^ (lm & 7)) * 16)) =
-              v4u{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const int r = i * 8 + rr;
-          const v4u v = *reinterpret_cast<const v4u*>(wbuf + r * (WN * 2) + ((cc ^ (r & 7)) * 16));
-          buffer_store_b128_guarded<2>(v, c_rsrc, c_lane, c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes);
-        }
-      }
-      stored = true;
-    }
-    if (!has_next) break;
-    // ---- on to the block's next tile
-    ++k;
-    slab = 0;
-    tm = tm2;
-    tn = tn2;
-    cur_at = next_at;
-    has_next = k + 1 < njobs;
-    if (has_next) {
-      tile_coords(run_begin + my + (k + 1) * nb, tiles_m, tiles_n, tm2, tn2);
-      next_at = tile_at(tm2, tn2);
-    }
-    if constexpr (BLOCKSCALE) bs_row = b_scales_c + (int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld;
-  }
-  if (wm == 0) __builtin_amdgcn_s_barrier();  // group 1's second half of its last slab
-  // the last copies (of nothing: every lane out of range) still write zeros into the stages: they
-  // must have landed before the block's LDS goes to another block
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
-
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool BLOCKSCALE>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_persist_pp_kernel(GemmArgs p) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  persist_pp_body<BM, BN, WAVES_M, WAVES_N, BLOCKSCALE>(p, smem);
 }
 
 // ---- grouped (MoE) matmul ---------------------------------------------------------------------
@@ -2035,6 +1669,21 @@ static bool persist_ok(const GemmArgs& p, bool blockscale, dim3 grid) {
   return true;
 }
 
+// The four-wave kernel (gemm_w4.hip) for a matmul the planner gave the 256 x 256 shape: 0 (no), or the sixteen-row
+// groups per wave -- 5: tiles of 160 x 256, 6: 192 x 256.
+bool gemm_w4_ok(const GemmArgs& p, bool blockscale);
+int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, hipStream_t stream);
+static int w4_rows(int64_t M, int64_t N, int64_t K, bool blockscale) {
+  const int forced = tuning().w4;
+  if (forced >= 0) return forced;
+  (void)M; (void)N; (void)K; (void)blockscale;
+  return 0;
+}
+static int w4_choice(const GemmArgs& p, bool blockscale, int variant, dim3 grid) {
+  if (variant != 1 || grid.y != 1 || grid.z != 1 || !tuning().persist || !gemm_w4_ok(p, blockscale)) return 0;
+  return w4_rows(p.M, p.N, p.K, blockscale);
+}
+
 int compute_units() {
   static int cached[64] = {0};
   int dev = 0;
@@ -2054,13 +1703,20 @@ static int launch_persist(const GemmArgs& p, hipStream_t stream, const char* nam
   const int64_t tiles = (int64_t)(p.M / 256) * (p.N / 256);
   const int cus = compute_units();
   const dim3 grid((unsigned)(tiles < cus ? tiles : cus));
-  // (the tuning switch `pingpong` = 1 selects the form whose two halves run half a slab apart; it needs two slabs to
-  // stagger)
-  if (tuning().pingpong && p.K > 128) {
-    static PerDeviceFlag attr_pp;
-    return launch_with_lds(gemm_persist_pp_kernel<256, 256, 2, 4, BLOCKSCALE>, attr_pp, lds + 8 * 1024, 512, p, grid, stream, name);
-  }
   return launch_with_lds(gemm_persist_kernel<256, 256, 2, 4, BLOCKSCALE>, attr_done, lds, 512, p, grid, stream, name);
+}
+
+// measurement aid: the persistent kernel's main loop on operands that stay in L2 (level 1) or in LDS (level 2), on every CU
+template <bool BLOCKSCALE, int PROBE>
+static int launch_persist_probe(const GemmArgs& p, hipStream_t stream) {
+  static PerDeviceFlag attr_done;
+  constexpr int lds = tile_lds_bytes<256, 256, 2, BLOCKSCALE>() + 8 * 2048;
+  return launch_with_lds(gemm_persist_probe_kernel<256, 256, 2, 4, BLOCKSCALE, PROBE>, attr_done, lds, 512, p,
+                         dim3((unsigned)compute_units()), stream, "gemm_persist_probe");
+}
+int gemm_persist_probe(const GemmArgs& p, bool blockscale, int level, hipStream_t stream) {
+  if (level == 1) return blockscale ? launch_persist_probe<true, 1>(p, stream) : launch_persist_probe<false, 1>(p, stream);
+  return blockscale ? launch_persist_probe<true, 2>(p, stream) : launch_persist_probe<false, 2>(p, stream);
 }
 
 // The work-split form: blocks = the CUs in whole rounds of the 8 XCDs; one workspace slot of 256 KB per block.
@@ -2434,6 +2090,7 @@ static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, di
     if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false, true>(p, grid, stream, "gemm_qkv_row_256x256");
     return launch_tiled<128, 128, 2, 2, 2, false, true>(p, grid, stream, "gemm_qkv_row_128x128");
   }
+  if (const int tm = w4_choice(p, blockscale, variant, grid)) return gemm_w4_launch(p, blockscale, tm, stream);
   if (variant == 1 && persist_ok(p, blockscale, grid))
     return blockscale ? launch_persist<true>(p, stream, "gemm_persist_block_256x256") : launch_persist<false>(p, stream, "gemm_persist_row_256x256");
   if (blockscale) {

@@ -1,0 +1,475 @@
+// Scaled FP8 matmul on gfx950 with FOUR waves per block, one wave per SIMD:  C[M,N] = A[M,K] . B[N,K]^T.
+//
+// The layout of max/kernels/src/linalg/matmul/gpu/amd/amd_4wave_matmul.mojo:13-33,415-419 (a 2 x 2 grid of waves, every
+// wave alone on its SIMD with the SIMD's whole register file) built for the block-scaled sum of
+// max/kernels/src/linalg/fp8_quantization.mojo:1576-1624, whose per-slab promotion acc += P * (a_s * b_s) needs the
+// accumulators as VALU operands: a wave owns 96 x 128 of a 192 x 256 tile (192 accumulator registers, ordinary VGPRs),
+// the products of the MFMAs in flight take 16 more, and the operand fragments live in the other half of the register
+// file (AGPRs: ds_read_b128 writes them and v_mfma reads its A / B operands from them directly).  The file is compiled
+// with the MFMA results forced into VGPRs (-amdgpu-mfma-vgpr-form): left to its own choice the compiler puts them into
+// AGPRs as soon as a kernel uses any and copies every product back for the promotion.
+//
+// Against eight waves of 128 x 64 on a 256 x 256 tile: 0.58 instead of 0.75 fragment reads per MFMA, four instead of
+// eight waves at the slab's barrier, and a wave that never shares its SIMD's issue slots.
+//
+// Pipeline of a block (persistent: one block per CU walks its share of the tiles, the slab stream never stops at a tile
+// boundary).  LDS holds TWO stages of activation rows (+ the slab's activation scales) and THREE stages of weight rows:
+// weight tiles are read by one XCD at a time and come from HBM, activation tiles are read by all eight at once and mostly
+// come from the memory-side cache, so the third stage goes to the operand with the longer way.  Per slab s:
+//
+//   groups 0, 1          copies of the weight rows of slab s + 2 (stage (s + 2) % 3, free since barrier s - 1)
+//   group TM - 2         the wave reads its last activation fragment of slab s, waits for its own copies of slab s + 1
+//                        and passes THE barrier of slab s: behind it slab s + 1 is in LDS for everybody and nobody
+//                        reads slab s any more.  The wave then reads the weight fragments, the first activation
+//                        fragment and the activation scales of slab s + 1 into its second set of fragment registers,
+//                        so that the first MFMA of slab s + 1 follows the last one of slab s without a wait for LDS.
+//   group TM - 1         copies of the activation rows (and scales) of slab s + 2 into the stage slab s has left
+//
+// Vector memory operations of a wave complete in order: at barrier s the wave may still have the PER_B weight copies of
+// slab s + 2 in flight (and, behind a tile's last slab, the tile's NSTORE stores of C, which sit between the activation
+// copies and those weight copies in issue order), so the waits are exact counts.
+//
+// Promotion: the MFMA of (16-row group mt, fragment nt) writes a fresh product, and the four FMAs that fold it into the
+// accumulators are issued LAG MFMAs later, when the product has left the matrix pipe.
+//
+// Tiles: whole 256-column tiles of C, any M (rows past M read as zero through the buffer descriptor and their stores fall
+// outside C's descriptor), K in an even number of 128-byte slabs (the two sets of fragment registers alternate).
+// Sums are formed in the same order as by the eight-wave kernels (one product per slab, promoted in slab order):
+// results are bit-equal to theirs.
+#include <stdlib.h>
+
+#include "common.h"
+#include "gemm_args.h"
+#include "gemm_device.h"
+#include "tuning.h"
+
+namespace maxfp8 {
+
+int compute_units();
+
+// a scalar load (the address is the same in every lane): through the constant address space, so that it does not
+// take a place in the wave's queue of vector memory operations, whose in-order completion the copy waits count on
+__device__ __forceinline__ float scalar_load_f32(const float* ptr) {
+  typedef __attribute__((address_space(4))) const float* const_ptr_t;
+  return *(const_ptr_t)(uintptr_t)ptr;
+}
+
+// A fragment belongs in the accumulation registers: the load writes them, the MFMA reads them, nothing else touches it.
+// (Without the hint the allocator fills the ordinary registers with fragments first and then spills accumulators.)
+__device__ __forceinline__ v8i in_agprs(v8i f) {
+  asm("" : "+a"(f));
+  return f;
+}
+
+// PROBE (measurement aid, results meaningless): 0 the matmul; 1 the same loop with every copy reading tile (0, 0) and
+// slabs 0..7 over and over, so that its operands stay in L2; 2 the same without copies, waits and barriers -- the
+// MFMA loop on what the prologue left in LDS.
+template <int TM, int TN, bool BLOCKSCALE, int PROBE>
+__device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
+  constexpr int WM = TM * 16, WN = TN * 16, BM = 2 * WM, BN = 2 * WN;
+  constexpr int IA = BM / 32, IB = BN / 32;                  // copy instructions per wave and slab (8 rows each)
+  constexpr int SCALE_BYTES = BLOCKSCALE ? 1024 : 0;         // 2 wave rows x 16 lane rows x 8 words
+  constexpr int A_STAGE = BM * 128 + SCALE_BYTES, B_STAGE = BN * 128;
+  constexpr int B_BASE = 2 * A_STAGE, SIDE_BASE = B_BASE + 3 * B_STAGE, SIDE_BYTES = 2048;
+  constexpr int PER_A = IA + (BLOCKSCALE ? 1 : 0), PER_B = IB;
+  constexpr int NSTORE = TM * TN / 2;                        // 16-byte stores per lane and tile
+  constexpr int LAG = 3;                                     // a product is folded in LAG MFMAs after its own
+  static_assert(TN == 8 && TM >= 3 && TM <= 8, "wave tile");
+  static_assert(PER_B + NSTORE < 64, "the count must fit the vmcnt field");
+  static_assert(IB % 2 == 0, "the weight copies go out in two halves");
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lm = lane & 15, lq = lane >> 4;
+  const int nslab = p.K / 128;                               // whole slabs, an even number of them (the host's rule)
+
+  // ---- this block's tiles: every nb-th tile of its XCD's contiguous run (blocks are dealt to the XCDs round-robin)
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = p.N / BN, total = tiles_m * tiles_n;
+  const int xcd = blockIdx.x & 7;
+  const int run_begin = xcd * (total >> 3) + (xcd < (total & 7) ? xcd : (total & 7));
+  const int run_len = (total >> 3) + (xcd < (total & 7) ? 1 : 0);
+  const int nb = ((int)gridDim.x - xcd + 7) >> 3;
+  const int my = blockIdx.x >> 3;
+  const int njobs = PROBE ? 1 : (my < run_len ? (run_len - my + nb - 1) / nb : 0);
+  if (njobs <= 0) return;
+
+  // ---- global -> LDS copy plan (LDS-DMA, 16 bytes per lane, 8 rows x 128 bytes per instruction; lane (r, p) fetches
+  // the chunk p ^ f(row) of its row, so the bytes land swizzled for conflict-free fragment reads)
+  const __amdgpu_buffer_rsrc_t a_rsrc = t2_rsrc(p.a, t2_clamp_u32((int64_t)(p.M - 1) * p.lda + p.K));
+  const __amdgpu_buffer_rsrc_t b_rsrc = t2_rsrc(p.b, t2_clamp_u32((int64_t)(p.N - 1) * p.ldb + p.K));
+  const int cr = lane >> 3, cp = lane & 7;
+  const int cchunk = cp ^ cr;
+  const int cchunk_b = cp ^ (((wave & 1) << 2) | (cr & 3));
+  const uint32_t a_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.lda + cchunk * 16;
+  const uint32_t b_voff = (uint32_t)(wave * 8 + cr) * (uint32_t)p.ldb + cchunk_b * 16;
+  const uint32_t a_istep = 32u * (uint32_t)p.lda, b_istep = 32u * (uint32_t)p.ldb;
+  // the slab's activation scales: word wm * 128 + lm * 8 + mt of the scale area holds the scale of row wm * WM + mt * 16
+  // + lm, so that a lane finds its TM scales in 32 consecutive bytes; wave w copies words [64 w, 64 w + 64)
+  __amdgpu_buffer_rsrc_t s_rsrc = t2_rsrc(nullptr, 0);
+  uint32_t s_voff = 0, s_slab_step = 0;
+  if constexpr (BLOCKSCALE) {
+    s_rsrc = t2_rsrc(p.a_scales, t2_clamp_u32(((int64_t)(nslab - 1) * p.a_scales_ld + p.M) * 4));
+    const int word = wave * 64 + lane, mt_w = word & 7, lm_w = (word >> 3) & 15, wm_w = word >> 7;
+    s_voff = (uint32_t)(wm_w * WM + mt_w * 16 + lm_w) * 4u;
+    if (mt_w >= TM) s_voff = 0x80000000u;
+    s_slab_step = (uint32_t)p.a_scales_ld * 4u;
+  }
+  struct TileAt { uint32_t a, b, s; };  // byte offsets of a tile's activation rows, weight rows and activation scales
+  auto tile_at = [&](int tm, int tn) {
+    if constexpr (PROBE != 0) return TileAt{0u, 0u, 0u};
+    return TileAt{(uint32_t)(tm * BM) * (uint32_t)p.lda, (uint32_t)(tn * BN) * (uint32_t)p.ldb, (uint32_t)(tm * BM) * 4u};
+  };
+  // copy number idx (0 .. PER_A - 1) of a slab's activation rows and scales into activation stage `stage`
+  // Where a slab's copies read: the scalar offsets of its first activation, weight and scale copy.  A slab of nothing
+  // (behind the block's last tile) gets offsets past 2^31: the scalar offset takes part in the descriptor's range
+  // check, so such copies write zeros.  (K is a whole number of slabs: no lane ever reads past a row's end.)
+  struct SlabAt { uint32_t a, b, s; };
+  auto slab_at = [&](const TileAt& at, int slab, uint32_t dead) {
+    if constexpr (PROBE != 0) slab &= 7;
+    const uint32_t koff = (uint32_t)slab * 128u;
+    return SlabAt{(at.a + koff) | dead, (at.b + koff) | dead, (at.s + (uint32_t)slab * s_slab_step) | dead};
+  };
+  // copy number idx (0 .. PER_A - 1) of a slab's activation rows and scales into activation stage `stage`
+  auto dma_a = [&](const SlabAt& at, int stage, int idx) {
+    uint8_t* sa = smem + stage * A_STAGE;
+    if (idx < IA) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(sa + (idx * 4 + wave) * 1024), 16, a_voff, at.a + idx * a_istep, 0, 0);
+    } else if constexpr (BLOCKSCALE) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(s_rsrc, (lds_ptr_t)(sa + BM * 128 + wave * 256), 4, s_voff, at.s, 0, 0);
+    }
+  };
+  // copy number idx (0 .. PER_B - 1) of a slab's weight rows into weight stage `stage`
+  auto dma_b = [&](const SlabAt& at, int stage, int idx) {
+    uint8_t* sb = smem + B_BASE + stage * B_STAGE;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(sb + (idx * 4 + wave) * 1024), 16, b_voff, at.b + idx * b_istep, 0, 0);
+  };
+
+  // ---- fragment read plan.  Activation fragment mt: rows mt * 16 + lm of the wave's rows.  Weight fragments come in
+  // pairs over 32 weight rows, MFMA row i <-> weight row 8 * (i / 4) + i % 4 (+ 4 for the odd fragment), which leaves a
+  // lane with 8 consecutive columns of C per pair.
+  const int sw = lm & 7;
+  const uint8_t* a_frag = smem + (uint32_t)(wm * WM) * 128 + lm * 128;
+  const uint32_t a_lo = (uint32_t)((lq ^ sw) << 4), a_hi = (uint32_t)(((lq + 4) ^ sw) << 4);
+  auto read_afrag = [&](int stage, int mt) -> v8i {
+    const uint8_t* g = a_frag + stage * A_STAGE + mt * 2048;
+    const v4i lo = *reinterpret_cast<const v4i*>(g + a_lo);
+    const v4i hi = *reinterpret_cast<const v4i*>(g + a_hi);
+    return in_agprs(v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w});
+  };
+  const int wrow = 8 * (lm >> 2) + (lm & 3);
+  const int wsw = (((wrow >> 3) & 1) << 2) | (wrow & 3);
+  const uint8_t* b_frag = smem + B_BASE + (uint32_t)(wn * WN) * 128 + wrow * 128;
+  const uint32_t b_lo = (uint32_t)((lq ^ wsw) << 4), b_hi = (uint32_t)(((lq + 4) ^ wsw) << 4);
+  auto read_bfrag = [&](int stage, int t) -> v8i {
+    const uint8_t* g = b_frag + stage * B_STAGE + (t >> 1) * 4096 + (t & 1) * 512;
+    const v4i lo = *reinterpret_cast<const v4i*>(g + b_lo);
+    const v4i hi = *reinterpret_cast<const v4i*>(g + b_hi);
+    return in_agprs(v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w});
+  };
+  struct Scales { float v[TM]; };
+  const uint8_t* s_rd = smem + BM * 128 + (wm * 128 + lm * 8) * 4;
+  auto read_scales = [&](int stage) -> Scales {
+    Scales out;
+    const v4f lo = *reinterpret_cast<const v4f*>(s_rd + stage * A_STAGE);
+    out.v[0] = lo[0]; out.v[1] = lo[1]; out.v[2] = lo[2]; out.v[3] = lo[3];
+    if constexpr (TM > 6) {
+      const v4f hi = *reinterpret_cast<const v4f*>(s_rd + stage * A_STAGE + 16);
+      out.v[4] = hi[0]; out.v[5] = hi[1]; out.v[6] = hi[2];
+      if constexpr (TM > 7) out.v[7] = hi[3];
+    } else if constexpr (TM > 5) {
+      const v2f hi = *reinterpret_cast<const v2f*>(s_rd + stage * A_STAGE + 16);
+      out.v[4] = hi[0]; out.v[5] = hi[1];
+    } else if constexpr (TM > 4) {
+      out.v[4] = *reinterpret_cast<const float*>(s_rd + stage * A_STAGE + 16);
+    }
+    return out;
+  };
+
+  // ---- where C goes: through a 2 KB side buffer per wave, 16 rows x 64 columns at a time, so that a store instruction
+  // writes 8 rows x one whole 128-byte line
+  uint8_t* wbuf = smem + SIDE_BASE + wave * SIDE_BYTES;
+  const __amdgpu_buffer_rsrc_t c_rsrc = t2_rsrc(p.c, t2_clamp_u32(((int64_t)(p.M - 1) * p.ldc + p.N) * 2));
+  const uint32_t c_row_bytes = (uint32_t)p.ldc * 2u;
+
+  // ---- prologue: slabs 0 and 1 of the first tile
+  int tm, tn;
+  tile_coords(run_begin + my, tiles_m, tiles_n, tm, tn);
+  if constexpr (PROBE != 0) tm = tn = 0;
+  TileAt cur_at = tile_at(tm, tn);
+  {
+    const SlabAt s0 = slab_at(cur_at, 0, 0u), s1 = slab_at(cur_at, 1, 0u);
+#pragma unroll
+    for (int idx = 0; idx < PER_A; ++idx) dma_a(s0, 0, idx);
+#pragma unroll
+    for (int idx = 0; idx < PER_B; ++idx) dma_b(s0, 0, idx);
+#pragma unroll
+    for (int idx = 0; idx < PER_A; ++idx) dma_a(s1, 1, idx);
+#pragma unroll
+    for (int idx = 0; idx < PER_B; ++idx) dma_b(s1, 1, idx);
+  }
+  if constexpr (PROBE == 2) {
+    const SlabAt s2 = slab_at(cur_at, 2, 0u);
+#pragma unroll
+    for (int idx = 0; idx < PER_B; ++idx) dma_b(s2, 2, idx);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_A + PER_B) : "memory");
+  }
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  const int bs_blk = 2 * tn + wn;  // (BN = 256: two weight-scale blocks per tile, one per wave column)
+  float bs_nxt = 1.f;
+  if constexpr (BLOCKSCALE) bs_nxt = scalar_load_f32(p.b_scales + (int64_t)(PROBE ? wn : bs_blk) * p.b_scales_ld);
+
+  v8i bf[2][TN], af0[2];
+  Scales sraw[2];
+#pragma unroll
+  for (int t = 0; t < TN; ++t) bf[0][t] = read_bfrag(0, t);
+  af0[0] = read_afrag(0, 0);
+  if constexpr (BLOCKSCALE) sraw[0] = read_scales(0);
+
+  int bst = 0;          // weight stage of the slab being multiplied
+  bool stored = false;  // a tile's stores sit in front of the weight copies now in flight
+  for (int k = 0; k < njobs; ++k) {
+    const bool has_next = k + 1 < njobs;
+    int tm2 = tm, tn2 = tn;
+    if (has_next) tile_coords(run_begin + my + (k + 1) * nb, tiles_m, tiles_n, tm2, tn2);
+    const TileAt next_at = tile_at(tm2, tn2);
+    const uint32_t next_dead = has_next ? 0u : 0x80000000u;
+    const float* bs_row = nullptr;
+    if constexpr (BLOCKSCALE) bs_row = p.b_scales + (int64_t)(PROBE ? wn : 2 * tn + wn) * p.b_scales_ld;
+    const float* bs_row2 = nullptr;
+    if constexpr (BLOCKSCALE) bs_row2 = p.b_scales + (int64_t)(PROBE ? wn : 2 * tn2 + wn) * p.b_scales_ld;
+
+    v4f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    // one slab; PAR = its parity = its activation stage = the set of fragment registers it multiplies from
+    // (AFTER_STORES: the tile before this one has just been stored -- only a tile's first slab can be that.  A template
+    // flag and not a branch at the wait: a branch there would cut the slab's straight-line code in two, and the compiler
+    // schedules each part on its own -- it then issued forty MFMAs in a row and parked their products in AGPRs)
+    auto slab_body = [&](auto PAR_C, auto AFTER_STORES_C, const int slab) {
+      constexpr int PAR = decltype(PAR_C)::value;
+      constexpr bool AFTER_STORES = decltype(AFTER_STORES_C)::value;
+      // slab + 2 of this tile, or slab (+ 2 - nslab) of the next one
+      const bool over = slab + 2 >= nslab;
+      const SlabAt dat = slab_at(over ? next_at : cur_at, over ? slab + 2 - nslab : slab + 2, over ? next_dead : 0u);
+      const int bst1 = bst == 2 ? 0 : bst + 1, bst2 = bst == 0 ? 2 : bst - 1;  // stages of slabs s + 1 and s + 2
+
+      float s_cur[TM];
+      if constexpr (BLOCKSCALE) {
+        const float bs = bs_nxt;
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) s_cur[mt] = sraw[PAR].v[mt] * bs;
+        // the weight-block scale of the next slab (of the next tile behind this tile's last slab)
+        const int ps = PROBE ? ((slab + 1) & 7) : slab + 1;
+        bs_nxt = scalar_load_f32(slab + 1 < nslab ? bs_row + ps : bs_row2);
+      }
+      v8i af = af0[PAR];
+      [[maybe_unused]] v4f part[LAG + 1];
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        v8i af_next = af;
+        if (mt + 1 < TM) af_next = read_afrag(PAR, mt + 1);
+#pragma unroll
+        for (int nt = 0; nt < TN; ++nt) {
+          if constexpr (BLOCKSCALE) {
+            constexpr v4f zero = {0.f, 0.f, 0.f, 0.f};
+            const int i = mt * TN + nt;
+            part[i % (LAG + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[PAR][nt], af, zero, 0, 0, 0, 0, 0, 0);
+            // issue order, pinned: one MFMA, then the four FMAs of the product that left the pipe LAG MFMAs ago
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i >= LAG) {
+              const int j = i - LAG;
+              acc[j / TN][j % TN] += part[j % (LAG + 1)] * s_cur[j / TN];
+              __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+            }
+          } else {
+            acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[PAR][nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
+          }
+        }
+        if constexpr (PROBE != 2) {
+          // weight rows of slab s + 2, in two halves
+          if (mt < 2) {
+#pragma unroll
+            for (int idx = mt * (PER_B / 2); idx < (mt + 1) * (PER_B / 2); ++idx) dma_b(dat, bst2, idx);
+          }
+        }
+        if (mt == TM - 2) {
+          // the slab's last fragment read is out: wait for it and for this wave's copies of slab s + 1, then the barrier
+          if constexpr (PROBE != 2) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_B + (AFTER_STORES ? NSTORE : 0)) : "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+          }
+          // the first fragments of slab s + 1
+#pragma unroll
+          for (int t = 0; t < TN; ++t) bf[PAR ^ 1][t] = read_bfrag(bst1, t);
+          af0[PAR ^ 1] = read_afrag(PAR ^ 1, 0);
+          if constexpr (BLOCKSCALE) sraw[PAR ^ 1] = read_scales(PAR ^ 1);
+        }
+        if constexpr (PROBE != 2) {
+          // activation rows and scales of slab s + 2 into the stage this slab has left
+          if (mt == TM - 1) {
+#pragma unroll
+            for (int idx = 0; idx < PER_A; ++idx) dma_a(dat, PAR, idx);
+          }
+        }
+        af = af_next;
+      }
+      if constexpr (BLOCKSCALE) {
+#pragma unroll
+        for (int j = TM * TN - LAG; j < TM * TN; ++j) acc[j / TN][j % TN] += part[j % (LAG + 1)] * s_cur[j / TN];
+      }
+      bst = bst1;
+    };
+
+    constexpr std::integral_constant<int, 0> EVEN{};
+    constexpr std::integral_constant<int, 1> ODD{};
+    if (stored) slab_body(EVEN, std::true_type{}, 0);
+    else slab_body(EVEN, std::false_type{}, 0);
+    slab_body(ODD, std::false_type{}, 1);
+    for (int slab = 2; slab < nslab; slab += 2) {
+      slab_body(EVEN, std::false_type{}, slab);
+      slab_body(ODD, std::false_type{}, slab + 1);
+    }
+
+    // ---- the tile leaves, 16 rows x 64 columns of the wave's part at a time
+    // (row scaling: every scale of the tile is loaded before the first store, so that no later wait for a load also
+    // waits for the stores in front of it)
+    float b_s[TN / 2][8], a_s_all[TM];
+    if constexpr (!BLOCKSCALE) {
+#pragma unroll
+      for (int q = 0; q < TN / 2; ++q)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          b_s[q][i] = scale_at(p.b_scales, (int64_t)(tn * BN + wn * WN + q * 32 + lq * 8 + i) * p.b_scale_stride, p.scales_dtype);
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        int64_t m = (int64_t)tm * BM + wm * WM + mt * 16 + lm;
+        if (m >= p.M) m = p.M - 1;
+        a_s_all[mt] = scale_at(p.a_scales, m * p.a_scale_stride, p.scales_dtype);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    const uint32_t c_tile = ((uint32_t)(tm * BM + wm * WM) * (uint32_t)p.ldc + (uint32_t)(tn * BN + wn * WN)) * 2u;
+    // (the lane's offsets are formed here, out of sight of the optimiser: hoisted out of the tile loop they would sit in
+    // vector registers all through the slab loop, which has none to spare)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int lm_e = lane_e & 15, lq_e = lane_e >> 4, rr = lane_e >> 3, cc = lane_e & 7;
+    const uint32_t c_lane = (uint32_t)rr * c_row_bytes + (uint32_t)cc * 16u;
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) {
+      float a_s = 1.f;
+      if constexpr (!BLOCKSCALE) a_s = a_s_all[mt];
+#pragma unroll
+      for (int h = 0; h < TN / 4; ++h) {
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq) {
+          const int q = 2 * h + qq;
+          v4f lo = acc[mt][2 * q], hi = acc[mt][2 * q + 1];
+          if constexpr (!BLOCKSCALE) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float t_lo = lo[i] * a_s, t_hi = hi[i] * a_s;
+              lo[i] = t_lo * b_s[q][i];
+              hi[i] = t_hi * b_s[q][4 + i];
+            }
+          }
+          // (written and read back through the same vector type: to the compiler a store through one type and a load
+          // through another need not alias, and it may then move the load in front of the store)
+          *reinterpret_cast<v4u_t*>(wbuf + lm_e * 128 + (((qq * 4 + lq_e) ^ (lm_e & 7)) * 16)) =
+              v4u_t{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
+        }
+        // (a wave reads back only what it wrote itself, and its LDS operations execute in order)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int r = i * 8 + rr;
+          const v4u_t v = *reinterpret_cast<const v4u_t*>(wbuf + r * 128 + ((cc ^ (r & 7)) * 16));
+          // (non-temporal: C is not read again here, and its lines should not push the operands out of L2)
+          buffer_store_b128_guarded<2>(v, c_rsrc, c_lane, c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes + (uint32_t)h * 128u);
+        }
+      }
+    }
+    stored = true;
+    tm = tm2;
+    tn = tn2;
+    cur_at = next_at;
+  }
+  // the last copies (of nothing: every lane out of range) still write zeros into the stages: they must have landed
+  // before the block's LDS goes to another block
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+template <int TM, int TN, bool BLOCKSCALE, int PROBE>
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_w4_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  w4_body<TM, TN, BLOCKSCALE, PROBE>(p, smem);
+}
+
+template <int TM, int TN, bool BLOCKSCALE>
+constexpr int w4_lds_bytes() {
+  return 2 * (TM * 32 * 128 + (BLOCKSCALE ? 1024 : 0)) + 3 * (TN * 32 * 128) + 4 * 2048;
+}
+
+// The shapes this kernel takes: bf16 C with 16-byte aligned rows, whole 256-column tiles, K a whole and even number of
+// slabs, operands whose byte offsets fit 31 bits (a tile's position rides in the copies' scalar offset).
+bool gemm_w4_ok(const GemmArgs& p, bool blockscale) {
+  if (p.M <= 0 || p.N <= 0 || p.N % 256 != 0 || p.K < 256 || p.K % 256 != 0) return false;
+  const int64_t nslab = p.K / 128;
+  if (p.kv_on || p.splits > 1) return false;
+  if (p.c_dtype != MAXFP8_BF16 || !p.c_vec8_ok) return false;
+  const int64_t lim = 0x7ff00000ll;
+  const int64_t rows = ceil_div(p.M, 192) * 192 + 192;
+  if (rows * p.lda >= lim || (int64_t)p.N * p.ldb >= lim) return false;
+  if (blockscale && (nslab * p.a_scales_ld + rows) * 4 >= lim) return false;
+  if (rows * p.ldc * 2 >= lim) return false;
+  return true;
+}
+
+template <int TM, bool BLOCKSCALE, int PROBE>
+static int launch_w4(const GemmArgs& p, unsigned blocks, hipStream_t stream, const char* name) {
+  static PerDeviceFlag attr_done;
+  constexpr int lds = w4_lds_bytes<TM, 8, BLOCKSCALE>();
+  static_assert(lds <= 160 * 1024, "one block's LDS");
+  auto kern = gemm_w4_kernel<TM, 8, BLOCKSCALE, PROBE>;
+  bool& done = attr_done.here();
+  if (!done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, lds, hipGetErrorString(e));
+    done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, stream, p);
+  return launch_status(name);
+}
+
+// rows of a tile: 32 * tm (tm = 5 or 6 sixteen-row groups per wave)
+int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, hipStream_t stream) {
+  const int64_t tiles = ceil_div(p.M, 32 * tm) * (p.N / 256);
+  const int cus = compute_units();
+  const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+  if (tm == 5)
+    return blockscale ? launch_w4<5, true, 0>(p, blocks, stream, "gemm_w4_block_160x256") : launch_w4<5, false, 0>(p, blocks, stream, "gemm_w4_row_160x256");
+  return blockscale ? launch_w4<6, true, 0>(p, blocks, stream, "gemm_w4_block_192x256") : launch_w4<6, false, 0>(p, blocks, stream, "gemm_w4_row_192x256");
+}
+
+// measurement aid: the kernel's main loop on operands that stay in L2 (level 1) or in LDS (level 2), on every CU
+int gemm_w4_probe(const GemmArgs& p, bool blockscale, int level, int tm, hipStream_t stream) {
+  const unsigned blocks = (unsigned)compute_units();
+  const char* name = "gemm_w4_probe";
+  if (tm == 5) {
+    if (level == 1) return blockscale ? launch_w4<5, true, 1>(p, blocks, stream, name) : launch_w4<5, false, 1>(p, blocks, stream, name);
+    return blockscale ? launch_w4<5, true, 2>(p, blocks, stream, name) : launch_w4<5, false, 2>(p, blocks, stream, name);
+  }
+  if (level == 1) return blockscale ? launch_w4<6, true, 1>(p, blocks, stream, name) : launch_w4<6, false, 1>(p, blocks, stream, name);
+  return blockscale ? launch_w4<6, true, 2>(p, blocks, stream, name) : launch_w4<6, false, 2>(p, blocks, stream, name);
+}
+
+}  // namespace maxfp8

@@ -7,8 +7,8 @@
 //   MAXFP8_SPLITK=n            force the K split of the tiled matmul
 //   MAXFP8_ONE_REGION=1        never cut a matmul into two regions
 //   MAXFP8_PERSIST=0           per-tile kernels instead of the persistent one
-//   MAXFP8_PINGPONG=1          persistent kernel: the block's two halves half a slab apart (a barrier every half slab)
-//                              instead of one barrier per slab for the whole block; same sums, measured 2 % slower
+//   MAXFP8_W4=0 / 5 / 6        whole-tile matmuls: the four-wave kernel never / in 160 x 256 / in 192 x 256 tiles
+//                              (default: where the cost model says it pays)
 //   MAXFP8_STREAMK=0 / 2       never / always split the work of whole-tile matmuls evenly over the blocks
 //                              (default 1: where the cost model says it pays)
 //   MAXFP8_BIG_ROWS=n          grouped: slots with at least n rows use the large-tile launch (1024)
@@ -26,7 +26,7 @@ struct Tuning {
   int splitk = 0;
   bool one_region = false;
   bool persist = true;
-  bool pingpong = false;
+  int w4 = -1;               // -1: the planner decides
   int streamk = 1;
   int big_rows = 1024;
   bool grouped_persist = true;

@@ -201,16 +201,17 @@ def test_two_region_launch(dev, tune, M, K, N, kind):
 PERSIST_SHAPES = [(512, 512, 256), (4096, 8192, 256), (2560, 7680, 384), (8192, 8192, 128), (1024, 4096, 144), (256, 256, 1024)]
 
 
-# Its second form (MAXFP8_PINGPONG=1: the block's two halves run half a slab apart, a barrier every half slab) makes
-# the same sums in the same order and is held to the same bits.
-FORMS = {"one barrier per slab": None, "halves half a slab apart": "1"}
+# The four-wave kernel (MAXFP8_W4=5 / 6: 160 x 256 / 192 x 256 tiles, one wave per SIMD; it takes the shapes whose K is an
+# even number of slabs and leaves the others to the eight-wave kernel) makes the same sums in the same order and is held
+# to the same bits.
+FORMS = {"eight waves": "0", "four waves, 160 rows": "5", "four waves, 192 rows": "6"}
 
 
 @pytest.mark.parametrize("M,N,K", PERSIST_SHAPES)
 @pytest.mark.parametrize("kind", ["block", "row"])
 @pytest.mark.parametrize("form", list(FORMS))
 def test_persistent_kernel_equals_per_tile_kernel(dev, tune, M, N, K, kind, form):
-    tune(MAXFP8_TILE="1", MAXFP8_PINGPONG=FORMS[form])
+    tune(MAXFP8_TILE="1", MAXFP8_W4=FORMS[form])
     if kind == "block":
         a, b, sa, sb = make_block(M, N, K, seed=M + K)
         cfg = BLK
@@ -234,7 +235,7 @@ def test_persistent_kernel_equals_per_tile_kernel(dev, tune, M, N, K, kind, form
 @pytest.mark.parametrize("M,N,K", [(512, 768, 384), (2560, 7680, 144)])
 @pytest.mark.parametrize("form", list(FORMS))
 def test_persistent_kernel_exact(dev, tune, M, N, K, form):
-    tune(MAXFP8_TILE="1", MAXFP8_PINGPONG=FORMS[form])
+    tune(MAXFP8_TILE="1", MAXFP8_W4=FORMS[form])
     a, b, sa, sb, want = exact_case(M, N, K, seed=M + N + K)
     cb = mm(a, b, sa, sb, BLK, dev, out=torch.bfloat16, algo="tiled")
     assert torch.equal(cb.cpu(), torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16))
@@ -253,7 +254,7 @@ def test_persistent_kernel_leaves_other_outputs_alone(dev, tune):
 def test_persistent_kernel_many_tiles_per_block_repeated(dev, tune, form):
     # short K, sixteen tiles per block: the stores of one tile are still in flight when the next tile's first slab
     # is waited for.  Twelve launches with fresh activations, each compared with the per-tile kernel.
-    tune(MAXFP8_TILE="1", MAXFP8_PINGPONG=FORMS[form])
+    tune(MAXFP8_TILE="1", MAXFP8_W4=FORMS[form])
     M, N, K = 8192, 32768, 256
     b = synth.random_fp8((N, K), 77).to(dev)
     sb = synth.random_scales((N // 128, K // 128), 78).to(dev)
