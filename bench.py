@@ -375,13 +375,14 @@ def mfma_ceiling(slabs=4096, reps=20, settle_s=0.5):
     b_s = synth.random_scales((2, 8), 4).to(dev)
     c = torch.empty((256, 256), dtype=torch.bfloat16, device=dev)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
+    clocks = torch.zeros((cus, 2), dtype=torch.int64, device=dev)
     first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for kernel, (label, rows) in MFMA_CEILING_KERNELS.items():
         for block in (0, 1):
             for level in (2, 1):
                 def launch(n):
                     _lib.check(L.maxfp8_mfma_issue_probe(kernel, block, level, n, a.data_ptr(), b.data_ptr(), a_s.data_ptr(),
-                                                         b_s.data_ptr(), c.data_ptr(), stream))
+                                                         b_s.data_ptr(), c.data_ptr(), clocks.data_ptr(), stream))
                 t_end = time.perf_counter() + settle_s   # the clocks of an idle GPU take tenths of a second to settle
                 while time.perf_counter() < t_end:
                     launch(slabs)
@@ -393,11 +394,17 @@ def mfma_ceiling(slabs=4096, reps=20, settle_s=0.5):
                 torch.cuda.synchronize()
                 us_slab = first.elapsed_time(last) * 1e3 / reps / slabs
                 flops_slab = 2.0 * rows * 256 * 128 * cus
+                # the last launch's counters: core-clock cycles over 100 MHz ticks = the clock held in the slab loop;
+                # an MFMA of this shape occupies its SIMD's matrix pipe for 32 cycles
+                cyc, ticks = clocks[:, 0].double().mean().item(), clocks[:, 1].double().mean().item()
+                ghz = cyc / ticks * 0.1
+                busy = (rows // 4) * 32.0 * slabs / cyc   # rows / 4 MFMAs per SIMD and slab
                 yield {"kernel": label, "scaling": "block" if block else "row",
                        "level": "MFMA loop on LDS-resident operands" + (" + promotions" if block else "") if level == 2 else
                                 "whole loop (copies, waits, barriers), operands in L2",
                        "us_per_slab": round(us_slab, 4), "TFLOP/s": round(flops_slab / us_slab / 1e6, 1),
-                       "frac_of_peak": round(flops_slab / us_slab / 1e6 / PEAK_FP8_TFLOPS, 3), "slabs": slabs, "launches": reps,
+                       "frac_of_peak": round(flops_slab / us_slab / 1e6 / PEAK_FP8_TFLOPS, 3),
+                       "core_clock_GHz": round(ghz, 3), "matrix_pipe_busy": round(busy, 3), "slabs": slabs, "launches": reps,
                        "blocks": cus}
 
 

@@ -485,11 +485,13 @@ int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t
  *   level 1: the whole loop -- LDS-DMA copies, waits, barriers -- with operands that stay in L2 (slabs 0..7 of tile
  *            (0, 0) over and over).
  * a, b: 256 rows x 1024 bytes of e4m3fn each; a_scales: 8 x 256 floats, b_scales: 2 x 8 floats; c: 256 x 256 bf16, written
- * once at the end with meaningless values.  The kernel's time over slabs * 256 * 256 * 128 * 2 flops per block (four waves:
+ * once at the end with meaningless values; clocks: null, or two 64-bit words per compute unit, which receive what the
+ * block's first wave counted around its slab loop -- cycles of the core clock and ticks of the constant 100 MHz clock --
+ * so that the clock the chip held under the load can be read off.  The kernel's time over slabs * 256 * 256 * 128 * 2 flops per block (four waves:
  * 160 or 192 rows) is the issue ceiling the matmul kernels are measured against.
  */
 int maxfp8_mfma_issue_probe(int kernel, int blockscale, int level, int64_t slabs, const void* a, const void* b, const float* a_scales,
-                            const float* b_scales, void* c, void* stream);
+                            const float* b_scales, void* c, uint64_t* clocks, void* stream);
 
 #ifdef __cplusplus
 }

@@ -125,7 +125,7 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_decode_weight_read_probe.restype = ci
     L.maxfp8_decode_weight_read_probe.argtypes = [vp, i64, i64, i64, i64, vp]
     L.maxfp8_mfma_issue_probe.restype = ci
-    L.maxfp8_mfma_issue_probe.argtypes = [ci, ci, ci, i64, vp, vp, vp, vp, vp, vp]
+    L.maxfp8_mfma_issue_probe.argtypes = [ci, ci, ci, i64, vp, vp, vp, vp, vp, vp, vp]
     _lib = L
     return L
 

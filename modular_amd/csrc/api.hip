@@ -761,8 +761,9 @@ int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t
 }
 
 int maxfp8_mfma_issue_probe(int kernel, int blockscale, int level, int64_t slabs, const void* a, const void* b, const float* a_scales,
-                            const float* b_scales, void* c, void* stream) {
+                            const float* b_scales, void* c, uint64_t* clocks, void* stream) {
   if (!a || !b || !c || !a_scales || !b_scales) MAXFP8_FAIL(MAXFP8_ERR_NULL, "issue probe: null pointer");
+  if (clocks && !is_aligned(clocks, 8)) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "issue probe: clocks must be 8-byte aligned");
   if ((kernel != 0 && kernel != 5 && kernel != 6) || (level != 1 && level != 2) || slabs < 8 || slabs > (1 << 22) || slabs % 2 != 0)
     MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "issue probe: kernel 0 / 5 / 6, level 1 / 2, an even number of slabs in [8, 2^22]");
   if (!is_aligned(a, 16) || !is_aligned(b, 16) || !is_aligned(c, 16)) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "issue probe: 16-byte aligned buffers");
@@ -781,6 +782,7 @@ int maxfp8_mfma_issue_probe(int kernel, int blockscale, int level, int64_t slabs
   p.scales_dtype = MAXFP8_F32;
   p.c_vec_ok = 1; p.c_vec8_ok = 1;
   p.splits = 1;
+  p.workspace = reinterpret_cast<float*>(clocks);
   return kernel == 0 ? gemm_persist_probe(p, blockscale != 0, level, (hipStream_t)stream) : gemm_w4_probe(p, blockscale != 0, level, kernel, (hipStream_t)stream);
 }
 

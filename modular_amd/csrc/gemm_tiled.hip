@@ -814,6 +814,12 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
   float bs_nxt = 1.f;
   if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn * BN + wn * WN) / 128) * p.b_scales_ld + cur.s0];
 
+  // (probe: the core clock's cycle counter and the constant 100 MHz counter, around the slab loop)
+  [[maybe_unused]] uint64_t probe_c0 = 0, probe_r0 = 0;
+  if constexpr (PROBE != 0) {
+    probe_c0 = clock64();
+    probe_r0 = wall_clock64();
+  }
   int buf = 0;
   bool stored = false;  // the wave's last vector memory operations are a tile's NSTORE stores
   for (int k = 0; k < njobs; ++k) {
@@ -937,6 +943,13 @@ const ScaleRow<TM> a_sc = read_scales<TM>(sa + s_rd);
         }
       }
       buf ^= 1;
+    }
+    if constexpr (PROBE != 0) {
+      if (p.workspace != nullptr && tid == 0) {
+        uint64_t* out = reinterpret_cast<uint64_t*>(p.workspace) + 2 * blockIdx.x;
+        out[0] = clock64() - probe_c0;
+        out[1] = wall_clock64() - probe_r0;
+      }
     }
     // the first weight-block scale of the next job travels while this one is stored
     if constexpr (BLOCKSCALE) bs_nxt = p.b_scales[(int64_t)((tn2 * BN + wn * WN) / 128) * p.b_scales_ld + nxt.s0];

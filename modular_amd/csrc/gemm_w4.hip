@@ -13,27 +13,26 @@
 // eight waves at the slab's barrier, and a wave that never shares its SIMD's issue slots.
 //
 // Pipeline of a block (persistent: one block per CU walks its share of the tiles, the slab stream never stops at a tile
-// boundary).  LDS holds TWO stages of activation rows (+ the slab's activation scales) and THREE stages of weight rows:
-// weight tiles are read by one XCD at a time and come from HBM, activation tiles are read by all eight at once and mostly
-// come from the memory-side cache, so the third stage goes to the operand with the longer way.  Per slab s:
-//
-//   groups 0, 1          copies of the weight rows of slab s + 2 (stage (s + 2) % 3, free since barrier s - 1)
-//   group TM - 2         the wave reads its last activation fragment of slab s, waits for its own copies of slab s + 1
-//                        and passes THE barrier of slab s: behind it slab s + 1 is in LDS for everybody and nobody
-//                        reads slab s any more.  The wave then reads the weight fragments, the first activation
-//                        fragment and the activation scales of slab s + 1 into its second set of fragment registers,
-//                        so that the first MFMA of slab s + 1 follows the last one of slab s without a wait for LDS.
-//   group TM - 1         copies of the activation rows (and scales) of slab s + 2 into the stage slab s has left
+// boundary).  The registers are a pipeline stage of their own: a wave holds TWO sets of fragment registers, multiplies
+// slab s from one and reads ALL fragments of slab s + 1 from LDS into the other meanwhile, one fragment every third
+// MFMA.  So at the barrier of slab s (the slab's first instruction) nobody reads slab s's LDS any more, and what the
+// barrier publishes -- slab s + 1, copied during slab s - 1 -- is not needed by any MFMA before the next barrier: no
+// wave waits for LDS behind a barrier.  LDS holds TWO stages of activation rows (+ the slab's activation scales) and
+// THREE stages of weight rows: weight tiles are read by one XCD at a time and come from HBM, activation tiles are read
+// by all eight at once and mostly come from the memory-side cache, so the third stage goes to the operand with the
+// longer way.  Behind the barrier of slab s a wave issues, one copy every third MFMA, the activation rows (and scales)
+// of slab s + 2 into the stage slab s has left, then the weight rows of slab s + 3 into the weight stage it has left.
 //
 // Vector memory operations of a wave complete in order: at barrier s the wave may still have the PER_B weight copies of
-// slab s + 2 in flight (and, behind a tile's last slab, the tile's NSTORE stores of C, which sit between the activation
-// copies and those weight copies in issue order), so the waits are exact counts.
+// slab s + 2 in flight (and, in front of a tile's first slab, the NSTORE stores of the tile before, which sit between
+// them and the activation copies in issue order), so the waits are exact counts.
 //
 // Promotion: the MFMA of (16-row group mt, fragment nt) writes a fresh product, and the four FMAs that fold it into the
 // accumulators are issued LAG MFMAs later, when the product has left the matrix pipe.
 //
 // Tiles: whole 256-column tiles of C, any M (rows past M read as zero through the buffer descriptor and their stores fall
-// outside C's descriptor), K in an even number of 128-byte slabs (the two sets of fragment registers alternate).
+// outside C's descriptor), K an even number (at least four) of whole 128-byte slabs (the two sets of fragment registers
+// alternate).
 // Sums are formed in the same order as by the eight-wave kernels (one product per slab, promoted in slab order):
 // results are bit-equal to theirs.
 #include <stdlib.h>
@@ -60,6 +59,9 @@ __device__ __forceinline__ v8i in_agprs(v8i f) {
   asm("" : "+a"(f));
   return f;
 }
+
+// the immediate of s_waitcnt on gfx9: vmcnt in bits 3:0 and 15:14, expcnt (left at its maximum) in 6:4, lgkmcnt in 11:8
+constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) { return (vmcnt & 15) | ((vmcnt >> 4) << 14) | (7 << 4) | (lgkmcnt << 8); }
 
 // PROBE (measurement aid, results meaningless): 0 the matmul; 1 the same loop with every copy reading tile (0, 0) and
 // slabs 0..7 over and over, so that its operands stay in L2; 2 the same without copies, waits and barriers -- the
@@ -155,7 +157,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     const uint8_t* g = a_frag + stage * A_STAGE + mt * 2048;
     const v4i lo = *reinterpret_cast<const v4i*>(g + a_lo);
     const v4i hi = *reinterpret_cast<const v4i*>(g + a_hi);
-    return in_agprs(v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w});
+    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
   const int wrow = 8 * (lm >> 2) + (lm & 3);
   const int wsw = (((wrow >> 3) & 1) << 2) | (wrow & 3);
@@ -165,7 +167,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     const uint8_t* g = b_frag + stage * B_STAGE + (t >> 1) * 4096 + (t & 1) * 512;
     const v4i lo = *reinterpret_cast<const v4i*>(g + b_lo);
     const v4i hi = *reinterpret_cast<const v4i*>(g + b_hi);
-    return in_agprs(v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w});
+    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
   struct Scales { float v[TM]; };
   const uint8_t* s_rd = smem + BM * 128 + (wm * 128 + lm * 8) * 4;
@@ -198,7 +200,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   if constexpr (PROBE != 0) tm = tn = 0;
   TileAt cur_at = tile_at(tm, tn);
   {
-    const SlabAt s0 = slab_at(cur_at, 0, 0u), s1 = slab_at(cur_at, 1, 0u);
+    const SlabAt s0 = slab_at(cur_at, 0, 0u), s1 = slab_at(cur_at, 1, 0u), s2 = slab_at(cur_at, 2, 0u);
 #pragma unroll
     for (int idx = 0; idx < PER_A; ++idx) dma_a(s0, 0, idx);
 #pragma unroll
@@ -207,14 +209,13 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     for (int idx = 0; idx < PER_A; ++idx) dma_a(s1, 1, idx);
 #pragma unroll
     for (int idx = 0; idx < PER_B; ++idx) dma_b(s1, 1, idx);
-  }
-  if constexpr (PROBE == 2) {
-    const SlabAt s2 = slab_at(cur_at, 2, 0u);
 #pragma unroll
     for (int idx = 0; idx < PER_B; ++idx) dma_b(s2, 2, idx);
+  }
+  if constexpr (PROBE == 2) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   } else {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_A + PER_B) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_A + 2 * PER_B) : "memory");
   }
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
@@ -223,12 +224,21 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   float bs_nxt = 1.f;
   if constexpr (BLOCKSCALE) bs_nxt = scalar_load_f32(p.b_scales + (int64_t)(PROBE ? wn : bs_blk) * p.b_scales_ld);
 
-  v8i bf[2][TN], af0[2];
+  // two sets of fragment registers: a slab is multiplied from one while the next slab's fragments arrive in the other
+  v8i bf[2][TN], af[2][TM];
   Scales sraw[2];
 #pragma unroll
   for (int t = 0; t < TN; ++t) bf[0][t] = read_bfrag(0, t);
-  af0[0] = read_afrag(0, 0);
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt) af[0][mt] = read_afrag(0, mt);
   if constexpr (BLOCKSCALE) sraw[0] = read_scales(0);
+
+  // (probe: the core clock's cycle counter and the constant 100 MHz counter, around the slab loop)
+  [[maybe_unused]] uint64_t probe_c0 = 0, probe_r0 = 0;
+  if constexpr (PROBE != 0) {
+    probe_c0 = clock64();
+    probe_r0 = wall_clock64();
+  }
 
   int bst = 0;          // weight stage of the slab being multiplied
   bool stored = false;  // a tile's stores sit in front of the weight copies now in flight
@@ -249,17 +259,39 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    // one slab; PAR = its parity = its activation stage = the set of fragment registers it multiplies from
+    // One slab.  PAR = its parity = its activation stage = the set of fragment registers it multiplies from.
     // (AFTER_STORES: the tile before this one has just been stored -- only a tile's first slab can be that.  A template
     // flag and not a branch at the wait: a branch there would cut the slab's straight-line code in two, and the compiler
     // schedules each part on its own -- it then issued forty MFMAs in a row and parked their products in AGPRs)
     auto slab_body = [&](auto PAR_C, auto AFTER_STORES_C, const int slab) {
       constexpr int PAR = decltype(PAR_C)::value;
       constexpr bool AFTER_STORES = decltype(AFTER_STORES_C)::value;
-      // slab + 2 of this tile, or slab (+ 2 - nslab) of the next one
-      const bool over = slab + 2 >= nslab;
-      const SlabAt dat = slab_at(over ? next_at : cur_at, over ? slab + 2 - nslab : slab + 2, over ? next_dead : 0u);
-      const int bst1 = bst == 2 ? 0 : bst + 1, bst2 = bst == 0 ? 2 : bst - 1;  // stages of slabs s + 1 and s + 2
+      constexpr int NSLOT = TM * TN;            // MFMAs of the slab
+      constexpr int NREAD = TN + TM + (BLOCKSCALE ? 1 : 0);  // fragments (and the scales) of the next slab
+      constexpr int NCOPY = PER_A + PER_B;
+      // slab + d of this tile, or of the next one
+      auto at_of = [&](int d) {
+        const int t = slab + d;
+        const bool over = t >= nslab;
+        return slab_at(over ? next_at : cur_at, over ? t - nslab : t, over ? next_dead : 0u);
+      };
+      const int bst1 = bst == 2 ? 0 : bst + 1;  // weight stage of slab s + 1
+
+      // ---- the barrier of slab s: this wave's copies of slab s + 1 have landed (its weight copies of slab s + 2, and a
+      // tile's stores, may stay in flight) and its reads of slab s, issued during slab s - 1, have returned
+      if constexpr (PROBE != 2) {
+        // (the waits are the builtin, not inline assembly: the compiler's own bookkeeping of outstanding loads reads it, and
+        // knows from here on that every fragment register has its value -- behind an opaque wait it guards the first use of
+        // each with a wait of its own, which, with a scalar load in flight, is a wait for ALL of the slab's new reads)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(PER_B + (AFTER_STORES ? NSTORE : 0), 0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+      }
+      const SlabAt dat_a = at_of(2), dat_b = at_of(3);
+      // (the hint sits here, where the whole set has arrived: right behind a read it would be a use of the value, and the
+      // compiler would wait for the read on the spot)
 
       float s_cur[TM];
       if constexpr (BLOCKSCALE) {
@@ -270,63 +302,54 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         const int ps = PROBE ? ((slab + 1) & 7) : slab + 1;
         bs_nxt = scalar_load_f32(slab + 1 < nslab ? bs_row + ps : bs_row2);
       }
-      v8i af = af0[PAR];
       [[maybe_unused]] v4f part[LAG + 1];
-#pragma unroll
-      for (int mt = 0; mt < TM; ++mt) {
-        v8i af_next = af;
-        if (mt + 1 < TM) af_next = read_afrag(PAR, mt + 1);
-#pragma unroll
-        for (int nt = 0; nt < TN; ++nt) {
-          if constexpr (BLOCKSCALE) {
-            constexpr v4f zero = {0.f, 0.f, 0.f, 0.f};
-            const int i = mt * TN + nt;
-            part[i % (LAG + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[PAR][nt], af, zero, 0, 0, 0, 0, 0, 0);
-            // issue order, pinned: one MFMA, then the four FMAs of the product that left the pipe LAG MFMAs ago
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i >= LAG) {
-              const int j = i - LAG;
-              acc[j / TN][j % TN] += part[j % (LAG + 1)] * s_cur[j / TN];
-              __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-            }
-          } else {
-            acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[PAR][nt], af, acc[mt][nt], 0, 0, 0, 0, 0, 0);
+      // Slot i = MFMA i of the slab, the four FMAs of the product that left the pipe LAG MFMAs ago, and at most one
+      // piece of memory work: a fragment read of slab s + 1 (two 16-byte LDS reads) or one copy instruction -- spread
+      // evenly, because a wave that issues several of them in a row stalls on the queue and its matrix pipe drains.
+      static_for<NSLOT>([&](auto I) {
+        constexpr int i = decltype(I)::value, mt = i / TN, nt = i % TN;
+        if constexpr (BLOCKSCALE) {
+          constexpr v4f zero = {0.f, 0.f, 0.f, 0.f};
+          part[i % (LAG + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[PAR][nt], af[PAR][mt], zero, 0, 0, 0, 0, 0, 0);
+          if constexpr (i >= LAG) {
+            constexpr int j = i - LAG;
+            acc[j / TN][j % TN] += part[j % (LAG + 1)] * s_cur[j / TN];
+          }
+        } else {
+          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[PAR][nt], af[PAR][mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
+        }
+        // read item r goes to slot r * NSLOT / NREAD: the scales, the weight fragments, the activation fragments
+        constexpr int r = (i * NREAD + NSLOT - 1) / NSLOT;  // the first item whose slot is >= i
+        if constexpr (r < NREAD && r * NSLOT / NREAD == i) {
+          constexpr int f = r - (BLOCKSCALE ? 1 : 0);
+          if constexpr (f < 0) sraw[PAR ^ 1] = read_scales(PAR ^ 1);
+          else if constexpr (f < TN) bf[PAR ^ 1][f] = read_bfrag(bst1, f);
+          else af[PAR ^ 1][f - TN] = read_afrag(PAR ^ 1, f - TN);
+        }
+        // copy d goes to slot d * NSLOT / NCOPY + 1: the activation rows and scales of slab s + 2 into the stage this slab
+        // has left, then the weight rows of slab s + 3 into the weight stage it has left
+        if constexpr (PROBE != 2 && i >= 1) {
+          constexpr int d = ((i - 1) * NCOPY + NSLOT - 1) / NSLOT;
+          if constexpr (d < NCOPY && d * NSLOT / NCOPY == i - 1) {
+            if constexpr (d < PER_A) dma_a(dat_a, PAR, d);
+            else dma_b(dat_b, bst, d - PER_A);
           }
         }
-        if constexpr (PROBE != 2) {
-          // weight rows of slab s + 2, in two halves
-          if (mt < 2) {
-#pragma unroll
-            for (int idx = mt * (PER_B / 2); idx < (mt + 1) * (PER_B / 2); ++idx) dma_b(dat, bst2, idx);
-          }
-        }
-        if (mt == TM - 2) {
-          // the slab's last fragment read is out: wait for it and for this wave's copies of slab s + 1, then the barrier
-          if constexpr (PROBE != 2) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_B + (AFTER_STORES ? NSTORE : 0)) : "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-          }
-          // the first fragments of slab s + 1
-#pragma unroll
-          for (int t = 0; t < TN; ++t) bf[PAR ^ 1][t] = read_bfrag(bst1, t);
-          af0[PAR ^ 1] = read_afrag(PAR ^ 1, 0);
-          if constexpr (BLOCKSCALE) sraw[PAR ^ 1] = read_scales(PAR ^ 1);
-        }
-        if constexpr (PROBE != 2) {
-          // activation rows and scales of slab s + 2 into the stage this slab has left
-          if (mt == TM - 1) {
-#pragma unroll
-            for (int idx = 0; idx < PER_A; ++idx) dma_a(dat, PAR, idx);
-          }
-        }
-        af = af_next;
-      }
+        // (nothing moves from one slot to another: left to itself the scheduler folds a product in right behind its own
+        // MFMA and fills the wait with idle cycles, or runs a dozen MFMAs ahead and parks their products)
+        __builtin_amdgcn_sched_barrier(0);
+      });
       if constexpr (BLOCKSCALE) {
 #pragma unroll
-        for (int j = TM * TN - LAG; j < TM * TN; ++j) acc[j / TN][j % TN] += part[j % (LAG + 1)] * s_cur[j / TN];
+        for (int j = NSLOT - LAG; j < NSLOT; ++j) acc[j / TN][j % TN] += part[j % (LAG + 1)] * s_cur[j / TN];
       }
+      // (the hint sits at the slab's end, where the whole set has arrived: right behind a read it would be a use of the
+      // value, and the compiler would wait for the read on the spot)
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < TN; ++t) bf[PAR ^ 1][t] = in_agprs(bf[PAR ^ 1][t]);
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) af[PAR ^ 1][mt] = in_agprs(af[PAR ^ 1][mt]);
       bst = bst1;
     };
 
@@ -340,6 +363,13 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       slab_body(ODD, std::false_type{}, slab + 1);
     }
 
+    if constexpr (PROBE != 0) {
+      if (p.workspace != nullptr && tid == 0) {
+        uint64_t* out = reinterpret_cast<uint64_t*>(p.workspace) + 2 * blockIdx.x;
+        out[0] = clock64() - probe_c0;
+        out[1] = wall_clock64() - probe_r0;
+      }
+    }
     // ---- the tile leaves, 16 rows x 64 columns of the wave's part at a time
     // (row scaling: every scale of the tile is loaded before the first store, so that no later wait for a load also
     // waits for the stores in front of it)
@@ -422,7 +452,7 @@ constexpr int w4_lds_bytes() {
 // The shapes this kernel takes: bf16 C with 16-byte aligned rows, whole 256-column tiles, K a whole and even number of
 // slabs, operands whose byte offsets fit 31 bits (a tile's position rides in the copies' scalar offset).
 bool gemm_w4_ok(const GemmArgs& p, bool blockscale) {
-  if (p.M <= 0 || p.N <= 0 || p.N % 256 != 0 || p.K < 256 || p.K % 256 != 0) return false;
+  if (p.M <= 0 || p.N <= 0 || p.N % 256 != 0 || p.K < 512 || p.K % 256 != 0) return false;
   const int64_t nslab = p.K / 128;
   if (p.kv_on || p.splits > 1) return false;
   if (p.c_dtype != MAXFP8_BF16 || !p.c_vec8_ok) return false;
