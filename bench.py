@@ -482,6 +482,8 @@ def kernels_launched(kind, M, K, N):
     first = plan.split(" + ")[0]
     if plan.startswith("skinny"):
         return "gemm_skinny_kernel", plan
+    if "four waves" in first:
+        return "gemm_w4_kernel", plan
     if "persistent" in first:
         return "gemm_persist_kernel", plan
     if "stream-K" in first:

@@ -1682,20 +1682,9 @@ static bool persist_ok(const GemmArgs& p, bool blockscale, dim3 grid) {
   return true;
 }
 
-// The four-wave kernel (gemm_w4.hip) for a matmul the planner gave the 256 x 256 shape: 0 (no), or the sixteen-row
-// groups per wave -- 5: tiles of 160 x 256, 6: 192 x 256.
+// The four-wave kernel (gemm_w4.hip): 0 (no), or the sixteen-row groups per wave -- 5: tiles of 160 x 256, 6: 192 x 256.
 bool gemm_w4_ok(const GemmArgs& p, bool blockscale);
 int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, hipStream_t stream);
-static int w4_rows(int64_t M, int64_t N, int64_t K, bool blockscale) {
-  const int forced = tuning().w4;
-  if (forced >= 0) return forced;
-  (void)M; (void)N; (void)K; (void)blockscale;
-  return 0;
-}
-static int w4_choice(const GemmArgs& p, bool blockscale, int variant, dim3 grid) {
-  if (variant != 1 || grid.y != 1 || grid.z != 1 || !tuning().persist || !gemm_w4_ok(p, blockscale)) return 0;
-  return w4_rows(p.M, p.N, p.K, blockscale);
-}
 
 int compute_units() {
   static int cached[64] = {0};
@@ -1928,8 +1917,48 @@ static TwoRegionPlan pick_two_regions(int64_t M, int64_t N, int nslab, bool bloc
   return best;
 }
 
-// What a tiled matmul will launch: one shape (possibly with K split), or two regions.
-struct TiledPlan { int variant; int splits; TwoRegionPlan two; bool streamk; };
+// What a tiled matmul will launch: one shape (possibly with K split), two regions, or the four-wave kernel (w4: 0, or
+// its sixteen-row groups per wave).
+struct TiledPlan { int variant; int splits; TwoRegionPlan two; bool streamk; int w4; };
+
+// One persistent launch of `tiles` tiles on `slots` CUs, a tile taking t microseconds with the chip full: whole rounds
+// cost t each; a last round that fills only part of the chip is faster than a full one but not in proportion (fewer
+// CUs share the clock budget, the L2s and the fabric; each tile still walks all of K) -- measured 0.76 ... 0.78 t at a
+// fill of 3 ... 40 %, 0.98 ... 1.03 t at 75 ... 85 %.
+static float persistent_cost(int64_t tiles, int slots, float t) {
+  const int64_t full = tiles / slots, rest = tiles % slots;
+  return (float)full * t + (rest ? t * (0.75f + 0.3f * (float)rest / (float)slots) : 0.f);
+}
+
+// Per-slab and per-tile times (microseconds, chip full, operands from HBM) of the four-wave kernel's two tile heights:
+// index 0: 160 x 256, 1: 192 x 256.  Against the eight-wave persistent kernel's 1.63 / 1.40 per slab of a 256 x 256 tile
+// that is 6 ... 9 % less per flop with block scaling and level with row scaling; what decides between the three is
+// mostly how the tile count divides by the CUs.
+static const float kW4SlabBlock[2] = {1.00f, 1.14f}, kW4SlabRow[2] = {0.88f, 1.00f}, kW4Tile = 5.5f;
+
+// The shapes the four-wave kernel takes (see gemm_w4_ok; pointers and strides are checked at the launch).
+static bool w4_shape(int64_t M, int64_t N, int64_t K) { return M > 0 && N > 0 && N % 256 == 0 && K >= 512 && K % 256 == 0; }
+
+// Which four-wave tile height, if any, beats `other_cost` (microseconds, what the plan made of the eight-wave shapes
+// costs) by at least 3 %.
+static int pick_w4(int64_t M, int64_t N, int64_t K, bool blockscale, float other_cost) {
+  const int forced = tuning().w4;
+  if (forced == 0 || !tuning().persist || !w4_shape(M, N, K)) return 0;
+  if (forced > 0) return forced;
+  const int nslab = (int)(K / 128), slots = compute_units();
+  int best = 0;
+  float best_cost = 0.97f * other_cost;
+  for (int i = 0; i < 2; ++i) {
+    const int tm = 5 + i;
+    const float t = (float)nslab * (blockscale ? kW4SlabBlock[i] : kW4SlabRow[i]) + kW4Tile;
+    const int64_t tiles = ceil_div(M, 32 * tm) * (N / 256);
+    if (tiles < slots) continue;  // (less than one round: the shapes with more, smaller tiles and a K split are the better fit)
+    const float cost = persistent_cost(tiles, slots, t);
+    if (cost < best_cost) { best = tm; best_cost = cost; }
+  }
+  return best;
+}
+
 
 // The work-split persistent kernel takes matmuls of whole 256 x 256 tiles that are at least one tile per block (so a
 // tile has at most two parts) and not a whole number of rounds (those have nothing to gain), when the caller's
@@ -1941,7 +1970,7 @@ static bool streamk_shape(int64_t M, int64_t N, size_t workspace_bytes) {
 }
 static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, size_t workspace_bytes,
                            int64_t batch, bool kv_on) {
-  TiledPlan plan = {0, 1, {0, 0, 0, 0, 0.f}, false};
+  TiledPlan plan = {0, 1, {0, 0, 0, 0, 0.f}, false, 0};
   const int nslab = (int)ceil_div(K, 128);
   plan.variant = tile_override();
   const bool free_choice = plan.variant == 0;
@@ -1968,6 +1997,14 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
     const float cost = 23.0f + tiles / g * (float)nslab * per_slab;
     const float other = plan.two.axis ? plan.two.cost : region_cost(M, N, nslab, t, blockscale);
     plan.streamk = tuning().streamk == 2 || cost < 0.9f * other;
+  }
+  // the four-wave kernel against whatever the eight-wave shapes make of the matmul (one launch; a forced tile shape other
+  // than 256 x 256, a K split, a batch or the fused QKV epilogue keep it out)
+  if (batch == 1 && !kv_on && plan.splits == 1 && !plan.streamk && (free_choice || plan.variant == 1)) {
+    float other = plan.two.axis ? plan.two.cost : region_cost(M, N, nslab, t, blockscale);
+    if (!plan.two.axis && persist_shape(M, N, plan.variant))
+      other = persistent_cost(tiles, t.slots, (float)nslab * (blockscale ? t.t_slab_block : t.t_slab_row) + tile_overhead(M, N, plan.variant - 1, 1));
+    plan.w4 = pick_w4(M, N, K, blockscale, other);
   }
   return plan;
 }
@@ -2014,6 +2051,8 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
   auto count = [](int64_t m, int64_t n, const TileShape& t) { return (long long)(ceil_div(m, t.bm) * ceil_div(n, t.bn)); };
   // (what a bf16 result with 16-byte aligned rows gets)
   auto how = [](int64_t m, int64_t n, int variant) { return persist_shape(m, n, variant) ? " persistent" : (variant == 4 ? " three-stage" : ""); };
+  if (plan.w4)
+    return snprintf(buf, len, "%dx256 x%lld persistent, four waves", 32 * plan.w4, (long long)(ceil_div(M, 32 * plan.w4) * (N / 256)));
   if (plan.two.axis && !plan.streamk) {
     const TileShape &a = kShapes[plan.two.v1 - 1], &b = kShapes[plan.two.v2 - 1];
     const bool cols = plan.two.axis == 1;
@@ -2050,6 +2089,11 @@ int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_
     // (the plan knows the shape; whether this call's pointers and strides suit the persistent kernels is checked here)
     if (persist_ok(p, blockscale, dim3(1, 1, 1)))
       return blockscale ? launch_streamk<true>(p, stream, "gemm_streamk_block_256x256") : launch_streamk<false>(p, stream, "gemm_streamk_row_256x256");
+  }
+  if (plan.w4) {
+    p.splits = 1;
+    // (the plan knows the shape; whether this call's pointers and strides suit the kernel is checked here)
+    if (gemm_w4_ok(p, blockscale)) return gemm_w4_launch(p, blockscale, plan.w4, stream);
   }
   if (plan.two.axis) {
     const TwoRegionPlan& two = plan.two;
@@ -2103,7 +2147,6 @@ static int gemm_tiled_launch(const GemmArgs& p, bool blockscale, int variant, di
     if (variant == 1) return launch_tiled<256, 256, 2, 4, 2, false, true>(p, grid, stream, "gemm_qkv_row_256x256");
     return launch_tiled<128, 128, 2, 2, 2, false, true>(p, grid, stream, "gemm_qkv_row_128x128");
   }
-  if (const int tm = w4_choice(p, blockscale, variant, grid)) return gemm_w4_launch(p, blockscale, tm, stream);
   if (variant == 1 && persist_ok(p, blockscale, grid))
     return blockscale ? launch_persist<true>(p, stream, "gemm_persist_block_256x256") : launch_persist<false>(p, stream, "gemm_persist_row_256x256");
   if (blockscale) {

@@ -75,7 +75,8 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   constexpr int B_BASE = 2 * A_STAGE, SIDE_BASE = B_BASE + 3 * B_STAGE, SIDE_BYTES = 2048;
   constexpr int PER_A = IA + (BLOCKSCALE ? 1 : 0), PER_B = IB;
   constexpr int NSTORE = TM * TN / 2;                        // 16-byte stores per lane and tile
-  constexpr int LAG = 3;                                     // a product is folded in LAG MFMAs after its own
+  // a product is folded in LAG MFMAs after its own (2: 4 ... 6 % slower, the FMAs then wait for the matrix pipe; 4: the same)
+  constexpr int LAG = 3;
   static_assert(TN == 8 && TM >= 3 && TM <= 8, "wave tile");
   static_assert(PER_B + NSTORE < 64, "the count must fit the vmcnt field");
   static_assert(IB % 2 == 0, "the weight copies go out in two halves");
@@ -221,8 +222,10 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   asm volatile("" ::: "memory");
 
   const int bs_blk = 2 * tn + wn;  // (BN = 256: two weight-scale blocks per tile, one per wave column)
+  // The weight-block scale of a slab is element bs_cur of the weight scales: that of the slab to come is loaded a slab ahead.
+  uint32_t bs_cur = (uint32_t)((PROBE ? wn : bs_blk) * p.b_scales_ld);
   float bs_nxt = 1.f;
-  if constexpr (BLOCKSCALE) bs_nxt = scalar_load_f32(p.b_scales + (int64_t)(PROBE ? wn : bs_blk) * p.b_scales_ld);
+  if constexpr (BLOCKSCALE) bs_nxt = scalar_load_f32(p.b_scales + bs_cur);
 
   // two sets of fragment registers: a slab is multiplied from one while the next slab's fragments arrive in the other
   v8i bf[2][TN], af[2][TM];
@@ -242,16 +245,21 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
 
   int bst = 0;          // weight stage of the slab being multiplied
   bool stored = false;  // a tile's stores sit in front of the weight copies now in flight
+  // Where the copies of the slab about to start read: the activation rows (and scales) of its slab + 2, the weight rows
+  // of its slab + 3.  Running offsets, 128 bytes (one row of scales) further with every slab, set to the next tile's
+  // first slab when they pass the end of K -- a handful of scalar instructions per slab; worked out from the slab number
+  // every time they were two dozen, and a wave alone on its SIMD pays for every instruction it issues.
+  SlabAt cur = slab_at(cur_at, 2, 0u);
+  cur.b = slab_at(cur_at, 3, 0u).b;
+
   for (int k = 0; k < njobs; ++k) {
     const bool has_next = k + 1 < njobs;
     int tm2 = tm, tn2 = tn;
     if (has_next) tile_coords(run_begin + my + (k + 1) * nb, tiles_m, tiles_n, tm2, tn2);
     const TileAt next_at = tile_at(tm2, tn2);
-    const uint32_t next_dead = has_next ? 0u : 0x80000000u;
-    const float* bs_row = nullptr;
-    if constexpr (BLOCKSCALE) bs_row = p.b_scales + (int64_t)(PROBE ? wn : 2 * tn + wn) * p.b_scales_ld;
-    const float* bs_row2 = nullptr;
-    if constexpr (BLOCKSCALE) bs_row2 = p.b_scales + (int64_t)(PROBE ? wn : 2 * tn2 + wn) * p.b_scales_ld;
+    // slab 0 of the next tile (of nothing behind the block's last tile: offsets past 2^31 read as zeros)
+    const SlabAt next0 = slab_at(next_at, 0, has_next ? 0u : 0x80000000u);
+    const uint32_t next_bs0 = (uint32_t)((PROBE ? wn : 2 * tn2 + wn) * p.b_scales_ld);
 
     v4f acc[TM][TN];
 #pragma unroll
@@ -260,21 +268,15 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
     // One slab.  PAR = its parity = its activation stage = the set of fragment registers it multiplies from.
-    // (AFTER_STORES: the tile before this one has just been stored -- only a tile's first slab can be that.  A template
-    // flag and not a branch at the wait: a branch there would cut the slab's straight-line code in two, and the compiler
-    // schedules each part on its own -- it then issued forty MFMAs in a row and parked their products in AGPRs)
+    // AFTER_STORES: the tile before this one has just been stored -- only a tile's first slab can be that.  A template flag
+    // and not a branch at the wait: a branch would cut the slab's straight-line code in two, and the compiler schedules
+    // each part on its own -- it then issued forty MFMAs in a row and parked their products in AGPRs.
     auto slab_body = [&](auto PAR_C, auto AFTER_STORES_C, const int slab) {
       constexpr int PAR = decltype(PAR_C)::value;
       constexpr bool AFTER_STORES = decltype(AFTER_STORES_C)::value;
       constexpr int NSLOT = TM * TN;            // MFMAs of the slab
       constexpr int NREAD = TN + TM + (BLOCKSCALE ? 1 : 0);  // fragments (and the scales) of the next slab
       constexpr int NCOPY = PER_A + PER_B;
-      // slab + d of this tile, or of the next one
-      auto at_of = [&](int d) {
-        const int t = slab + d;
-        const bool over = t >= nslab;
-        return slab_at(over ? next_at : cur_at, over ? t - nslab : t, over ? next_dead : 0u);
-      };
       const int bst1 = bst == 2 ? 0 : bst + 1;  // weight stage of slab s + 1
 
       // ---- the barrier of slab s: this wave's copies of slab s + 1 have landed (its weight copies of slab s + 2, and a
@@ -289,9 +291,17 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
       }
-      const SlabAt dat_a = at_of(2), dat_b = at_of(3);
-      // (the hint sits here, where the whole set has arrived: right behind a read it would be a use of the value, and the
-      // compiler would wait for the read on the spot)
+      const SlabAt my = cur;
+      // (the offsets of the next slab's copies: K has at least four slabs, so each of them passes the end of K once a tile)
+      if constexpr (PROBE != 0) {
+        cur.a = (cur.a + 128u) & 1023u;
+        cur.b = (cur.b + 128u) & 1023u;
+        cur.s = cur.s + s_slab_step == 8u * s_slab_step ? 0u : cur.s + s_slab_step;
+      } else {
+        cur.a = slab + 3 == nslab ? next0.a : cur.a + 128u;
+        cur.s = slab + 3 == nslab ? next0.s : cur.s + s_slab_step;
+        cur.b = slab + 4 == nslab ? next0.b : cur.b + 128u;
+      }
 
       float s_cur[TM];
       if constexpr (BLOCKSCALE) {
@@ -299,8 +309,9 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
 #pragma unroll
         for (int mt = 0; mt < TM; ++mt) s_cur[mt] = sraw[PAR].v[mt] * bs;
         // the weight-block scale of the next slab (of the next tile behind this tile's last slab)
-        const int ps = PROBE ? ((slab + 1) & 7) : slab + 1;
-        bs_nxt = scalar_load_f32(slab + 1 < nslab ? bs_row + ps : bs_row2);
+        if constexpr (PROBE != 0) bs_cur = (bs_cur & ~7u) | ((bs_cur + 1u) & 7u);
+        else bs_cur = slab + 1 == nslab ? next_bs0 : bs_cur + 1u;
+        bs_nxt = scalar_load_f32(p.b_scales + bs_cur);
       }
       [[maybe_unused]] v4f part[LAG + 1];
       // Slot i = MFMA i of the slab, the four FMAs of the product that left the pipe LAG MFMAs ago, and at most one
@@ -331,21 +342,21 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         if constexpr (PROBE != 2 && i >= 1) {
           constexpr int d = ((i - 1) * NCOPY + NSLOT - 1) / NSLOT;
           if constexpr (d < NCOPY && d * NSLOT / NCOPY == i - 1) {
-            if constexpr (d < PER_A) dma_a(dat_a, PAR, d);
-            else dma_b(dat_b, bst, d - PER_A);
+            if constexpr (d < PER_A) dma_a(my, PAR, d);
+            else dma_b(my, bst, d - PER_A);
           }
         }
         // (nothing moves from one slot to another: left to itself the scheduler folds a product in right behind its own
         // MFMA and fills the wait with idle cycles, or runs a dozen MFMAs ahead and parks their products)
         __builtin_amdgcn_sched_barrier(0);
       });
+      // (the slab's last products: folding them in during the first MFMAs of the next slab instead measured 7 % slower)
       if constexpr (BLOCKSCALE) {
 #pragma unroll
         for (int j = NSLOT - LAG; j < NSLOT; ++j) acc[j / TN][j % TN] += part[j % (LAG + 1)] * s_cur[j / TN];
       }
       // (the hint sits at the slab's end, where the whole set has arrived: right behind a read it would be a use of the
       // value, and the compiler would wait for the read on the spot)
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < TN; ++t) bf[PAR ^ 1][t] = in_agprs(bf[PAR ^ 1][t]);
 #pragma unroll

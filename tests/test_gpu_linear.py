@@ -60,13 +60,14 @@ def test_rowwise_linear_and_bias(dev):
     assert_rel(f32_np(y0(x.to(dev))), ref, 1e-2, "rowwise linear")
 
 
-@pytest.mark.parametrize("M,K,N", [(2048, 2048, 28672), (16, 512, 4096), (256, 1024, 1536)])
-def test_linear_replays_from_a_graph(dev, M, K, N):
-    """An FP8 linear (quantise + matmul) has no host synchronisation, so it records into a HIP graph: the
-    persistent kernel with a second region in another tile shape, the decode kernel, and the K-split shapes with
-    their workspace.  Every replay, with eager work and synchronisations between them and new activations in the
-    same buffer, must give the eager result."""
+@pytest.mark.parametrize("M,K,N,w4", [(2048, 2048, 28672, None), (2048, 2048, 28672, "0"), (16, 512, 4096, None), (256, 1024, 1536, None)])
+def test_linear_replays_from_a_graph(dev, tune, M, K, N, w4):
+    """An FP8 linear (quantise + matmul) has no host synchronisation, so it records into a HIP graph: the four-wave
+    persistent kernel, the eight-wave persistent kernel with a second region in another tile shape, the decode kernel,
+    and the K-split shapes with their workspace.  Every replay, with eager work and synchronisations between them and
+    new activations in the same buffer, must give the eager result."""
     from modular_amd import _lib
+    tune(MAXFP8_W4=w4)
     cfg = mx.blockwise_fp8_config()
     wq, ws = synth.quantize_weight_block(synth.weights_f32(N, K, seed=3))
     lin = mx.Linear(K, N, cfg, device=dev)
@@ -74,7 +75,8 @@ def test_linear_replays_from_a_graph(dev, M, K, N):
     lin.weight_scale.copy_(ws.to(dev))
     x = synth.activations(M, K, seed=4).to(dev)
     if M == 2048:
-        assert " + " in _lib.matmul_describe(M, N, K) and "persistent" in _lib.matmul_describe(M, N, K)
+        plan = _lib.matmul_describe(M, N, K)
+        assert "persistent" in plan and ("four waves" in plan if w4 is None else " + " in plan), plan
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         lin(x)  # first call outside the capture: it sets the kernels' LDS attributes

@@ -176,7 +176,7 @@ def test_grouped_small_tiles_exact(dev):
 def test_two_region_launch(dev, tune, M, K, N, kind):
     # (with a workspace, shapes of whole 256 x 256 tiles now split their work between the blocks instead: that path
     # has its own tests below; here it is switched off so that the cut is what runs)
-    tune(MAXFP8_STREAMK="0")
+    tune(MAXFP8_STREAMK="0", MAXFP8_W4="0")
     assert " + " in _lib.matmul_describe(M, N, K, kind == "block"), "this shape is meant to run as two launches"
     cfg = BLK if kind == "block" else ROW
     x = synth.activations(M, K, seed=0, outlier_frac=0.0 if kind == "row" else 0.01, device=dev)

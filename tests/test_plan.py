@@ -28,7 +28,8 @@ def test_single_shapes_and_k_split():
     assert _lib.matmul_describe(0, 10, 10) == "nothing to do"
 
 
-def test_two_regions_cover_the_problem_once():
+def test_two_regions_cover_the_problem_once(tune):
+    tune(MAXFP8_W4="0")  # (the four-wave kernel, which takes such shapes in one launch, has its own test below)
     for (M, N, K) in [(2048, 28672, 4096), (28672, 2048, 4096), (2040, 28600, 4096)]:
         text = _lib.matmul_describe(M, N, K)
         assert " + " in text, text
@@ -42,3 +43,16 @@ def test_two_regions_cover_the_problem_once():
             assert cut % bm1 == 0 and 0 < cut < M
             assert n1 == (cut // bm1) * ceil(N, bn1) and n2 == ceil(M - cut, bm2) * ceil(N, bn2)
         assert n1 % 256 == 0, "the first region runs in whole rounds of the 256 CUs"
+
+
+def test_four_wave_kernel_where_its_tile_count_fits_the_chip(tune):
+    # DeepSeek-V3 o_proj at M = 4096: 448 tiles of 256 x 256 are 1.75 rounds of the 256 CUs, 728 tiles of 160 x 256 are 2.84
+    assert _lib.matmul_describe(4096, 7168, 16384) == "160x256 x728 persistent, four waves"
+    # ragged N, an odd number of slabs, and less than one round of tiles stay with the eight-wave shapes
+    assert "four waves" not in _lib.matmul_describe(4096, 7160, 16384)
+    assert "four waves" not in _lib.matmul_describe(4096, 7168, 16384 + 128)
+    assert "four waves" not in _lib.matmul_describe(128, 28672, 4096, False)
+    tune(MAXFP8_W4="0")
+    assert "four waves" not in _lib.matmul_describe(4096, 7168, 16384)
+    tune(MAXFP8_W4="6")
+    assert _lib.matmul_describe(4096, 7168, 16384) == "192x256 x616 persistent, four waves"
