@@ -244,8 +244,9 @@ def config_cells():
     for proj, (K, N) in (("qkv", (4096, 6144)), ("o_proj", (4096, 4096)), ("gate_up", (4096, 28672)), ("down", (14336, 4096))):
         for M in (1, 16, 128, 2048):
             cells[f"llama8b_{proj}_m{M}"] = ("block", M, K, N)
+    # (q_a_kv_a: the one matmul over the stacked q_a and kv_a weights that the reference's FP8 MLA issues, N = 1536 + 576)
     for proj, (K, N) in (("q_a", (7168, 1536)), ("q_b", (1536, 24576)), ("kv_a", (7168, 576)), ("kv_b", (512, 32768)),
-                         ("o_proj", (16384, 7168))):
+                         ("o_proj", (16384, 7168)), ("q_a_kv_a", (7168, 2112))):
         for M in (256, 1024, 4096):
             cells[f"dsv3_{proj}_m{M}"] = ("block", M, K, N)
     for proj, (K, N) in (("qkv", (8192, 10240)), ("gate_up", (8192, 57344)), ("down", (28672, 8192))):

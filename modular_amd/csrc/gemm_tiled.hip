@@ -1937,7 +1937,7 @@ static float persistent_cost(int64_t tiles, int slots, float t) {
 static const float kW4SlabBlock[2] = {1.00f, 1.14f}, kW4SlabRow[2] = {0.88f, 1.00f}, kW4Tile = 5.5f;
 
 // The shapes the four-wave kernel takes (see gemm_w4_ok; pointers and strides are checked at the launch).
-static bool w4_shape(int64_t M, int64_t N, int64_t K) { return M > 0 && N > 0 && N % 256 == 0 && K >= 512 && K % 256 == 0; }
+static bool w4_shape(int64_t M, int64_t N, int64_t K) { return M > 0 && N > 0 && N % 8 == 0 && K >= 512 && K % 256 == 0; }
 
 // Which four-wave tile height, if any, beats `other_cost` (microseconds, what the plan made of the eight-wave shapes
 // costs) by at least 3 %.
@@ -1951,8 +1951,8 @@ static int pick_w4(int64_t M, int64_t N, int64_t K, bool blockscale, float other
   for (int i = 0; i < 2; ++i) {
     const int tm = 5 + i;
     const float t = (float)nslab * (blockscale ? kW4SlabBlock[i] : kW4SlabRow[i]) + kW4Tile;
-    const int64_t tiles = ceil_div(M, 32 * tm) * (N / 256);
-    if (tiles < slots) continue;  // (less than one round: the shapes with more, smaller tiles and a K split are the better fit)
+    const int64_t tiles = ceil_div(M, 32 * tm) * ceil_div(N, 256);
+    if (tiles * 4 < (int64_t)slots * 3) continue;  // (well under one round: more, smaller tiles and a K split are the better fit)
     const float cost = persistent_cost(tiles, slots, t);
     if (cost < best_cost) { best = tm; best_cost = cost; }
   }
@@ -2052,7 +2052,7 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
   // (what a bf16 result with 16-byte aligned rows gets)
   auto how = [](int64_t m, int64_t n, int variant) { return persist_shape(m, n, variant) ? " persistent" : (variant == 4 ? " three-stage" : ""); };
   if (plan.w4)
-    return snprintf(buf, len, "%dx256 x%lld persistent, four waves", 32 * plan.w4, (long long)(ceil_div(M, 32 * plan.w4) * (N / 256)));
+    return snprintf(buf, len, "%dx256 x%lld persistent, four waves", 32 * plan.w4, (long long)(ceil_div(M, 32 * plan.w4) * ceil_div(N, 256)));
   if (plan.two.axis && !plan.streamk) {
     const TileShape &a = kShapes[plan.two.v1 - 1], &b = kShapes[plan.two.v2 - 1];
     const bool cols = plan.two.axis == 1;

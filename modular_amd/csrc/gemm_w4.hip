@@ -30,8 +30,8 @@
 // Promotion: the MFMA of (16-row group mt, fragment nt) writes a fresh product, and the four FMAs that fold it into the
 // accumulators are issued LAG MFMAs later, when the product has left the matrix pipe.
 //
-// Tiles: whole 256-column tiles of C, any M (rows past M read as zero through the buffer descriptor and their stores fall
-// outside C's descriptor), K an even number (at least four) of whole 128-byte slabs (the two sets of fragment registers
+// Tiles: any M and any N that is a multiple of 8 (rows of either operand past the end read as zero through the buffer
+// descriptors, stores of rows past M fall outside C's descriptor, lanes whose columns lie past N store nothing), K an even number (at least four) of whole 128-byte slabs (the two sets of fragment registers
 // alternate).
 // Sums are formed in the same order as by the eight-wave kernels (one product per slab, promoted in slab order):
 // results are bit-equal to theirs.
@@ -88,7 +88,8 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   const int nslab = p.K / 128;                               // whole slabs, an even number of them (the host's rule)
 
   // ---- this block's tiles: every nb-th tile of its XCD's contiguous run (blocks are dealt to the XCDs round-robin)
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = p.N / BN, total = tiles_m * tiles_n;
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN, total = tiles_m * tiles_n;
+  const int bs_rows = (p.N + 127) / 128;  // rows of the weight scales: a wave whose columns all lie past N reads the last one
   const int xcd = blockIdx.x & 7;
   const int run_begin = xcd * (total >> 3) + (xcd < (total & 7) ? xcd : (total & 7));
   const int run_len = (total >> 3) + (xcd < (total & 7) ? 1 : 0);
@@ -221,9 +222,14 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 
-  const int bs_blk = 2 * tn + wn;  // (BN = 256: two weight-scale blocks per tile, one per wave column)
+  // (BN = 256: two weight-scale blocks per tile, one per wave column)
+  auto bs_block = [&](int tile_n) {
+    if constexpr (PROBE != 0) return wn;
+    const int blk = 2 * tile_n + wn;
+    return blk < bs_rows ? blk : bs_rows - 1;
+  };
   // The weight-block scale of a slab is element bs_cur of the weight scales: that of the slab to come is loaded a slab ahead.
-  uint32_t bs_cur = (uint32_t)((PROBE ? wn : bs_blk) * p.b_scales_ld);
+  uint32_t bs_cur = (uint32_t)(bs_block(tn) * p.b_scales_ld);
   float bs_nxt = 1.f;
   if constexpr (BLOCKSCALE) bs_nxt = scalar_load_f32(p.b_scales + bs_cur);
 
@@ -259,7 +265,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     const TileAt next_at = tile_at(tm2, tn2);
     // slab 0 of the next tile (of nothing behind the block's last tile: offsets past 2^31 read as zeros)
     const SlabAt next0 = slab_at(next_at, 0, has_next ? 0u : 0x80000000u);
-    const uint32_t next_bs0 = (uint32_t)((PROBE ? wn : 2 * tn2 + wn) * p.b_scales_ld);
+    const uint32_t next_bs0 = (uint32_t)(bs_block(tn2) * p.b_scales_ld);
 
     v4f acc[TM][TN];
 #pragma unroll
@@ -390,7 +396,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       for (int q = 0; q < TN / 2; ++q)
 #pragma unroll
         for (int i = 0; i < 8; ++i)
-          b_s[q][i] = scale_at(p.b_scales, (int64_t)(tn * BN + wn * WN + q * 32 + lq * 8 + i) * p.b_scale_stride, p.scales_dtype);
+          b_s[q][i] = scale_at(p.b_scales, (int64_t)min(tn * BN + wn * WN + q * 32 + lq * 8 + i, p.N - 1) * p.b_scale_stride, p.scales_dtype);
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt) {
         int64_t m = (int64_t)tm * BM + wm * WM + mt * 16 + lm;
@@ -406,6 +412,11 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     asm volatile("" : "+v"(lane_e));
     const int lm_e = lane_e & 15, lq_e = lane_e >> 4, rr = lane_e >> 3, cc = lane_e & 7;
     const uint32_t c_lane = (uint32_t)rr * c_row_bytes + (uint32_t)cc * 16u;
+    // (the last column tile may reach past N, which is a multiple of 8: a lane whose eight columns lie there stores out of
+    // the descriptor's range, i.e. nothing -- every store is still issued, so the counts of the waits stay exact)
+    uint32_t c_lane_h[TN / 4];
+#pragma unroll
+    for (int h = 0; h < TN / 4; ++h) c_lane_h[h] = tn * BN + wn * WN + h * 64 + cc * 8 < p.N ? c_lane : 0x80000000u;
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) {
       float a_s = 1.f;
@@ -435,7 +446,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
           const int r = i * 8 + rr;
           const v4u_t v = *reinterpret_cast<const v4u_t*>(wbuf + r * 128 + ((cc ^ (r & 7)) * 16));
           // (non-temporal: C is not read again here, and its lines should not push the operands out of L2)
-          buffer_store_b128_guarded<2>(v, c_rsrc, c_lane, c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes + (uint32_t)h * 128u);
+          buffer_store_b128_guarded<2>(v, c_rsrc, c_lane_h[h], c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes + (uint32_t)h * 128u);
         }
       }
     }
@@ -460,16 +471,16 @@ constexpr int w4_lds_bytes() {
   return 2 * (TM * 32 * 128 + (BLOCKSCALE ? 1024 : 0)) + 3 * (TN * 32 * 128) + 4 * 2048;
 }
 
-// The shapes this kernel takes: bf16 C with 16-byte aligned rows, whole 256-column tiles, K a whole and even number of
-// slabs, operands whose byte offsets fit 31 bits (a tile's position rides in the copies' scalar offset).
+// The shapes this kernel takes: bf16 C with 16-byte aligned rows, N a multiple of 8, K a whole and even number of slabs,
+// operands whose byte offsets fit 31 bits (a tile's position rides in the copies' scalar offset).
 bool gemm_w4_ok(const GemmArgs& p, bool blockscale) {
-  if (p.M <= 0 || p.N <= 0 || p.N % 256 != 0 || p.K < 512 || p.K % 256 != 0) return false;
+  if (p.M <= 0 || p.N <= 0 || p.N % 8 != 0 || p.K < 512 || p.K % 256 != 0) return false;
   const int64_t nslab = p.K / 128;
   if (p.kv_on || p.splits > 1) return false;
   if (p.c_dtype != MAXFP8_BF16 || !p.c_vec8_ok) return false;
   const int64_t lim = 0x7ff00000ll;
   const int64_t rows = ceil_div(p.M, 192) * 192 + 192;
-  if (rows * p.lda >= lim || (int64_t)p.N * p.ldb >= lim) return false;
+  if (rows * p.lda >= lim || (ceil_div(p.N, 256) * 256) * p.ldb >= lim) return false;
   if (blockscale && (nslab * p.a_scales_ld + rows) * 4 >= lim) return false;
   if (rows * p.ldc * 2 >= lim) return false;
   return true;
@@ -493,7 +504,7 @@ static int launch_w4(const GemmArgs& p, unsigned blocks, hipStream_t stream, con
 
 // rows of a tile: 32 * tm (tm = 5 or 6 sixteen-row groups per wave)
 int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, hipStream_t stream) {
-  const int64_t tiles = ceil_div(p.M, 32 * tm) * (p.N / 256);
+  const int64_t tiles = ceil_div(p.M, 32 * tm) * ceil_div(p.N, 256);
   const int cus = compute_units();
   const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
   if (tm == 5)

@@ -6,13 +6,15 @@
 Shapes follow the reference's tests (test_naive_blockwise_fp8_matmul.mojo:194-200,
 test_scaled_matmul.mojo:332-377, test_fp8_matmul_gpu.py:40-442) and BASELINE's configs;
 at sizes the CPU cannot finish, the bit-exact-to-oracle naive kernel checks sampled rows."""
+import os
+
 import numpy as np
 import pytest
 import torch
 
 import modular_amd as mx
 import oracle
-from modular_amd import synth
+from modular_amd import _lib, synth
 from modular_amd.quant_config import InputScaleSpec, QuantConfig, ScaleGranularity, ScaleOrigin, WeightScaleSpec
 from util import F32_BUDGET, assert_rel, bf16_bits, f32_np, fp8_bytes, fp8_from_bytes, rel_err
 
@@ -293,7 +295,10 @@ def test_empty(dev):
 # scalar-order kernel (bit-identical to the CPU oracle, tested above) needs a second per 24 rows at these sizes.
 
 LLAMA8B = {"qkv": (4096, 6144), "gate_up": (4096, 28672), "down": (14336, 4096), "o_proj": (4096, 4096)}
-DSV3 = {"q_a": (7168, 1536), "q_b": (1536, 24576), "kv_a": (7168, 576), "kv_b": (512, 32768), "o_proj": (16384, 7168)}
+DSV3 = {"q_a": (7168, 1536), "q_b": (1536, 24576), "kv_a": (7168, 576), "kv_b": (512, 32768), "o_proj": (16384, 7168),
+        # the call the reference's FP8 MLA issues for q_a and kv_a: one matmul over the two weights stacked, N = 1536 + 576
+        # (max/python/max/nn/attention/multi_latent_attention_fp8.py:595-603)
+        "q_a_kv_a": (7168, 2112)}
 CONFIG_CELLS = ([("single_linear", 64, 4096, 4096)]
                 + [(f"llama8b_{n}", M, K, N) for n, (K, N) in LLAMA8B.items() for M in (1, 16, 128, 2048)]
                 + [(f"dsv3_{n}", M, K, N) for n, (K, N) in DSV3.items() for M in (256, 1024, 4096)])
@@ -321,8 +326,15 @@ def test_config_shapes_blockwise(dev, name, M, K, N):
                                    BLK.weight_scale, out_type=torch.float32, algo="naive")
     torch.cuda.synchronize()
     fig = assert_rel(f32_np(c[rows]), f32_np(ref), TOL, f"config {name} {M}x{N}x{K}", natural_scale=True)
-    print(f"[parity] {name} M={M}: rel err {fig['rel_err']:.2e} (floor 2^-4 rms), {fig['rel_err_strict_floor']:.2e} "
-          f"(floor 2^-8 rms), |err| <= {fig['err_over_rms']:.2e} rms, reference-style excess {fig['reference_style_excess']:.2f}")
+    line = (f"{name} M={M} K={K} N={N}: rel err {fig['rel_err']:.2e} (floor 2^-4 rms), {fig['rel_err_strict_floor']:.2e} "
+            f"(floor 2^-8 rms), |err| <= {fig['err_over_rms']:.2e} rms, reference-style excess {fig['reference_style_excess']:.2f}"
+            f" | {_lib.matmul_describe(M, N, K, True, True)}")
+    print("[parity] " + line)
+    # (the figures of a run are kept beside the run's other results)
+    out_dir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "parity_figures.txt"), "a") as f:
+        f.write(line + "\n")
     # one row against the CPU oracle itself
     r0 = int(rows[-1])
     cpu = oracle.matmul_blockwise(fp8_bytes(q[r0:r0 + 1]), fp8_bytes(w), f32_np(sa[:, r0:r0 + 1]), f32_np(sb), threads=NT)

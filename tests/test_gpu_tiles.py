@@ -241,6 +241,41 @@ def test_persistent_kernel_exact(dev, tune, M, N, K, form):
     assert torch.equal(cb.cpu(), torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 2112, 7168), (320, 264, 512), (1000, 8, 1024), (161, 1544, 768)])
+@pytest.mark.parametrize("kind", ["block", "row"])
+@pytest.mark.parametrize("rows", ["5", "6"])
+def test_four_wave_kernel_ragged_edges(dev, tune, M, N, K, kind, rows):
+    # a last row tile past M and a last column tile past N (DeepSeek-V3's fused q_a + kv_a projection: N = 1536 + 576 = 2112 =
+    # 8 tiles and a quarter): bit-equal to the per-tile kernel, and nothing written outside the result.  Through the C ABI,
+    # so that the result can sit in the middle of a larger buffer.
+    L = _lib.lib()
+    if kind == "block":
+        a, b, sa, sb = make_block(M, N, K, seed=M + N)
+        gin, gw, g, a_ld, b_ld = _lib.GRAN_BLOCK, _lib.GRAN_BLOCK, (1, 128, 128), sa.shape[1], K // 128
+    else:
+        a, b = synth.random_fp8((M, K), M), synth.random_fp8((N, K), N + 1)
+        sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+        gin, gw, g, a_ld, b_ld = _lib.GRAN_COLWISE, _lib.GRAN_ROWWISE, (-1, -1, -1), M, 1
+    a, b, sa, sb = a.to(dev), b.to(dev), sa.to(dev).contiguous(), sb.to(dev).contiguous()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def run(c):
+        st = L.maxfp8_matmul_dynamic_scaled_fp8(c.data_ptr(), a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), M, N, K,
+                                                K, K, N, gin, gw, *g, a_ld, b_ld, _lib.BF16, _lib.F32, _lib.ALGO_TILED, None, 0, stream)
+        assert st == 0, _lib.last_error()
+
+    tune(MAXFP8_TILE="1", MAXFP8_W4=rows)
+    assert "four waves" in _lib.matmul_describe(M, N, K, kind == "block", False)
+    guard = torch.full((M + 2, N), -7.0, dtype=torch.bfloat16, device=dev)
+    run(guard[1:M + 1])
+    tune(MAXFP8_PERSIST="0")
+    want = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    run(want)
+    torch.cuda.synchronize()
+    assert torch.equal(guard[1:M + 1].view(torch.int16), want.view(torch.int16))
+    assert bool((guard[0] == -7.0).all()) and bool((guard[M + 1] == -7.0).all())
+
+
 def test_persistent_kernel_leaves_other_outputs_alone(dev, tune):
     # f32 output, rows of C that are not 16-byte aligned and partial tiles stay with the per-tile kernel
     tune(MAXFP8_TILE="1")
