@@ -409,6 +409,71 @@ def mfma_ceiling(slabs=4096, reps=20, settle_s=0.5):
                        "blocks": cus}
 
 
+VENDOR_CELLS = [(4096, 7168, 16384), (8192, 8192, 8192), (2048, 28672, 4096), (2048, 6144, 4096), (4096, 24576, 1536),
+                (256, 2304, 16384), (16, 2304, 16384), (64, 28672, 4096), (128, 8192, 28672), (8, 57344, 8192)]
+
+
+def vendor_compare(steps=30):
+    """Per-token x per-channel scaled FP8 matmuls (the one scaling form the vendor library has) through this library and
+    through hipBLASLt (reached by torch._scaled_mm) on the same operands, weights rotating through enough copies to come
+    from HBM.  Yields one record per (M, N, K): microseconds each, and the largest difference of the two bf16 results in
+    bf16 steps of the larger value."""
+    import torch
+    from modular_amd import kernels as mx, synth
+    from modular_amd.quant_config import InputScaleSpec, ScaleGranularity, ScaleOrigin, WeightScaleSpec
+
+    dev = torch.device("cuda:0")
+    in_spec = InputScaleSpec(granularity=ScaleGranularity.COLWISE, origin=ScaleOrigin.DYNAMIC, dtype=torch.float32)
+    w_spec = WeightScaleSpec(granularity=ScaleGranularity.ROWWISE, dtype=torch.float32)
+
+    def timed(fn):
+        t_end = time.perf_counter() + 0.3
+        i = 0
+        while time.perf_counter() < t_end:
+            fn(i)
+            i += 1
+            torch.cuda.synchronize()
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(5):
+            fn(i)
+        first.record()
+        for i in range(steps):
+            fn(i)
+        last.record()
+        torch.cuda.synchronize()
+        return first.elapsed_time(last) * 1e3 / steps
+
+    for (M, N, K) in VENDOR_CELLS:
+        copies = max(2, int(CACHE_BUST_BYTES // (N * K)) + 1)
+        a = synth.random_fp8((M, K), 1, device=dev)
+        ws = [synth.random_fp8((N, K), 2 + i, device=dev) for i in range(copies)]
+        sa = synth.random_scales((1, M), 3, device=dev, lo=0.01, hi=0.1)
+        sb = synth.random_scales((N, 1), 4, device=dev, lo=0.001, hi=0.01)
+        sa_col = sa.t().contiguous()  # [M, 1], the vendor call's layout
+        sb_row = sb.t().contiguous()  # [1, N]
+        ours = lambda i: mx.dynamic_scaled_matmul(a, ws[i % copies], sa, sb, in_spec, w_spec, out_type=torch.bfloat16)
+        theirs = lambda i: torch._scaled_mm(a, ws[i % copies].t(), scale_a=sa_col, scale_b=sb_row, out_dtype=torch.bfloat16)
+        rec = {"M": M, "N": N, "K": K, "scaling": "per-token x per-channel", "weight_copies": copies}
+        try:
+            c_v = theirs(0)
+        except Exception as e:  # a shape the vendor path does not take
+            rec["vendor_error"] = str(e)[:200]
+            c_v = None
+        c_o = ours(0)
+        torch.cuda.synchronize()
+        rec["ours_us"] = round(timed(ours), 2)
+        if c_v is not None:
+            rec["vendor_us"] = round(timed(theirs), 2)
+            rec["vendor_over_ours"] = round(rec["vendor_us"] / rec["ours_us"], 3)
+            big = torch.maximum(c_o.float().abs(), c_v.float().abs()).clamp_min(1e-30)
+            step = torch.exp2(torch.floor(torch.log2(big)) - 7)
+            rec["max_diff_bf16_steps"] = round(float(((c_o.float() - c_v.float()).abs() / step).max()), 2)
+        rec["TFLOP/s_ours"] = round(2.0 * M * N * K / rec["ours_us"] / 1e6, 1)
+        yield rec
+        del ws
+        torch.cuda.empty_cache()
+
+
 def cpu_baseline(wl, budget_s=15.0):
     """The oracle (a port of the reference's host loops) on this host's cores, on a bounded
     slice of the same workload; throughput in the metric's unit."""
@@ -571,6 +636,9 @@ def main():
                     help="the dense kernels' main loops on operands that stay on the chip (LDS-resident: MFMA loop alone and "
                          "with promotions; L2-resident: with copies and barriers), one JSON line each: the issue ceiling the "
                          "dense matmuls are measured against")
+    ap.add_argument("--vendor", action="store_true",
+                    help="per-token x per-channel scaled matmuls through this library and through hipBLASLt (torch._scaled_mm) "
+                         "on the same operands, one JSON line per shape")
     ap.add_argument("--read-ceiling", action="store_true",
                     help="for every decode workload (M <= 16): the matmul kernel's time beside the time of its read-only "
                          "probe (same grid and weight traffic, no arithmetic), one JSON line each")
@@ -627,6 +695,10 @@ def main():
         return
     if args.mfma_ceiling:
         for rec in mfma_ceiling():
+            print(json.dumps(rec), flush=True)
+        return
+    if args.vendor:
+        for rec in vendor_compare():
             print(json.dumps(rec), flush=True)
         return
     if args.read_ceiling:

@@ -471,8 +471,9 @@ int maxfp8_copy_bytes(void* dst, const void* src, int64_t n, void* stream);
 
 /*
  * Measurement aid with no counterpart in the reference: streams the weight matrix b[N, K] (row stride ldb bytes)
- * through the decode (M <= 16) matmul's own grid, LDS ring and DMA instructions -- the shape MAXFP8_ALGO_AUTO
- * would pick for (M, N, K) with row scaling -- and does nothing else: no activations, no MFMA, no stores.  Its
+ * through the weight-streaming (decode) matmul's own grid, LDS ring and DMA instructions -- the shape MAXFP8_ALGO_AUTO
+ * would pick for (M, N, K) with row scaling; that kernel takes up to 64 rows, the probe models it for M <= 16 -- and
+ * does nothing else: no activations, no MFMA, no stores.  Its
  * time is the ceiling the weight-streaming matmul is measured against.
  */
 int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t K, int64_t ldb, void* stream);

@@ -397,9 +397,10 @@ static int matmul_common(void* c, const void* a, const void* b, const void* a_sc
     else if (gemm_skinny_preferred(M, N, K)) algo = MAXFP8_ALGO_SKINNY;
     else algo = MAXFP8_ALGO_TILED;
     // 33 to 64 rows: the tiles win through their K split.  Without the workspace the split needs, a narrow weight
-    // matrix would run on a fraction of the chip: the streaming kernel then.
+    // matrix would run on a fraction of the chip: the streaming kernel then.  (What this shape's own plan needs, not the
+    // worst case over all tile shapes: a plan that does not split runs the same with and without a workspace.)
     if (algo == MAXFP8_ALGO_TILED && M <= gemm_skinny_max_m() && bt.n == 1 &&
-        gemm_tiled_workspace_bytes(M, N, K) > (workspace ? workspace_bytes : 0))
+        gemm_tiled_plan_workspace_bytes(M, N, K, block) > (workspace ? workspace_bytes : 0))
       algo = MAXFP8_ALGO_SKINNY;
   }
   if (algo == MAXFP8_ALGO_NAIVE) {
@@ -452,7 +453,8 @@ int maxfp8_matmul_describe(int64_t M, int64_t N, int64_t K, int block_scaling, i
   if (!buf || len == 0) return 0;
   if (M <= 0 || N <= 0 || K <= 0) return snprintf(buf, len, "nothing to do");
   if (gemm_skinny_preferred(M, N, K)) return snprintf(buf, len, "skinny");
-  if (M <= gemm_skinny_max_m() && !with_workspace && gemm_tiled_workspace_bytes(M, N, K) > 0) return snprintf(buf, len, "skinny");
+  if (M <= gemm_skinny_max_m() && !with_workspace && gemm_tiled_plan_workspace_bytes(M, N, K, block_scaling != 0) > 0)
+    return snprintf(buf, len, "skinny");
   return gemm_tiled_describe(M, N, K, block_scaling != 0, with_workspace != 0, buf, len);
 }
 

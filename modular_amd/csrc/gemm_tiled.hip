@@ -1237,13 +1237,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_grouped_large_k
 // Every block builds the same four prefix tables over the slots in LDS (row tiles of each kind before slot z); a
 // claimed index is a (row tile, column tile) pair, column tiles fastest, found by bisection.  No list of tiles in
 // memory, no host synchronisation.  The result of a tile does not depend on which block computes it.
-constexpr int kGroupedCtrSlots = 64;
+constexpr int kGroupedCtrSlots = 64;      // sets handed to launches that run when they are issued ...
+constexpr int kGroupedCtrSlotsAll = 128;  // ... and as many again for launches recorded into a HIP graph
 constexpr int kGroupedMaxSlots = 512;   // slots (active experts) the LDS tables hold
 // Per launch in flight: a counter per (kind, XCD) and one that counts the blocks that are done.  All zero when the
 // module is loaded; the last block of a launch to finish puts its set back to zero, so a set is clean whenever a
 // launch takes it (sets are handed out round-robin: 64 grouped matmuls are never in flight together).
 constexpr int kGroupedCtrStride = 33;
-static __device__ unsigned int g_grouped_ctr[kGroupedCtrSlots * kGroupedCtrStride];
+static __device__ unsigned int g_grouped_ctr[kGroupedCtrSlotsAll * kGroupedCtrStride];
 
 // One wave: C[rows of the slot, 16 * NTW weight rows from n0 + 16 * NTW * wave] over the whole of K.  The weight slabs
 // (16 * NTW rows x 128 bytes) travel by LDS-DMA through the wave's own ring of DEPTH slots, the activations (at most
@@ -1635,6 +1636,7 @@ static int launch_grouped_large(const GemmArgs& p, dim3 grid, hipStream_t stream
 }
 
 int compute_units();
+static bool stream_is_capturing(hipStream_t stream);
 // One numbering of the launches for both scale modes: the two instantiations below share the counter sets (and, for the
 // work-split kernel, the flags) in device memory, so a counter of their own each would hand the same set, and the same
 // flag value, to a block-scaled and a row-scaled launch.
@@ -1651,8 +1653,16 @@ static int launch_grouped_persist(const GemmArgs& p, hipStream_t stream, const c
                 "the tables sit behind the largest tile");
   constexpr int lds = bodies + 4 * (kGroupedMaxSlots + 1) * 4;
   static_assert(lds + 64 <= 160 * 1024, "one block per CU");
-  // a set of counters per launch in flight (64 sets: launches that follow each other on a stream could share one)
-  const int slot = (int)(next_launch_number() % kGroupedCtrSlots);
+  // A set of counters per launch in flight (64 sets: launches that follow each other on a stream could share one).
+  // A launch recorded into a HIP graph keeps the set of the recording in every replay, and a replay may run beside
+  // launches issued on another stream: recorded launches draw from sets of their own, which no eager launch ever
+  // gets.  (Replays of one graph never overlap each other; two graphs share a set only when 64 launches were recorded
+  // between theirs.)
+  int slot = (int)(next_launch_number() % kGroupedCtrSlots);
+  if (stream_is_capturing(stream)) {
+    static std::atomic<unsigned int> recorded{0};
+    slot = kGroupedCtrSlots + (int)(recorded.fetch_add(1, std::memory_order_relaxed) % (kGroupedCtrSlotsAll - kGroupedCtrSlots));
+  }
   auto kern = gemm_grouped_persist_kernel<BLOCKSCALE>;
   bool& done = attr_done.here();
   if (!done) {

@@ -6,6 +6,8 @@ quantised grouped matmul of the MoE layers, `quantized_grouped_matmul`
 """
 from __future__ import annotations
 
+import weakref
+
 import torch
 
 from .kernels import (dynamic_scaled_matmul, fused_qkv_ragged_matmul_scaled_float8,
@@ -121,23 +123,24 @@ def quantized_fused_qkv_matmul(
 # The reference keeps stacked FP8 expert weights in storage layout [E, in, out] = [E, K, N] and
 # transposes them to [E, N, K] in the graph (quant_ops.py:941-944), where the transposition of a
 # constant weight is folded away at compile time.  The eager equivalent: a storage tensor is
-# transposed once and the K-innermost copy is kept for as long as the storage tensor stays as it is
-# (same memory, same shape, no in-place write since).
-_K_INNERMOST: dict[tuple, tuple[torch.Tensor, torch.Tensor]] = {}
-_K_INNERMOST_MAX = 16
+# transposed once and the K-innermost copy lives exactly as long as the storage tensor object does
+# (one entry per live tensor, found through a weak reference and dropped with it; remade after an
+# in-place write).  A model's every stacked weight and scale tensor keeps its copy, however many
+# layers there are.  A caller that hands in a new view object on every call (`w.data`) would get a
+# new copy every time: such callers transpose once themselves and pass k_innermost=True.
+_K_INNERMOST: dict[int, tuple] = {}   # id(storage tensor) -> (weak reference to it, what it looked like, the copy)
 
 
 def _k_innermost(t: torch.Tensor) -> torch.Tensor:
     """t.transpose(1, 2) as a contiguous tensor, made once per storage tensor."""
-    key = (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t.dtype, t.device, t._version)
+    looks = (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t.dtype, t.device, t._version)
+    key = id(t)
     hit = _K_INNERMOST.get(key)
-    if hit is not None and hit[0] is t:
-        return hit[1]
+    if hit is not None and hit[0]() is t and hit[1] == looks:
+        return hit[2]
     # (fp8 has no copy kernel of its own in every torch build: move the bytes)
     tt = t.view(torch.uint8).transpose(1, 2).contiguous().view(t.dtype) if t.element_size() == 1 else t.transpose(1, 2).contiguous()
-    if len(_K_INNERMOST) >= _K_INNERMOST_MAX:
-        _K_INNERMOST.pop(next(iter(_K_INNERMOST)))
-    _K_INNERMOST[key] = (t, tt)
+    _K_INNERMOST[key] = (weakref.ref(t, lambda _gone, key=key: _K_INNERMOST.pop(key, None)), looks, tt)
     return tt
 
 
@@ -149,6 +152,8 @@ def quantized_grouped_matmul(
     expert_ids: torch.Tensor,
     usage_stats: torch.Tensor,
     quant_config: QuantConfig,
+    *,
+    k_innermost: bool = False,
 ) -> torch.Tensor:
     """Single entry point of the quantised grouped matmuls of a MoE layer (quant_ops.py:880-1007),
     FP8 formats: x [T, K] bf16 with its rows sorted by expert; weight in STORAGE layout [E, K, N]
@@ -159,12 +164,16 @@ def quantized_grouped_matmul(
     Block scaling: both are transposed to the K-innermost orientation of the kernel, x is quantised
     in 1 x block groups with scales of the weight scales' dtype, then the grouped block-scaled matmul.
     Per-channel weight scales with per-token activation scales (no block size): the weight scales
-    are used as they are, the [1, T] scales of the quantiser become the kernel's [T, 1]."""
+    are used as they are, the [1, T] scales of the quantiser become the kernel's [T, 1].
+
+    k_innermost=True (not in the reference, whose compiler folds the transposition of a constant away): weight and
+    block scales are already in the kernel's orientation, [E, N, K] and [E, N/128, K/128] -- for callers that
+    transpose once at load time."""
     if quant_config.format not in (QuantFormat.COMPRESSED_TENSORS_FP8, QuantFormat.FBGEMM_FP8, QuantFormat.BLOCKSCALED_FP8):
         raise ValueError(f"Unsupported quantization format for grouped matmul: {quant_config.format}")
     if weight.dim() != 3:
         raise ValueError(f"expected weight of rank 3 but got {weight.dim()}")
-    weight_t = _k_innermost(weight)
+    weight_t = weight if k_innermost else _k_innermost(weight)
     stats_host = usage_stats.cpu()
     if quant_config.weight_scale.is_rowwise and quant_config.input_scale.block_size is None:
         x_fp8, x_scales = quantize_dynamic_scaled_float8(x, quant_config.input_scale, quant_config.weight_scale,
@@ -173,7 +182,7 @@ def quantized_grouped_matmul(
                                                          expert_start_indices, expert_ids, stats_host)
     assert quant_config.input_scale.block_size is not None
     input_block_size = quant_config.input_scale.block_size[1]
-    scale_t = _k_innermost(weight_scale)
+    scale_t = weight_scale if k_innermost else _k_innermost(weight_scale)
     x_fp8, x_scales = quantize_dynamic_scaled_float8(x, quant_config.input_scale, quant_config.weight_scale,
                                                      group_size_or_per_token=input_block_size, out_type=weight.dtype,
                                                      scales_type=quant_config.weight_scale.dtype)

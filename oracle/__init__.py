@@ -112,6 +112,8 @@ def quantize_dynamic_scaled_fp8(x: np.ndarray, group_size: int, *, in_dtype: int
     """x: [M, K] (uint16 bits for bf16/f16, float32 for f32).  Returns
     (q uint8 [M, K], scales [K/G, scales_ld]); unwritten scale columns hold NaN
     bit patterns (f32) / 0xFFFF (bf16) so a test can see they stay untouched."""
+    if scales_dtype not in (F32, BF16):
+        raise ValueError("the oracle's quantisers write f32 or bf16 scales")
     x = np.ascontiguousarray(x)
     M, K = x.shape
     G = K if group_size == -1 else group_size
@@ -144,6 +146,8 @@ def rms_norm_fused_quantize(x: np.ndarray, gamma: np.ndarray, epsilon: float, we
     """x: [rows, K], gamma: [K] (uint16 bits for bf16/f16, float32 for f32).  epsilon and
     weight_offset are rounded to the input dtype first, as the op registration does
     (builtin_kernels/quantization.mojo:205-213).  Returns (q uint8 [rows, K], scales [1, rows])."""
+    if scales_dtype not in (F32, BF16):
+        raise ValueError("the oracle's quantisers write f32 or bf16 scales")
     x = np.ascontiguousarray(x)
     gamma = np.ascontiguousarray(gamma)
     rows, K = x.shape

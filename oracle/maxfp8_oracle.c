@@ -179,6 +179,7 @@ int orc_quantize_dynamic_scaled_fp8(uint8_t* out, void* scales, const void* in,
                                     int scales_dtype, float scale_ub,
                                     int threads) {
   if (G <= 0 || K % G != 0) return -2;
+  if (scales_dtype != ORC_F32 && scales_dtype != ORC_BF16) return -3;  /* (f16 scales: not restated; the buffer would be written as f32) */
   int64_t ng = K / G;
 #ifdef _OPENMP
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
@@ -231,6 +232,7 @@ int orc_rms_norm_fused_quantize(uint8_t* out, void* scales, const void* in, cons
                                 int64_t rows, int64_t K, int64_t in_row_stride, int64_t out_row_stride,
                                 int in_dtype, int scales_dtype, float epsilon, float weight_offset,
                                 float scale_ub, int threads) {
+  if (scales_dtype != ORC_F32 && scales_dtype != ORC_BF16) return -3;
 #ifdef _OPENMP
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
 #endif

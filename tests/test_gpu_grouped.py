@@ -213,6 +213,49 @@ def test_launches_of_one_kind_of_tile_many_times(dev, counts, N):
         assert torch.equal(got, want), f"launch {launch}"
 
 
+def test_recorded_launch_replays_beside_eager_launches(dev):
+    """A grouped matmul recorded into a HIP graph keeps the counter set of the recording in every replay.  Replays run on
+    one stream while more eager launches than there are counter sets (64) run on another: were the recorded launch's set
+    one of those the eager launches draw from, a replay and an eager launch would sooner or later claim tiles from the
+    same counters at the same time.  Every result of both streams equals the scalar kernel's."""
+    rng = np.random.default_rng(77)
+    counts, N, K = [300] * 24 + [20] * 40, 1024, 512
+    E, T = len(counts), sum(counts)
+    a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (T, K)).astype(np.float32))).to(dev)
+    b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (E, N, K)).astype(np.float32))).to(dev)
+    sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (K // 128, -(-T // 4) * 4))).astype(np.float32)).to(dev)
+    sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (E, N // 128, K // 128))).astype(np.float32)).to(dev)
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32).to(dev)
+    idt = torch.arange(E, dtype=torch.int32).to(dev)
+    stats = torch.tensor([max(counts), E], dtype=torch.int64).to(torch.uint32)
+
+    def launch(algo="auto"):
+        return mx.grouped_dynamic_scaled_fp8_matmul(a, b, sa, sb, off, idt, stats, BLK.input_scale, BLK.weight_scale,
+                                                    out_type=torch.bfloat16, algo=algo)
+
+    want = launch("naive")
+    launch()  # (outside the capture: the kernel's LDS attribute is set at the first launch)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        recorded = launch()
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    eager = []
+    for i in range(72):
+        if i % 6 == 0:
+            recorded.zero_()
+            graph.replay()  # on the current stream, beside the launches of the other
+        with torch.cuda.stream(side):
+            eager.append(launch())
+        if i % 6 == 5:
+            torch.cuda.synchronize()
+            assert torch.equal(recorded, want), f"replay before eager launch {i}"
+    torch.cuda.synchronize()
+    for i, got in enumerate(eager):
+        assert torch.equal(got, want), f"eager launch {i}"
+
+
 def test_more_slots_than_the_persistent_launch_holds(dev):
     """600 active slots: more than the persistent launch's tables hold (512), so the two-launch form runs; exact on
     integer data like every other path."""
@@ -261,7 +304,11 @@ def test_quantized_grouped_matmul_from_the_storage_layout(dev):
     assert len(quant_ops._K_INNERMOST) == n_cached and torch.equal(y, y2)
     wd.view(torch.uint8)[3].zero_()   # expert 3 serves slot 1
     y3 = quant_ops.quantized_grouped_matmul(x.to(dev), wd, sd, off.to(dev), ids_t.to(dev), stats, BLK)
-    assert len(quant_ops._K_INNERMOST) == n_cached + 1
+    assert len(quant_ops._K_INNERMOST) == n_cached, "the tensor's entry is replaced, not added to"
+    # weights already in the kernel's orientation (transposed once at load time)
+    y4 = quant_ops.quantized_grouped_matmul(x.to(dev), wd.view(torch.uint8).transpose(1, 2).contiguous().view(wd.dtype),
+                                            sd.transpose(1, 2).contiguous(), off.to(dev), ids_t.to(dev), stats, BLK, k_innermost=True)
+    assert torch.equal(y4, y3) and len(quant_ops._K_INNERMOST) == n_cached
     lo = counts[0] + counts[1]
     assert torch.equal(y3[:counts[0]], y[:counts[0]]) and torch.equal(y3[lo:], y[lo:]) and not y3[counts[0]:lo].float().any()
 

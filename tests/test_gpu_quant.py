@@ -171,6 +171,7 @@ def test_empty_input(dev):
     (64, 4096, "blk", 128),        # configs[0]
     (2048, 14336, "blk", 128),     # Llama-8B down projection input
     (4096, 7168, "blk", 128),      # DeepSeek-V3 hidden
+    (4096, 16384, "blk", 128),     # DeepSeek-V3 o_proj input: the default benchmark line's quantiser call
     (8, 28672, "row", -1),         # 70B decode, per token
     (300, 8192, "row", -1),
     (1, 4096, "blk", 128),

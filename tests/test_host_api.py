@@ -266,7 +266,21 @@ def test_quantized_grouped_matmul_and_strategy_argument_rules():
     src.view(torch.uint8).add_(1)
     t2 = quant_ops._k_innermost(src)
     assert t2 is not t1 and torch.equal(t2.view(torch.uint8), src.view(torch.uint8).transpose(1, 2))
-    quant_ops._K_INNERMOST.clear()
+    assert len(quant_ops._K_INNERMOST) == 1, "an in-place write replaces the tensor's entry"
+    # every live storage tensor keeps its copy -- a model has more stacked weights than any fixed number of entries -- and
+    # an entry goes when its tensor goes
+    many = [torch.arange(2 * 3 * 5, dtype=torch.uint8).reshape(2, 3, 5) + i for i in range(40)]
+    copies = [quant_ops._k_innermost(t) for t in many]
+    for _ in range(3):
+        assert all(quant_ops._k_innermost(t) is c for t, c in zip(many, copies)), "no tensor is transposed twice"
+    assert len(quant_ops._K_INNERMOST) == 41
+    del many, copies
+    import gc
+    gc.collect()
+    assert len(quant_ops._K_INNERMOST) == 1
+    del src
+    gc.collect()
+    assert len(quant_ops._K_INNERMOST) == 0
     # a CPU tensor never reaches a kernel
     with pytest.raises(RuntimeError, match="GPU only"):
         quant_ops.quantized_grouped_matmul(x, w, torch.ones((2, 2, 1)), off, ids, stats, BLK)

@@ -177,3 +177,12 @@ def test_bf16_scales_are_the_correctly_rounded_quotient():
     recip = np.float32(1.0) / s32
     want_q = oracle.e4m3fn_encode((x * recip[:, None]).astype(np.float32))
     assert np.array_equal(q, want_q)
+
+
+def test_f16_scales_are_refused():
+    # the quantisers restate f32 and bf16 scales only: f16 is refused before any buffer is written
+    x = np.zeros((2, 128), dtype=np.uint16)
+    with pytest.raises(ValueError):
+        oracle.quantize_dynamic_scaled_fp8(x, 128, scales_dtype=oracle.F16)
+    with pytest.raises(ValueError):
+        oracle.rms_norm_fused_quantize(x, np.zeros(128, dtype=np.uint16), 1e-5, scales_dtype=oracle.F16)

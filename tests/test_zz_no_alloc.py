@@ -45,7 +45,10 @@ def test_noalloc_matmul_equals_the_plain_entry_point_twice_in_a_row(dev):
     assert L.maxfp8_matmul_noalloc_max_scratch_bytes() == 32 << 20
     # first call: a K-split plan with ~8 MiB of partial sums; second call: a smaller one that reuses the same array
     # (whatever the first call left in it); then a row-scaled shape and one that needs no scratch at all
-    for (M, N, K, block) in [(256, 576, 7168, True), (128, 512, 4096, True), (4096, 576, 7168, True), (100, 576, 7168, False), (2048, 1024, 512, True)]:
+    for (M, N, K, block) in [(256, 576, 7168, True), (128, 512, 4096, True), (4096, 576, 7168, True), (100, 576, 7168, False), (2048, 1024, 512, True),
+                              # 33 to 64 rows with a plan that does not split: both entry points run the tiles, not the
+                              # weight-streaming kernel
+                              (64, 28672, 4096, True), (48, 8192, 4096, False)]:
         print(f"[no-alloc] {M}x{N}x{K} {'block' if block else 'row'}: {_lib.matmul_describe(M, N, K, block, True)}", flush=True)
         c_plain, c_noalloc, (a, b, sa, sb), need = both_entry_points(M, N, K, block, dev, seed=M + N)
         assert bool(torch.isfinite(c_noalloc.float()).all())
