@@ -176,13 +176,18 @@ int maxfp8_batched_quantize_dynamic_scaled_fp8(
  *               (the reference's three scale dtypes, fp8_quantization.mojo:996-1018): widened to f32
  *               when the epilogue loads them, on every kernel.
  *   algo        a maxfp8_algo value.
- *   workspace   optional device scratch for split-K, 16-byte aligned, of
+ *   workspace   optional device scratch for partial sums (a split of K, a
+ *               last round of tiles computed in pieces), 16-byte aligned, of
  *               workspace_bytes bytes (maxfp8_matmul_workspace_bytes gives the
  *               size that allows every split the library would choose).  NULL
  *               or too small: the matmul runs unsplit (with at most 64 rows:
  *               on the weight-streaming kernel), which is slower only when
- *               its tiles cover a small part of the chip.  The contents
- *               are scratch: overwritten by the call, meaningless afterwards.
+ *               its tiles, or those of its last round, cover a small part of
+ *               the chip.  The f32 sums of a split are added in another order
+ *               than those of the unsplit matmul: results with and without a
+ *               workspace may differ in the last bit of a bf16 element.  The
+ *               contents are scratch: overwritten by the call, meaningless
+ *               afterwards; calls that overlap in time need a workspace each.
  */
 int maxfp8_matmul_dynamic_scaled_fp8(
     void* c, const void* a, const void* b,
@@ -199,15 +204,16 @@ int maxfp8_matmul_dynamic_scaled_fp8(
  * maxfp8_matmul_dynamic_scaled_fp8 for callers that cannot allocate device memory -- code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc -- and therefore cannot bring a
  * workspace.  No counterpart in the reference (its matmul takes temporaries from the device context's
- * caching allocator).  Same arguments without workspace / workspace_bytes, same result: the split-K
- * partial sums go to a static device array of the library,
- * maxfp8_matmul_noalloc_max_scratch_bytes() = 32 MiB per GPU, held from the first use of the library on
- * that GPU until the process ends.  The call allocates and frees nothing, on the device or through any
- * library.  A shape whose K split needs more than the array holds (splits x M x N x 4 bytes; the large-M,
- * narrow-N shapes) is refused with MAXFP8_ERR_WORKSPACE and a message that says so: for those,
- * maxfp8_matmul_dynamic_scaled_fp8 with workspace = NULL runs unsplit and allocates nothing either.  All calls on one GPU share that GPU's array: calls
- * that overlap on one GPU (two streams, two threads) race on it; calls in stream order are safe, and
- * nothing in the array needs clearing between them.
+ * caching allocator).  Same arguments without workspace / workspace_bytes, same result: the partial
+ * sums of a K split, or of the pieces a cut last round of tiles is computed in, go to a static device
+ * array of the library, maxfp8_matmul_noalloc_max_scratch_bytes() = 48 MiB per GPU, held from the first
+ * use of the library on that GPU until the process ends.  The call allocates and frees nothing, on the
+ * device or through any library.  A shape whose K split needs more than the array holds (splits x M x N
+ * x 4 bytes; the large-M, narrow-N shapes) is refused with MAXFP8_ERR_WORKSPACE and a message that says
+ * so: for those, maxfp8_matmul_dynamic_scaled_fp8 with workspace = NULL runs unsplit and allocates
+ * nothing either.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race on it; calls in stream order are safe, and nothing in the array needs
+ * clearing between them.
  */
 int maxfp8_matmul_dynamic_scaled_fp8_noalloc(
     void* c, const void* a, const void* b,
@@ -264,6 +270,15 @@ int maxfp8_matmul_describe(int64_t M, int64_t N, int64_t K, int block_scaling, i
 
 /* Bytes of workspace that lets AUTO use every kernel for this shape. */
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Diagnostic with no counterpart in the reference.  A matmul that computes its last round of tiles in pieces hands
+ * the pieces' sums from block to block inside one launch; a block that waits for a piece does so for a bounded time
+ * (seconds: only a GPU that stopped in the middle of a launch gets there), then fills its tile with NaN and counts
+ * the event.  Returns that count for the current device since the library was loaded (0 in a healthy process), or
+ * a negative maxfp8 error code.  Waits for the device's outstanding work.
+ */
+long long maxfp8_tail_cut_given_up(void);
 
 /*
  * Fused QKV projection with the K / V columns stored straight into a paged KV cache.

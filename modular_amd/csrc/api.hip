@@ -61,8 +61,8 @@ bool gemm_skinny_preferred(int64_t M, int64_t N, int64_t K);
 int gemm_skinny_read_probe(const void* b, int64_t M, int64_t N, int64_t K, int64_t ldb, hipStream_t stream);
 int gemm_persist_probe(const GemmArgs&, bool, int, hipStream_t);
 int gemm_w4_probe(const GemmArgs&, bool, int, int, hipStream_t);
-int gemm_w4_launch(const GemmArgs&, bool, int, hipStream_t);
 bool gemm_w4_ok(const GemmArgs&, bool);
+int gemm_w4_gave_up(unsigned int*);
 
 // v rounded to bf16 / f16 and widened back: how an op parameter of the input's dtype arrives
 static float round_to_dtype(float v, int dtype) {
@@ -87,7 +87,7 @@ static bool is_aligned(const void* p, uintptr_t a) { return (reinterpret_cast<ui
 // for hipGetSymbolAddress -- it is not a device address and is never passed to a kernel or a memory call.  The
 // address is looked up once per device, with that device current, and kept; kernels receive it as an argument,
 // exactly like a caller's workspace.
-constexpr size_t kScratchBytes = (size_t)32 << 20;
+constexpr size_t kScratchBytes = (size_t)48 << 20;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 static void* g_scratch_ptr[64] = {};
 static std::mutex g_scratch_mu;
@@ -138,6 +138,8 @@ static const Tuning* read_tuning(unsigned generation) {
   t->grouped_persist = num("MAXFP8_GROUPED_PERSIST", 1) != 0;
   const int w4 = num("MAXFP8_W4", -1);
   t->w4 = (w4 == 0 || w4 == 5 || w4 == 6) ? w4 : -1;
+  const int w4_split = num("MAXFP8_W4_SPLIT", -1);
+  t->w4_split = (w4_split == 0 || w4_split == 1) ? w4_split : -1;
   t->skinny_alds = num("MAXFP8_SKINNY_ALDS", 1) != 0;
   const char* sb = getenv("MAXFP8_GROUPED_SHARE");
   t->grouped_share = sb ? (float)atof(sb) : 0.5f;
@@ -484,7 +486,7 @@ int maxfp8_matmul_dynamic_scaled_fp8_noalloc(void* c, const void* a, const void*
   if (M > 0 && N > 0 && K > 0 && maxfp8_matmul_workspace_bytes(M, N, K) > 0) need = gemm_tiled_plan_workspace_bytes(M, N, K, block);
   if (need > kScratchBytes)
     MAXFP8_FAIL(MAXFP8_ERR_WORKSPACE,
-                "matmul (no-alloc): the K split of %lld x %lld x %lld uses %zu bytes of scratch, the library's static buffer holds "
+                "matmul (no-alloc): the split of %lld x %lld x %lld uses %zu bytes of scratch, the library's static buffer holds "
                 "%zu; call maxfp8_matmul_dynamic_scaled_fp8 with workspace = NULL (no split, no allocation) or with a workspace",
                 (long long)M, (long long)N, (long long)K, need, kScratchBytes);
   void* ws = nullptr;
@@ -760,6 +762,12 @@ int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t
   if (!is_aligned(b, 16) || K % 16 != 0 || ldb % 16 != 0) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "read probe: needs 16-byte aligned rows and K %% 16 == 0");
   if (!offsets_fit(K, ldb, ldb, 0, false)) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "read probe: rows too long for 32-bit tile offsets");
   return gemm_skinny_read_probe(b, M, N, K, ldb, (hipStream_t)stream);
+}
+
+long long maxfp8_tail_cut_given_up(void) {
+  unsigned int count = 0;
+  const int rc = gemm_w4_gave_up(&count);
+  return rc == MAXFP8_OK ? (long long)count : (long long)rc;
 }
 
 int maxfp8_mfma_issue_probe(int kernel, int blockscale, int level, int64_t slabs, const void* a, const void* b, const float* a_scales,

@@ -59,6 +59,9 @@ struct GemmArgs {
   // work split along K of the persistent kernel: which set of hand-over flags this launch uses, and the value a flag takes
   int streamk_slot;
   unsigned int streamk_seq;
+  // four-wave kernel only: slabs per block of the tail (the tiles beyond the last whole round of the chip, cut evenly along
+  // K among the blocks; 0: every tile is computed whole by one block)
+  int tail_units;           // the four-wave kernel: slabs of a run of its cut tail (0: whole tiles only)
   // fused QKV only
   int kv_on;
   KvStore kv;
@@ -143,5 +146,8 @@ __device__ __forceinline__ GemmArgs batch_view(const GemmArgs& p, int64_t b) {
   return q;
 }
 #endif
+
+// the four-wave kernel's tail cut: blocks, slabs of a run (0: none at this shape), bytes of workspace
+struct W4Split { int blocks; int unit; size_t bytes; };
 
 }  // namespace maxfp8

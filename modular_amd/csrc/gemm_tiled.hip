@@ -1694,7 +1694,8 @@ static bool persist_ok(const GemmArgs& p, bool blockscale, dim3 grid) {
 
 // The four-wave kernel (gemm_w4.hip): 0 (no), or the sixteen-row groups per wave -- 5: tiles of 160 x 256, 6: 192 x 256.
 bool gemm_w4_ok(const GemmArgs& p, bool blockscale);
-int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, hipStream_t stream);
+int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, bool split, hipStream_t stream);
+W4Split gemm_w4_split(int64_t M, int64_t N, int64_t K, int tm);
 
 int compute_units() {
   static int cached[64] = {0};
@@ -1876,6 +1877,7 @@ static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can
 
 static bool streamk_shape(int64_t M, int64_t N, size_t workspace_bytes);
 static bool streamk_planned(int64_t M, int64_t N, int64_t K, bool blockscale);
+size_t gemm_tiled_plan_workspace_bytes(int64_t M, int64_t N, int64_t K, bool blockscale);
 size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   // the largest split count any shape could choose for this problem
   size_t worst = 0;
@@ -1892,6 +1894,11 @@ size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   size_t split_work = 0;
   if (streamk_shape(M, N, ~(size_t)0) && (streamk_planned(M, N, K, true) || streamk_planned(M, N, K, false)))
     split_work = streamk_workspace_bytes();
+  // the four-wave kernel's tail cut: a slot per block for the sums of a piece of a tile
+  for (int bs = 0; bs < 2; ++bs) {
+    const size_t cut = gemm_tiled_plan_workspace_bytes(M, N, K, bs != 0);
+    if (cut > split_work) split_work = cut;
+  }
   return split_k > split_work ? split_k : split_work;
 }
 
@@ -1929,7 +1936,7 @@ static TwoRegionPlan pick_two_regions(int64_t M, int64_t N, int nslab, bool bloc
 
 // What a tiled matmul will launch: one shape (possibly with K split), two regions, or the four-wave kernel (w4: 0, or
 // its sixteen-row groups per wave).
-struct TiledPlan { int variant; int splits; TwoRegionPlan two; bool streamk; int w4; };
+struct TiledPlan { int variant; int splits; TwoRegionPlan two; bool streamk; int w4; bool w4_split; };
 
 // One persistent launch of `tiles` tiles on `slots` CUs, a tile taking t microseconds with the chip full: whole rounds
 // cost t each; a last round that fills only part of the chip is faster than a full one but not in proportion (fewer
@@ -1945,26 +1952,38 @@ static float persistent_cost(int64_t tiles, int slots, float t) {
 // that is 6 ... 9 % less per flop with block scaling and level with row scaling; what decides between the three is
 // mostly how the tile count divides by the CUs.
 static const float kW4SlabBlock[2] = {1.00f, 1.14f}, kW4SlabRow[2] = {0.88f, 1.00f}, kW4Tile = 5.5f;
+// With the tail cut: whole rounds, then a piece per block and the hand-over: a piece's sums written through to memory,
+// then read and added by the tile's last block, piece after piece (measured on 4096 x 7168 x 16384, 104 tiles in two
+// pieces each behind two whole rounds, and on 2048 x 7168 x 18432, 52 tiles in four pieces behind one).
+static const float kW4HandOver = 8.0f, kW4HandOverPiece = 7.0f;
 
 // The shapes the four-wave kernel takes (see gemm_w4_ok; pointers and strides are checked at the launch).
 static bool w4_shape(int64_t M, int64_t N, int64_t K) { return M > 0 && N > 0 && N % 8 == 0 && K >= 512 && K % 256 == 0; }
 
 // Which four-wave tile height, if any, beats `other_cost` (microseconds, what the plan made of the eight-wave shapes
-// costs) by at least 3 %.
-static int pick_w4(int64_t M, int64_t N, int64_t K, bool blockscale, float other_cost) {
-  const int forced = tuning().w4;
+// costs) by at least 3 %, and whether with its tail cut (*split; the workspace has to hold the pieces).
+static int pick_w4(int64_t M, int64_t N, int64_t K, bool blockscale, float other_cost, size_t workspace_bytes, bool* split) {
+  const int forced = tuning().w4, cut = tuning().w4_split;
+  *split = false;
   if (forced == 0 || !tuning().persist || !w4_shape(M, N, K)) return 0;
-  if (forced > 0) return forced;
   const int nslab = (int)(K / 128), slots = compute_units();
   int best = 0;
-  float best_cost = 0.97f * other_cost;
+  float best_cost = forced > 0 ? 3.0e38f : 0.97f * other_cost;  // (a forced height is taken whatever it costs)
   for (int i = 0; i < 2; ++i) {
     const int tm = 5 + i;
-    const float t = (float)nslab * (blockscale ? kW4SlabBlock[i] : kW4SlabRow[i]) + kW4Tile;
+    if (forced > 0 && tm != forced) continue;
+    const float t_slab = blockscale ? kW4SlabBlock[i] : kW4SlabRow[i], t = (float)nslab * t_slab + kW4Tile;
     const int64_t tiles = ceil_div(M, 32 * tm) * ceil_div(N, 256);
-    if (tiles * 4 < (int64_t)slots * 3) continue;  // (well under one round: more, smaller tiles and a K split are the better fit)
-    const float cost = persistent_cost(tiles, slots, t);
-    if (cost < best_cost) { best = tm; best_cost = cost; }
+    if (forced <= 0 && tiles * 4 < (int64_t)slots * 3) continue;  // (well under one round: more, smaller tiles and a K split are the better fit)
+    const float whole = persistent_cost(tiles, slots, t);
+    if (whole < best_cost) { best = tm; best_cost = whole; *split = false; }
+    const W4Split sp = gemm_w4_split(M, N, K, tm);
+    if (cut != 0 && sp.unit > 0 && sp.bytes <= workspace_bytes) {
+      const float pieces = (float)ceil_div(nslab, sp.unit);
+      float with_cut = (float)(tiles / sp.blocks) * t + (float)sp.unit * t_slab + kW4Tile + kW4HandOver + kW4HandOverPiece * (pieces - 1.f);
+      if (cut == 1) with_cut *= 1.0e-3f;  // (switched on: wherever there is one)
+      if (with_cut < best_cost) { best = tm; best_cost = with_cut; *split = true; }
+    }
   }
   return best;
 }
@@ -1980,7 +1999,7 @@ static bool streamk_shape(int64_t M, int64_t N, size_t workspace_bytes) {
 }
 static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, bool has_workspace, size_t workspace_bytes,
                            int64_t batch, bool kv_on) {
-  TiledPlan plan = {0, 1, {0, 0, 0, 0, 0.f}, false, 0};
+  TiledPlan plan = {0, 1, {0, 0, 0, 0, 0.f}, false, 0, false};
   const int nslab = (int)ceil_div(K, 128);
   plan.variant = tile_override();
   const bool free_choice = plan.variant == 0;
@@ -2014,7 +2033,7 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
     float other = plan.two.axis ? plan.two.cost : region_cost(M, N, nslab, t, blockscale);
     if (!plan.two.axis && persist_shape(M, N, plan.variant))
       other = persistent_cost(tiles, t.slots, (float)nslab * (blockscale ? t.t_slab_block : t.t_slab_row) + tile_overhead(M, N, plan.variant - 1, 1));
-    plan.w4 = pick_w4(M, N, K, blockscale, other);
+    plan.w4 = pick_w4(M, N, K, blockscale, other, has_workspace ? workspace_bytes : 0, &plan.w4_split);
   }
   return plan;
 }
@@ -2030,6 +2049,7 @@ size_t gemm_tiled_plan_workspace_bytes(int64_t M, int64_t N, int64_t K, bool blo
   const TiledPlan plan = make_plan(M, N, K, blockscale, true, ~(size_t)0, 1, false);
   // (a plan that splits the work between blocks instead has splits == 1: without the 64 MB of slots it needs, the
   // planner falls back to the persistent kernel, which forms the same sums)
+  if (plan.w4 && plan.w4_split) return gemm_w4_split(M, N, K, plan.w4).bytes;
   return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)N * 4 : 0;
 }
 
@@ -2061,6 +2081,9 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
   auto count = [](int64_t m, int64_t n, const TileShape& t) { return (long long)(ceil_div(m, t.bm) * ceil_div(n, t.bn)); };
   // (what a bf16 result with 16-byte aligned rows gets)
   auto how = [](int64_t m, int64_t n, int variant) { return persist_shape(m, n, variant) ? " persistent" : (variant == 4 ? " three-stage" : ""); };
+  if (plan.w4 && plan.w4_split)
+    return snprintf(buf, len, "%dx256 x%lld persistent, four waves, tail cut in pieces of %d slabs", 32 * plan.w4,
+                    (long long)(ceil_div(M, 32 * plan.w4) * ceil_div(N, 256)), gemm_w4_split(M, N, K, plan.w4).unit);
   if (plan.w4)
     return snprintf(buf, len, "%dx256 x%lld persistent, four waves", 32 * plan.w4, (long long)(ceil_div(M, 32 * plan.w4) * ceil_div(N, 256)));
   if (plan.two.axis && !plan.streamk) {
@@ -2103,7 +2126,7 @@ int gemm_tiled_dispatch(const GemmArgs& p_in, bool blockscale, size_t workspace_
   if (plan.w4) {
     p.splits = 1;
     // (the plan knows the shape; whether this call's pointers and strides suit the kernel is checked here)
-    if (gemm_w4_ok(p, blockscale)) return gemm_w4_launch(p, blockscale, plan.w4, stream);
+    if (gemm_w4_ok(p, blockscale)) return gemm_w4_launch(p, blockscale, plan.w4, plan.w4_split && p.workspace != nullptr, stream);
   }
   if (plan.two.axis) {
     const TwoRegionPlan& two = plan.two;

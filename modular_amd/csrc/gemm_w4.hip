@@ -31,11 +31,20 @@
 // accumulators are issued LAG MFMAs later, when the product has left the matrix pipe.
 //
 // Tiles: any M and any N that is a multiple of 8 (rows of either operand past the end read as zero through the buffer
-// descriptors, stores of rows past M fall outside C's descriptor, lanes whose columns lie past N store nothing), K an even number (at least four) of whole 128-byte slabs (the two sets of fragment registers
-// alternate).
+// descriptors, stores of rows past M fall outside C's descriptor, lanes whose columns lie past N store nothing), K an
+// even number (at least four) of whole 128-byte slabs (the two sets of fragment registers alternate).
 // Sums are formed in the same order as by the eight-wave kernels (one product per slab, promoted in slab order):
 // results are bit-equal to theirs.
+//
+// The last round.  Tiles are dealt out in whole rounds of the blocks; what is left for a last round is often a fraction
+// of a round, and its tiles take as long as any.  Where the caller brings a workspace, the tiles beyond the last whole
+// round are cut along K into two to four pieces, a block per piece (see the job list in w4_body): the pieces' f32 sums go
+// through the workspace and the block that holds a tile's last slabs adds them up, in slab order, and stores the tile.
+// These sums are added in another order than the uncut kernel's: equal where every sum is exact, a bf16 step apart at
+// most elsewhere; the same bits from launch to launch.
 #include <stdlib.h>
+
+#include <atomic>
 
 #include "common.h"
 #include "gemm_args.h"
@@ -60,8 +69,30 @@ __device__ __forceinline__ v8i in_agprs(v8i f) {
   return f;
 }
 
+// x, as a value the optimiser cannot see through and that is the same in every lane (in a scalar register)
+__device__ __forceinline__ int opaque_uniform(int x) {
+  asm volatile("" : "+v"(x));
+  return __builtin_amdgcn_readfirstlane(x);
+}
+
+// the lane's number, formed where it is asked for (from the execution mask) and opaque to the optimiser: a value that
+// is wanted only behind the slab loop then occupies no register across it
+__device__ __forceinline__ int lane_here() {
+  int l = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  asm volatile("" : "+v"(l));
+  return l;
+}
+
 // the immediate of s_waitcnt on gfx9: vmcnt in bits 3:0 and 15:14, expcnt (left at its maximum) in 6:4, lgkmcnt in 11:8
 constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) { return (vmcnt & 15) | ((vmcnt >> 4) << 14) | (7 << 4) | (lgkmcnt << 8); }
+
+// Flags of the tail pieces: a set per launch in flight (handed out round-robin: the first half to ordinary launches,
+// the second to launches recorded into a graph, which replay with the set of the recording), a word per block.  A
+// flag is raised by the block that wrote a piece and put back to zero by the one block that takes the piece, so a
+// launch leaves its set as it found it.  And the count of pieces a block gave up waiting for.
+constexpr int kW4FlagSets = 64, kW4MaxBlocks = 512;
+static __device__ unsigned int g_w4_flags[kW4FlagSets * kW4MaxBlocks];
+static __device__ unsigned int g_w4_gave_up;
 
 // PROBE (measurement aid, results meaningless): 0 the matmul; 1 the same loop with every copy reading tile (0, 0) and
 // slabs 0..7 over and over, so that its operands stay in L2; 2 the same without copies, waits and barriers -- the
@@ -90,12 +121,53 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // ---- this block's tiles: every nb-th tile of its XCD's contiguous run (blocks are dealt to the XCDs round-robin)
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN, total = tiles_m * tiles_n;
   const int bs_rows = (p.N + 127) / 128;  // rows of the weight scales: a wave whose columns all lie past N reads the last one
-  const int xcd = blockIdx.x & 7;
-  const int run_begin = xcd * (total >> 3) + (xcd < (total & 7) ? xcd : (total & 7));
-  const int run_len = (total >> 3) + (xcd < (total & 7) ? 1 : 0);
-  const int nb = ((int)gridDim.x - xcd + 7) >> 3;
-  const int my = blockIdx.x >> 3;
-  const int njobs = PROBE ? 1 : (my < run_len ? (run_len - my + nb - 1) / nb : 0);
+  // The tail (p.tail_units = u > 0; the host then launches a multiple of 8 blocks and no more than there are tiles): the
+  // T tiles beyond the last whole round of the blocks are not dealt out whole.  Each is cut along K into pieces of u slabs
+  // (P = ceil(slabs / u) of them, the same cuts in every tile; u and the slabs of a tile are multiples of 4, so every
+  // piece is at least four slabs and an even number; T P is no more than the blocks), and block number c (blocks of an
+  // XCD next to each other) takes piece c / T of tile c % T: the last round then takes the time of a piece, and the
+  // blocks of an XCD walk the same slabs of neighbouring tiles in step, as they do in the whole rounds -- they find each
+  // other's operands in their L2.
+  //
+  // A job: slabs [s0, s1) of a tile.  WHOLE: all of them, the tile is stored.  PART: the sum goes to this block's slot of
+  // the workspace and a flag follows.  LAST (the piece with the tile's last slab): waits for the tile's other pieces,
+  // adds them in the order of their slabs and stores the tile.
+  //
+  // (Jobs are worked out from the block's number every time one begins, behind a value the optimiser cannot see through:
+  // kept in scalar registers across the slab loop, the block's bookkeeping pushed the loop's own values out.)
+  enum { WHOLE = 0, PART = 1, LAST = 2 };
+  struct Job { int tile, s0, s1, kind; };
+  struct Plan { int main_total, run_begin, nb, my, n_main, tail_c, tail_u; };
+  auto plan_of = [&]() {
+    const int bid = opaque_uniform((int)blockIdx.x), G = (int)gridDim.x;
+    const int xcd = bid & 7, my = bid >> 3;
+    const int tail_u = PROBE ? 0 : p.tail_units;
+    const int main_total = tail_u > 0 ? (total / G) * G : total;
+    const int run_begin = xcd * (main_total >> 3) + (xcd < (main_total & 7) ? xcd : (main_total & 7));
+    const int run_len = (main_total >> 3) + (xcd < (main_total & 7) ? 1 : 0);
+    const int nb = (G - xcd + 7) >> 3;
+    const int n_main = PROBE ? 1 : (my < run_len ? (run_len - my + nb - 1) / nb : 0);
+    return Plan{main_total, run_begin, nb, my, n_main, xcd * (G >> 3) + my, tail_u};
+  };
+  // job k of this block; k == n_main: its piece of the tail, if it has one; *count = the number of jobs
+  auto job_of = [&](int k, int* count) {
+    const Plan pl = plan_of();
+    Job tail = {0, 0, 0, WHOLE};
+    int n_tail = 0;
+    if (pl.tail_u > 0) {
+      const int T = total - pl.main_total, P = (nslab + pl.tail_u - 1) / pl.tail_u;
+      if (pl.tail_c < T * P) {
+        const int q = pl.tail_c / T, s0 = q * pl.tail_u, s1 = min(s0 + pl.tail_u, nslab);
+        tail = Job{pl.main_total + (pl.tail_c - q * T), s0, s1, s1 == nslab ? (s0 == 0 ? WHOLE : LAST) : PART};
+        n_tail = 1;
+      }
+    }
+    if (count) *count = pl.n_main + n_tail;
+    if (k < pl.n_main) return Job{pl.run_begin + pl.my + k * pl.nb, 0, nslab, WHOLE};
+    return tail;
+  };
+  int njobs = 0;
+  Job job = job_of(0, &njobs);
   if (njobs <= 0) return;
 
   // ---- global -> LDS copy plan (LDS-DMA, 16 bytes per lane, 8 rows x 128 bytes per instruction; lane (r, p) fetches
@@ -198,11 +270,11 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
 
   // ---- prologue: slabs 0 and 1 of the first tile
   int tm, tn;
-  tile_coords(run_begin + my, tiles_m, tiles_n, tm, tn);
+  tile_coords(job.tile, tiles_m, tiles_n, tm, tn);
   if constexpr (PROBE != 0) tm = tn = 0;
   TileAt cur_at = tile_at(tm, tn);
   {
-    const SlabAt s0 = slab_at(cur_at, 0, 0u), s1 = slab_at(cur_at, 1, 0u), s2 = slab_at(cur_at, 2, 0u);
+    const SlabAt s0 = slab_at(cur_at, job.s0, 0u), s1 = slab_at(cur_at, job.s0 + 1, 0u), s2 = slab_at(cur_at, job.s0 + 2, 0u);
 #pragma unroll
     for (int idx = 0; idx < PER_A; ++idx) dma_a(s0, 0, idx);
 #pragma unroll
@@ -229,7 +301,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     return blk < bs_rows ? blk : bs_rows - 1;
   };
   // The weight-block scale of a slab is element bs_cur of the weight scales: that of the slab to come is loaded a slab ahead.
-  uint32_t bs_cur = (uint32_t)(bs_block(tn) * p.b_scales_ld);
+  uint32_t bs_cur = (uint32_t)(bs_block(tn) * p.b_scales_ld + job.s0);
   float bs_nxt = 1.f;
   if constexpr (BLOCKSCALE) bs_nxt = scalar_load_f32(p.b_scales + bs_cur);
 
@@ -241,6 +313,10 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
 #pragma unroll
   for (int mt = 0; mt < TM; ++mt) af[0][mt] = read_afrag(0, mt);
   if constexpr (BLOCKSCALE) sraw[0] = read_scales(0);
+#pragma unroll
+  for (int t = 0; t < TN; ++t) bf[0][t] = in_agprs(bf[0][t]);
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt) af[0][mt] = in_agprs(af[0][mt]);
 
   // (probe: the core clock's cycle counter and the constant 100 MHz counter, around the slab loop)
   [[maybe_unused]] uint64_t probe_c0 = 0, probe_r0 = 0;
@@ -255,17 +331,25 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // of its slab + 3.  Running offsets, 128 bytes (one row of scales) further with every slab, set to the next tile's
   // first slab when they pass the end of K -- a handful of scalar instructions per slab; worked out from the slab number
   // every time they were two dozen, and a wave alone on its SIMD pays for every instruction it issues.
-  SlabAt cur = slab_at(cur_at, 2, 0u);
-  cur.b = slab_at(cur_at, 3, 0u).b;
+  SlabAt cur = slab_at(cur_at, job.s0 + 2, 0u);
+  cur.b = slab_at(cur_at, job.s0 + 3, 0u).b;
+
+  // the pieces of tail tiles travel through the workspace: slot c = the sum of block c's PART, 64 lanes x 16 bytes per
+  // fragment; flags (one per block and launch in flight) say that a slot is written.  The hand-over crosses XCDs, whose L2s
+  // are not coherent with each other: stores and loads of the slots carry the device-scope cache policy.
+  constexpr int SLOT_BYTES = BM * BN * 4;
+  constexpr int kDeviceScope = 17;  // sc0 | sc1
 
   for (int k = 0; k < njobs; ++k) {
     const bool has_next = k + 1 < njobs;
+    const Job next_job = has_next ? job_of(k + 1, nullptr) : job;
     int tm2 = tm, tn2 = tn;
-    if (has_next) tile_coords(run_begin + my + (k + 1) * nb, tiles_m, tiles_n, tm2, tn2);
+    if (has_next) tile_coords(next_job.tile, tiles_m, tiles_n, tm2, tn2);
     const TileAt next_at = tile_at(tm2, tn2);
-    // slab 0 of the next tile (of nothing behind the block's last tile: offsets past 2^31 read as zeros)
-    const SlabAt next0 = slab_at(next_at, 0, has_next ? 0u : 0x80000000u);
-    const uint32_t next_bs0 = (uint32_t)(bs_block(tn2) * p.b_scales_ld);
+    // the first slab of the next job (of nothing behind the block's last one: offsets past 2^31 read as zeros)
+    const SlabAt next0 = slab_at(next_at, next_job.s0, has_next ? 0u : 0x80000000u);
+    const uint32_t next_bs0 = (uint32_t)(bs_block(tn2) * p.b_scales_ld + next_job.s0);
+    const int job_end = job.s1;
 
     v4f acc[TM][TN];
 #pragma unroll
@@ -304,9 +388,9 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         cur.b = (cur.b + 128u) & 1023u;
         cur.s = cur.s + s_slab_step == 8u * s_slab_step ? 0u : cur.s + s_slab_step;
       } else {
-        cur.a = slab + 3 == nslab ? next0.a : cur.a + 128u;
-        cur.s = slab + 3 == nslab ? next0.s : cur.s + s_slab_step;
-        cur.b = slab + 4 == nslab ? next0.b : cur.b + 128u;
+        cur.a = slab + 3 == job_end ? next0.a : cur.a + 128u;
+        cur.s = slab + 3 == job_end ? next0.s : cur.s + s_slab_step;
+        cur.b = slab + 4 == job_end ? next0.b : cur.b + 128u;
       }
 
       float s_cur[TM];
@@ -316,7 +400,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         for (int mt = 0; mt < TM; ++mt) s_cur[mt] = sraw[PAR].v[mt] * bs;
         // the weight-block scale of the next slab (of the next tile behind this tile's last slab)
         if constexpr (PROBE != 0) bs_cur = (bs_cur & ~7u) | ((bs_cur + 1u) & 7u);
-        else bs_cur = slab + 1 == nslab ? next_bs0 : bs_cur + 1u;
+        else bs_cur = slab + 1 == job_end ? next_bs0 : bs_cur + 1u;
         bs_nxt = scalar_load_f32(p.b_scales + bs_cur);
       }
       [[maybe_unused]] v4f part[LAG + 1];
@@ -372,19 +456,90 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
 
     constexpr std::integral_constant<int, 0> EVEN{};
     constexpr std::integral_constant<int, 1> ODD{};
-    if (stored) slab_body(EVEN, std::true_type{}, 0);
-    else slab_body(EVEN, std::false_type{}, 0);
-    slab_body(ODD, std::false_type{}, 1);
-    for (int slab = 2; slab < nslab; slab += 2) {
+    // (a job begins at an even slab and has an even number of slabs, four at least)
+    if (stored) slab_body(EVEN, std::true_type{}, job.s0);
+    else slab_body(EVEN, std::false_type{}, job.s0);
+    slab_body(ODD, std::false_type{}, job.s0 + 1);
+    for (int slab = job.s0 + 2; slab < job_end; slab += 2) {
       slab_body(EVEN, std::false_type{}, slab);
       slab_body(ODD, std::false_type{}, slab + 1);
     }
 
     if constexpr (PROBE != 0) {
-      if (p.workspace != nullptr && tid == 0) {
+      if (p.workspace != nullptr && wave == 0 && lane_here() == 0) {
         uint64_t* out = reinterpret_cast<uint64_t*>(p.workspace) + 2 * blockIdx.x;
         out[0] = clock64() - probe_c0;
         out[1] = wall_clock64() - probe_r0;
+      }
+    }
+    if (job.kind == PART) {
+      // ---- the sum of this piece goes to the block's slot; the flag follows once every wave's stores have completed
+      const Plan pl = plan_of();
+      const int tail_c = pl.tail_c;
+      const __amdgpu_buffer_rsrc_t w_rsrc = t2_rsrc(p.workspace, t2_clamp_u32((int64_t)gridDim.x * SLOT_BYTES));
+      unsigned int* const flags = g_w4_flags + (size_t)p.streamk_slot * kW4MaxBlocks;
+      const uint32_t base = (uint32_t)tail_c * SLOT_BYTES + (uint32_t)wave * (SLOT_BYTES / 4);
+      const int lane_p = lane_here();
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const v4f a4 = acc[i][j];
+          const v4u_t v = {__float_as_uint(a4[0]), __float_as_uint(a4[1]), __float_as_uint(a4[2]), __float_as_uint(a4[3])};
+          buffer_store_b128_guarded<kDeviceScope>(v, w_rsrc, (uint32_t)lane_p * 16u, base + (uint32_t)(i * TN + j) * 1024u);
+        }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      if (wave == 0 && lane_p == 0) __hip_atomic_store(flags + tail_c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      stored = false;  // (nothing of this wave is in flight any more)
+      job = next_job;
+      tm = tm2;
+      tn = tn2;
+      cur_at = next_at;
+      continue;
+    }
+    if (job.kind == LAST) {
+      // ---- the tile's other pieces, in the order of their slabs
+      const Plan pl = plan_of();
+      const int tail_c = pl.tail_c;
+      const __amdgpu_buffer_rsrc_t w_rsrc = t2_rsrc(p.workspace, t2_clamp_u32((int64_t)gridDim.x * SLOT_BYTES));
+      unsigned int* const flags = g_w4_flags + (size_t)p.streamk_slot * kW4MaxBlocks;
+      // (the piece before slab q u of tile t is the work of block (q - 1) T + t ...)
+      const int T = total - pl.main_total;
+      const int lane_l = lane_here();
+      for (int c = job.tile - pl.main_total; c < tail_c; c += T) {
+        // (in practice long written: the other blocks computed their pieces first.  Every lane reads the same word; a
+        // block that gives up -- its partner never ran: a hung GPU -- poisons its tile with NaN and counts the event)
+        bool there = false;
+        for (int spin = 0; spin < (1 << 22); ++spin) {
+          // (one value for the wave, so that the loop's exit is the same for every lane)
+          const unsigned int seen = __builtin_amdgcn_readfirstlane(__hip_atomic_load(flags + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+          if (seen != 0u) { there = true; break; }
+          __builtin_amdgcn_s_sleep(16);
+        }
+        asm volatile("" ::: "memory");
+        // (every wave has seen the flag: down it goes, for the next launch that uses this set)
+        __builtin_amdgcn_s_barrier();
+        if (wave == 0 && lane_l == 0) {
+          if (there) __hip_atomic_store(flags + c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          else atomicAdd(&g_w4_gave_up, 1u);
+        }
+        const uint32_t base = (uint32_t)c * SLOT_BYTES + (uint32_t)wave * (SLOT_BYTES / 4);
+
+        // (a row of fragments at a time: all the loads in flight at once would want as many registers again as the sums)
+        const uint32_t poison = there ? 0u : 0x7fc00000u;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          v4u_t v[TN];
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            v[j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (uint32_t)lane_l * 16u, base + (uint32_t)(i * TN + j) * 1024u, kDeviceScope);
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] += v4f{__uint_as_float(v[j].x | poison), __uint_as_float(v[j].y | poison), __uint_as_float(v[j].z | poison),
+                             __uint_as_float(v[j].w | poison)};
+          if (i & 1) asm volatile("" ::: "memory");
+        }
       }
     }
     // ---- the tile leaves, 16 rows x 64 columns of the wave's part at a time
@@ -408,8 +563,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     const uint32_t c_tile = ((uint32_t)(tm * BM + wm * WM) * (uint32_t)p.ldc + (uint32_t)(tn * BN + wn * WN)) * 2u;
     // (the lane's offsets are formed here, out of sight of the optimiser: hoisted out of the tile loop they would sit in
     // vector registers all through the slab loop, which has none to spare)
-    int lane_e = lane;
-    asm volatile("" : "+v"(lane_e));
+    const int lane_e = lane_here();
     const int lm_e = lane_e & 15, lq_e = lane_e >> 4, rr = lane_e >> 3, cc = lane_e & 7;
     const uint32_t c_lane = (uint32_t)rr * c_row_bytes + (uint32_t)cc * 16u;
     // (the last column tile may reach past N, which is a multiple of 8: a lane whose eight columns lie there stores out of
@@ -451,6 +605,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       }
     }
     stored = true;
+    job = next_job;
     tm = tm2;
     tn = tn2;
     cur_at = next_at;
@@ -502,14 +657,62 @@ static int launch_w4(const GemmArgs& p, unsigned blocks, hipStream_t stream, con
   return launch_status(name);
 }
 
-// rows of a tile: 32 * tm (tm = 5 or 6 sixteen-row groups per wave)
-int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, hipStream_t stream) {
+// The tail cut of an M x N x K matmul in tiles of 32 tm rows: the blocks it runs on, the slabs of a piece and the bytes
+// of workspace (a slot of a tile's sums per block); unit == 0: this shape has no cut.  It takes more than one tile per
+// block (what is cut is what lies beyond the last whole round), slabs in whole fours per tile, and a last round of at
+// most half the blocks' number of tiles: every tile is cut into the same number of pieces, two to four, at the same
+// slabs, and every piece is one block's work.
+W4Split gemm_w4_split(int64_t M, int64_t N, int64_t K, int tm) {
+  const W4Split none = {0, 0, 0};
+  const int64_t tiles = ceil_div(M, 32 * tm) * ceil_div(N, 256), nslab = K / 128;
+  int g = (compute_units() / 8) * 8;
+  if (g > kW4MaxBlocks) g = kW4MaxBlocks;
+  if (g < 8 || K % 512 != 0 || tiles <= g || tiles % g == 0) return none;
+  int64_t pieces = g / (tiles % g);
+  if (pieces > 4) pieces = 4;
+  if (pieces < 2) return none;
+  const int64_t u = ceil_div(ceil_div(nslab, pieces), 4) * 4;
+  if (u >= nslab) return none;
+  return W4Split{g, (int)u, (size_t)g * 32 * tm * 256 * 4};
+}
+
+// rows of a tile: 32 * tm (tm = 5 or 6 sixteen-row groups per wave); split: cut the tail (p.workspace holds what
+// gemm_w4_split asks for)
+int gemm_w4_launch(const GemmArgs& p_in, bool blockscale, int tm, bool split, hipStream_t stream) {
+  GemmArgs p = p_in;
   const int64_t tiles = ceil_div(p.M, 32 * tm) * ceil_div(p.N, 256);
   const int cus = compute_units();
-  const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+  unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+  p.tail_units = 0;
+  if (split) {
+    const W4Split sp = gemm_w4_split(p.M, p.N, p.K, tm);
+    if (sp.unit > 0 && p.workspace != nullptr) {
+      blocks = (unsigned)sp.blocks;
+      p.tail_units = sp.unit;
+      // a set of flags per launch in flight; a launch recorded into a graph keeps the set of the recording in every
+      // replay, which may run beside launches of another stream: recorded launches draw from sets of their own
+      static std::atomic<unsigned int> issued{0}, recorded{0};
+      hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        status = hipStreamCaptureStatusNone;
+      }
+      p.streamk_slot = status == hipStreamCaptureStatusNone ? (int)(issued.fetch_add(1, std::memory_order_relaxed) % (kW4FlagSets / 2))
+                                                            : kW4FlagSets / 2 + (int)(recorded.fetch_add(1, std::memory_order_relaxed) % (kW4FlagSets / 2));
+    }
+  }
   if (tm == 5)
     return blockscale ? launch_w4<5, true, 0>(p, blocks, stream, "gemm_w4_block_160x256") : launch_w4<5, false, 0>(p, blocks, stream, "gemm_w4_row_160x256");
   return blockscale ? launch_w4<6, true, 0>(p, blocks, stream, "gemm_w4_block_192x256") : launch_w4<6, false, 0>(p, blocks, stream, "gemm_w4_row_192x256");
+}
+
+// Pieces of a cut tail that a block stopped waiting for, on the current device since the library was loaded (0 unless
+// a GPU hung in the middle of a launch; the tiles concerned hold NaN).  Waits for the device's work to finish.
+int gemm_w4_gave_up(unsigned int* count) {
+  hipError_t e = hipDeviceSynchronize();
+  if (e == hipSuccess) e = hipMemcpyFromSymbol(count, HIP_SYMBOL(g_w4_gave_up), sizeof(unsigned int));
+  if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "tail cut: cannot read the count of abandoned pieces: %s", hipGetErrorString(e));
+  return MAXFP8_OK;
 }
 
 // measurement aid: the kernel's main loop on operands that stay in L2 (level 1) or in LDS (level 2), on every CU

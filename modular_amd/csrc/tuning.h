@@ -27,6 +27,7 @@ struct Tuning {
   bool one_region = false;
   bool persist = true;
   int w4 = -1;               // -1: the planner decides
+  int w4_split = -1;         // the four-wave kernel's tail cut: -1 the planner decides, 0 never, 1 wherever the shape has one
   int streamk = 1;
   int big_rows = 1024;
   bool grouped_persist = true;

@@ -211,7 +211,7 @@ FORMS = {"eight waves": "0", "four waves, 160 rows": "5", "four waves, 192 rows"
 @pytest.mark.parametrize("kind", ["block", "row"])
 @pytest.mark.parametrize("form", list(FORMS))
 def test_persistent_kernel_equals_per_tile_kernel(dev, tune, M, N, K, kind, form):
-    tune(MAXFP8_TILE="1", MAXFP8_W4=FORMS[form])
+    tune(MAXFP8_TILE="1", MAXFP8_W4=FORMS[form], MAXFP8_W4_SPLIT="0")   # (whole tiles only: pieces add up in another order)
     if kind == "block":
         a, b, sa, sb = make_block(M, N, K, seed=M + K)
         cfg = BLK
@@ -264,7 +264,7 @@ def test_four_wave_kernel_ragged_edges(dev, tune, M, N, K, kind, rows):
                                                 K, K, N, gin, gw, *g, a_ld, b_ld, _lib.BF16, _lib.F32, _lib.ALGO_TILED, None, 0, stream)
         assert st == 0, _lib.last_error()
 
-    tune(MAXFP8_TILE="1", MAXFP8_W4=rows)
+    tune(MAXFP8_TILE="1", MAXFP8_W4=rows, MAXFP8_W4_SPLIT="0")
     assert "four waves" in _lib.matmul_describe(M, N, K, kind == "block", False)
     guard = torch.full((M + 2, N), -7.0, dtype=torch.bfloat16, device=dev)
     run(guard[1:M + 1])
@@ -289,7 +289,7 @@ def test_persistent_kernel_leaves_other_outputs_alone(dev, tune):
 def test_persistent_kernel_many_tiles_per_block_repeated(dev, tune, form):
     # short K, sixteen tiles per block: the stores of one tile are still in flight when the next tile's first slab
     # is waited for.  Twelve launches with fresh activations, each compared with the per-tile kernel.
-    tune(MAXFP8_TILE="1", MAXFP8_W4=FORMS[form])
+    tune(MAXFP8_TILE="1", MAXFP8_W4=FORMS[form], MAXFP8_W4_SPLIT="0")
     M, N, K = 8192, 32768, 256
     b = synth.random_fp8((N, K), 77).to(dev)
     sb = synth.random_scales((N // 128, K // 128), 78).to(dev)
@@ -302,6 +302,150 @@ def test_persistent_kernel_many_tiles_per_block_repeated(dev, tune, form):
         want = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
         torch.cuda.synchronize()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"launch {seed}"
+
+
+# ---- the four-wave kernel with its last round cut into pieces ------------------------------------------------------
+# Tiles beyond the last whole round of the CUs are each cut along K into two to four pieces, a block per piece: the
+# pieces' f32 sums travel through the workspace and the block with a tile's last slabs adds them up.  That changes the
+# order of the f32 sums: bit-equal to the uncut kernel where every sum is exact, one bf16 step apart at most elsewhere.
+TAIL_CUT_SHAPES = [(2040, 6144, 4096), (3000, 7000, 3584), (4096, 7168, 2048), (2048, 7168, 18432)]
+
+
+def _tail_cut_operands(M, N, K, kind, exact, dev, seed=0):
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K + seed)
+    if exact:   # small integers times powers of two: every partial sum is exact in f32, whatever its order
+        a = torch.randint(-2, 3, (M, K), generator=g).float().to(torch.float8_e4m3fn)
+        b = torch.randint(-2, 3, (N, K), generator=g).float().to(torch.float8_e4m3fn)
+        if kind == "block":
+            sa = torch.pow(2.0, torch.randint(-3, 2, (K // 128, -(-M // 4) * 4), generator=g).float())
+            sb = torch.pow(2.0, torch.randint(-3, 2, (-(-N // 128), K // 128), generator=g).float())
+        else:
+            sa = torch.pow(2.0, torch.randint(-3, 2, (1, M), generator=g).float())
+            sb = torch.pow(2.0, torch.randint(-3, 2, (N, 1), generator=g).float())
+    elif kind == "block":
+        a, b, sa, sb = make_block(M, N, K, seed=M + K + seed)
+    else:
+        a, b = synth.random_fp8((M, K), M + seed), synth.random_fp8((N, K), N + 1)
+        sa, sb = synth.random_scales((1, M), 3, lo=0.01, hi=0.1), synth.random_scales((N, 1), 4, lo=0.001, hi=0.01)
+    return [t.to(dev) for t in (a, b, sa, sb)]
+
+
+def _one_bf16_step_apart(got, want):
+    """|got - want| within a bf16 step of the element, or (sums that cancel to nearly nothing) within what reordering
+    f32 sums of this size can move them: 2^-12 of the mean magnitude."""
+    g, w = got.float(), want.float()
+    assert bool(torch.isfinite(g).all())
+    excess = ((g - w).abs() - (2.0 ** -7 * w.abs() + 2.0 ** -12 * w.abs().mean())).max().item()
+    assert excess <= 0, f"further apart than a bf16 step: by {excess:.3g}"
+
+
+@pytest.mark.parametrize("M,N,K", TAIL_CUT_SHAPES)
+@pytest.mark.parametrize("kind", ["block", "row"])
+@pytest.mark.parametrize("rows", ["5", "6"])
+def test_tail_cut_against_the_uncut_kernel(dev, tune, M, N, K, kind, rows):
+    if kind == "row" and K > 4096:
+        pytest.skip("one long-K case is enough")
+    cfg = BLK if kind == "block" else ROW
+    tune(MAXFP8_W4=rows, MAXFP8_W4_SPLIT="1")   # 1: wherever the shape has a cut, whatever the cost model says
+    cut_text = _lib.matmul_describe(M, N, K, kind == "block", True)
+    if "tail cut" not in cut_text:
+        pytest.skip(f"no cut at this tile height: {cut_text}")
+    assert "tail cut" not in _lib.matmul_describe(M, N, K, kind == "block", False)   # no workspace, no pieces
+    for exact in (True, False):
+        ops = _tail_cut_operands(M, N, K, kind, exact, dev)
+        run = lambda: mx.dynamic_scaled_matmul(*ops, cfg.input_scale, cfg.weight_scale, out_type=torch.bfloat16, algo="tiled")
+        tune(MAXFP8_W4=rows, MAXFP8_W4_SPLIT="1")
+        got, again = run(), run()
+        tune(MAXFP8_W4=rows, MAXFP8_W4_SPLIT="0")
+        assert "tail cut" not in _lib.matmul_describe(M, N, K, kind == "block", True)
+        want = run()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), again.view(torch.int16)), "two launches, two results"
+        if exact:
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        else:
+            _one_bf16_step_apart(got, want)
+
+
+def test_tail_cut_against_the_oracle(dev, tune):
+    tune(MAXFP8_W4="5", MAXFP8_W4_SPLIT="1")
+    for (M, N, K) in [(2040, 6144, 1024), (2200, 7168, 512)]:
+        if "tail cut" not in _lib.matmul_describe(M, N, K, True, True):
+            continue
+        a, b, sa, sb = make_block(M, N, K, seed=M)
+        ref = oracle_block(a, b, sa, sb)
+        c = mm(a, b, sa, sb, BLK, dev, out=torch.bfloat16, algo="tiled")
+        assert_rel(f32_np(c), ref, TOL, f"tail cut {M}x{N}x{K}")
+        return
+    pytest.skip("no shape of this list has a cut on this chip")
+
+
+def test_tail_cut_repeated_launches_with_fresh_data(dev, tune):
+    """The pieces go through memory that other CUs (and other XCDs, whose L2 caches are not coherent with each other)
+    wrote, behind flags that a launch raises and lowers again: thirty launches in a row, block-scaled and row-scaled
+    taking turns (they share the flags), each with new activations, each against the uncut kernel.  A block that read a stale piece, or found a flag still up, would show here."""
+    M, N, K = 2040, 6144, 2048
+    tune(MAXFP8_W4="5", MAXFP8_W4_SPLIT="1")
+    if "tail cut" not in _lib.matmul_describe(M, N, K, True, True):
+        pytest.skip("no cut at this shape on this chip")
+    L = _lib.lib()
+    assert L.maxfp8_matmul_workspace_bytes(M, N, K) >= 160 * 256 * 4 * 8
+    fixed = {kind: _tail_cut_operands(M, N, K, kind, False, dev) for kind in ("block", "row")}
+    for seed in range(30):
+        kind = "block" if seed % 2 == 0 else "row"
+        cfg = BLK if kind == "block" else ROW
+        _, b, sa, sb = fixed[kind]
+        a = synth.random_fp8((M, K), 100 + seed).to(dev)
+        run = lambda: mx.dynamic_scaled_matmul(a, b, sa, sb, cfg.input_scale, cfg.weight_scale, out_type=torch.bfloat16, algo="tiled")
+        tune(MAXFP8_W4="5", MAXFP8_W4_SPLIT="1")
+        got = run()
+        tune(MAXFP8_W4="5", MAXFP8_W4_SPLIT="0")
+        want = run()
+        torch.cuda.synchronize()
+        _one_bf16_step_apart(got, want)
+    assert L.maxfp8_tail_cut_given_up() == 0
+
+
+def test_tail_cut_recorded_into_a_graph(dev, tune):
+    # A recorded launch replays with the arguments of the recording -- the set of flags among them.  The flags are
+    # lowered by the launch that raised them, so a replay finds them as the recording did; recorded launches draw
+    # their sets from a range that eager launches never get.  Four replays, each on new activations, eager launches
+    # of the same shape in between, each replay against the eager result, bit for bit.
+    M, N, K = 2040, 6144, 2048
+    tune(MAXFP8_W4="5", MAXFP8_W4_SPLIT="1")
+    if "tail cut" not in _lib.matmul_describe(M, N, K, True, True):
+        pytest.skip("no cut at this shape on this chip")
+    ad, bd, sad, sbd = _tail_cut_operands(M, N, K, "block", False, dev)
+    L = _lib.lib()
+    need = L.maxfp8_matmul_workspace_bytes(M, N, K)
+    ws = torch.empty((need,), dtype=torch.uint8, device=dev)
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+
+    def run(dst, stream):
+        st = L.maxfp8_matmul_dynamic_scaled_fp8(dst.data_ptr(), ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), M, N, K,
+                                                K, K, N, _lib.GRAN_BLOCK, _lib.GRAN_BLOCK, 1, 128, 128, sad.shape[1], K // 128,
+                                                _lib.BF16, _lib.F32, _lib.ALGO_TILED, ws.data_ptr(), need, stream.cuda_stream)
+        assert st == 0, _lib.last_error()
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(out, side)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            run(out, side)
+    torch.cuda.current_stream().wait_stream(side)
+    eager = torch.empty_like(out)
+    for seed in range(4):
+        ad.copy_(synth.random_fp8((M, K), 100 + seed).to(dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        run(eager, torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), eager.view(torch.int16)), f"replay {seed}"
+    assert L.maxfp8_tail_cut_given_up() == 0
 
 
 # ---- the persistent kernel with its work split along K ("stream-K") --------------------------------------------
@@ -330,7 +474,7 @@ def test_stream_k_equals_per_tile_kernel(dev, tune, M, N, K, kind):
     run = lambda: mx.dynamic_scaled_matmul(ad, bd, sad, sbd, cfg.input_scale, cfg.weight_scale, out_type=torch.bfloat16,
                                            algo="tiled")
     got = run()
-    tune(MAXFP8_STREAMK="0")
+    tune(MAXFP8_STREAMK="0", MAXFP8_W4="0")   # (the eight-wave persistent kernel: the four-wave one may cut its last round, in another order of sums)
     assert "stream-K" not in _lib.matmul_describe(M, N, K, kind == "block", True)
     persistent = run()
     tune(MAXFP8_PERSIST="0")

@@ -47,7 +47,10 @@ def test_two_regions_cover_the_problem_once(tune):
 
 def test_four_wave_kernel_where_its_tile_count_fits_the_chip(tune):
     # DeepSeek-V3 o_proj at M = 4096: 448 tiles of 256 x 256 are 1.75 rounds of the 256 CUs, 728 tiles of 160 x 256 are 2.84
-    assert _lib.matmul_describe(4096, 7168, 16384) == "160x256 x728 persistent, four waves"
+    assert _lib.matmul_describe(4096, 7168, 16384, True, False) == "160x256 x728 persistent, four waves"
+    # with a workspace for the pieces: 616 tiles of 192 x 256 as two whole rounds and 104 tiles in two pieces each
+    assert _lib.matmul_describe(4096, 7168, 16384) == "192x256 x616 persistent, four waves, tail cut in pieces of 64 slabs"
+    assert _lib.lib().maxfp8_matmul_workspace_bytes(4096, 7168, 16384) >= 256 * 192 * 256 * 4
     # a ragged last column tile is fine as long as C's rows keep their 16-byte alignment (N a multiple of 8): the one matmul
     # over DeepSeek-V3's stacked q_a and kv_a weights, N = 1536 + 576
     assert _lib.matmul_describe(4096, 2112, 7168) == "160x256 x234 persistent, four waves"
@@ -57,5 +60,10 @@ def test_four_wave_kernel_where_its_tile_count_fits_the_chip(tune):
     assert "four waves" not in _lib.matmul_describe(128, 28672, 4096, False)
     tune(MAXFP8_W4="0")
     assert "four waves" not in _lib.matmul_describe(4096, 7168, 16384)
-    tune(MAXFP8_W4="6")
+    tune(MAXFP8_W4="6", MAXFP8_W4_SPLIT="0")
     assert _lib.matmul_describe(4096, 7168, 16384) == "192x256 x616 persistent, four waves"
+    # the cut wants a last round of at most half the CUs' number of tiles (216 of 160 x 256 are too many), slabs in fours
+    tune(MAXFP8_W4="5", MAXFP8_W4_SPLIT="1")
+    assert _lib.matmul_describe(4096, 7168, 16384) == "160x256 x728 persistent, four waves"
+    assert "tail cut in pieces of 8 slabs" in _lib.matmul_describe(2040, 6144, 4096)
+    assert "tail cut" not in _lib.matmul_describe(2040, 6144, 4096 + 256)

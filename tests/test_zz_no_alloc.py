@@ -42,17 +42,24 @@ def both_entry_points(M, N, K, block, dev, seed, out=torch.bfloat16):
 
 def test_noalloc_matmul_equals_the_plain_entry_point_twice_in_a_row(dev):
     L = _lib.lib()
-    assert L.maxfp8_matmul_noalloc_max_scratch_bytes() == 32 << 20
+    assert L.maxfp8_matmul_noalloc_max_scratch_bytes() == 48 << 20
     # first call: a K-split plan with ~8 MiB of partial sums; second call: a smaller one that reuses the same array
     # (whatever the first call left in it); then a row-scaled shape and one that needs no scratch at all
     for (M, N, K, block) in [(256, 576, 7168, True), (128, 512, 4096, True), (4096, 576, 7168, True), (100, 576, 7168, False), (2048, 1024, 512, True),
                               # 33 to 64 rows with a plan that does not split: both entry points run the tiles, not the
                               # weight-streaming kernel
-                              (64, 28672, 4096, True), (48, 8192, 4096, False)]:
+                              (64, 28672, 4096, True), (48, 8192, 4096, False),
+                              # a last round of tiles computed in pieces, their sums in the scratch: 48 MiB, all of the array
+                              # (too long for the CPU oracle here: held to the plain entry point's bits, and that one to
+                              # the uncut kernel by the tests of the tiles)
+                              (4096, 7168, 16384, True)]:
         print(f"[no-alloc] {M}x{N}x{K} {'block' if block else 'row'}: {_lib.matmul_describe(M, N, K, block, True)}", flush=True)
         c_plain, c_noalloc, (a, b, sa, sb), need = both_entry_points(M, N, K, block, dev, seed=M + N)
         assert bool(torch.isfinite(c_noalloc.float()).all())
         assert torch.equal(c_plain, c_noalloc), f"{M}x{N}x{K}: the two entry points differ"
+        if 2.0 * M * N * K > 2e11:
+            assert "tail cut" in _lib.matmul_describe(M, N, K, block, True) and need == 48 << 20
+            continue
         if block:
             ref = oracle.matmul_blockwise(fp8_bytes(a), fp8_bytes(b), sa.cpu().numpy(), sb.cpu().numpy(), threads=NT)
         else:
