@@ -85,6 +85,35 @@ def measured_traffic(name):
     return None
 
 
+def measured_ceiling(plan, kind):
+    """The issue ceiling of the dense kernel that `plan` launches (the library's own description of the launches), from
+    the committed run of `bench.py --mfma-ceiling` (profiles/mfma_issue_ceiling.txt): the rate of the kernel's main loop
+    on operands that never leave the chip -- the MFMA loop alone (row scaling) or with its promotions (block scaling),
+    fragments from LDS; and the whole loop with its copies, waits and barriers, operands in L2.  None where the
+    workload's kernel has no such probe (decode, grouped, the per-tile kernels) or the file is missing."""
+    first = plan.split(" + ")[0]
+    if "four waves" in first:
+        label = "four waves, %s x 256 tiles" % first.split("x")[0]
+    elif first.startswith("256x256") and "persistent" in first:
+        label = "eight waves, 256 x 256 tiles"
+    else:
+        return None
+    found = {}
+    try:
+        for line in open(os.path.join(ROOT, "profiles", "mfma_issue_ceiling.txt")):
+            parts = [x.strip() for x in line.split("|")]
+            if len(parts) >= 8 and parts[0] == "ceiling" and parts[1].startswith(label) and parts[2] == kind:
+                found["mfma_loop" if parts[3].startswith("MFMA loop") else "whole_loop"] = float(parts[5])
+    except OSError:
+        return None
+    if len(found) != 2:
+        return None
+    return {"kernel": label, "mfma_loop_lds_resident": found["mfma_loop"], "whole_loop_l2_resident": found["whole_loop"],
+            "unit": "TFLOP/s",
+            "source": "profiles/mfma_issue_ceiling.txt: bench.py --mfma-ceiling (maxfp8_mfma_issue_probe: the kernel's own "
+                      "main loop, one block per CU, operands that never leave the chip); committed figures, not values of this run"}
+
+
 def algorithmic(kind, M, K, N):
     """(flops, HBM bytes) of one step's matmul, and bytes of the quantisation."""
     flops = 2.0 * M * N * K
@@ -590,6 +619,11 @@ def result_line(name, steps, warmup, with_cpu=True):
     # large-tile launch and the rest): kernel_ms_* is the time of all of them
     roof["kernel"], roof["launches"] = kernels_launched(kind, M, K, N)
     roof["kernel_ms_avg"], roof["kernel_ms_median"], roof["kernel_ms_min"] = mm_avg, mm_med, mm_min
+    if roof["bound"] == "mfma" and kind in ("block", "row"):
+        ceiling = measured_ceiling(roof["launches"], kind)
+        if ceiling is not None:
+            ceiling["frac_of_whole_loop"] = roof["achieved"] / ceiling["whole_loop_l2_resident"]
+            roof["ceiling"] = ceiling
     out = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

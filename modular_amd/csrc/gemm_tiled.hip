@@ -1878,7 +1878,26 @@ static int pick_shape(int64_t M, int64_t N, int nslab, bool blockscale, bool can
 static bool streamk_shape(int64_t M, int64_t N, size_t workspace_bytes);
 static bool streamk_planned(int64_t M, int64_t N, int64_t K, bool blockscale);
 size_t gemm_tiled_plan_workspace_bytes(int64_t M, int64_t N, int64_t K, bool blockscale);
+static size_t workspace_bytes_uncached(int64_t M, int64_t N, int64_t K);
+// (callers ask before every matmul: the answers are kept, like the plans, keyed by the shape and the generation of the
+// tuning switches)
 size_t gemm_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  struct Entry { int64_t M, N, K; unsigned generation; bool valid; size_t bytes; };
+  static Entry table[128];
+  static std::mutex mu;
+  const unsigned generation = (unsigned)tuning().generation;
+  const uint64_t h = ((uint64_t)M * 0x9e3779b97f4a7c15ull) ^ ((uint64_t)N * 0xc2b2ae3d27d4eb4full) ^ ((uint64_t)K * 0x165667b19e3779f9ull);
+  Entry& e = table[(h >> 32) % 128];
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (e.valid && e.M == M && e.N == N && e.K == K && e.generation == generation) return e.bytes;
+  }
+  const size_t bytes = workspace_bytes_uncached(M, N, K);
+  std::lock_guard<std::mutex> lock(mu);
+  e = Entry{M, N, K, generation, true, bytes};
+  return bytes;
+}
+static size_t workspace_bytes_uncached(int64_t M, int64_t N, int64_t K) {
   // the largest split count any shape could choose for this problem
   size_t worst = 0;
   const int nslab = (int)ceil_div(K, 128);
@@ -2046,7 +2065,8 @@ static bool streamk_planned(int64_t M, int64_t N, int64_t K, bool blockscale) {
 // The split-K scratch of the plan an unlimited workspace gets (0: that plan does not split).  A workspace of this size --
 // or of gemm_tiled_workspace_bytes, which is never smaller -- leads to this same plan.
 size_t gemm_tiled_plan_workspace_bytes(int64_t M, int64_t N, int64_t K, bool blockscale) {
-  const TiledPlan plan = make_plan(M, N, K, blockscale, true, ~(size_t)0, 1, false);
+  // (from the table of plans: the entry points ask this on every call of a matmul of at most 64 rows)
+  const TiledPlan plan = cached_plan(M, N, K, blockscale, true, ~(size_t)0, 1, false);
   // (a plan that splits the work between blocks instead has splits == 1: without the 64 MB of slots it needs, the
   // planner falls back to the persistent kernel, which forms the same sums)
   if (plan.w4 && plan.w4_split) return gemm_w4_split(M, N, K, plan.w4).bytes;
@@ -2062,8 +2082,11 @@ static TiledPlan cached_plan(int64_t M, int64_t N, int64_t K, bool blockscale, b
   static Entry table[128];
   static std::mutex mu;
   const int flags = (blockscale ? 1 : 0) | (has_workspace ? 2 : 0) | (kv_on ? 4 : 0) | (int)(tuning().generation << 3);
+  // (every part of the key reaches the high bits that pick the slot: one shape is asked for with several workspace
+  // sizes and scale modes in turn, and those must not push each other out)
   const uint64_t h = ((uint64_t)M * 0x9e3779b97f4a7c15ull) ^ ((uint64_t)N * 0xc2b2ae3d27d4eb4full) ^ ((uint64_t)K * 0x165667b19e3779f9ull) ^
-                     ((uint64_t)batch << 7) ^ (uint64_t)flags;
+                     ((uint64_t)batch * 0xd6e8feb86659fd93ull) ^ ((uint64_t)flags * 0xa0761d6478bd642full) ^
+                     ((uint64_t)workspace_bytes * 0xe7037ed1a0b428dbull);
   Entry& e = table[(h >> 32) % 128];
   {
     std::lock_guard<std::mutex> lock(mu);
