@@ -272,13 +272,15 @@ int maxfp8_matmul_describe(int64_t M, int64_t N, int64_t K, int block_scaling, i
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
- * Diagnostic with no counterpart in the reference.  A matmul that computes its last round of tiles in pieces hands
- * the pieces' sums from block to block inside one launch; a block that waits for a piece does so for a bounded time
- * (seconds: only a GPU that stopped in the middle of a launch gets there), then fills its tile with NaN and counts
- * the event.  Returns that count for the current device since the library was loaded (0 in a healthy process), or
- * a negative maxfp8 error code.  Waits for the device's outstanding work.
+ * Diagnostic with no counterpart in the reference.  Two kernels hand f32 sums from block to block inside one launch
+ * (the four-wave kernel that computes its last round of tiles in pieces; the eight-wave kernel's work split along K,
+ * MAXFP8_STREAMK).  A block that waits for such a hand-over does so for a bounded time (seconds: a GPU that stopped in
+ * the middle of a launch gets there, and so would more such launches in flight at once on different streams than
+ * there are sets of flags: 32 and 64), then fills its tile with NaN and counts the event: the call that launched it
+ * has long returned MAXFP8_OK.  Returns that count for the current device since the library was loaded (0 in a
+ * healthy process), or a negative maxfp8 error code.  Waits for the device's outstanding work.
  */
-long long maxfp8_tail_cut_given_up(void);
+long long maxfp8_handovers_given_up(void);
 
 /*
  * Fused QKV projection with the K / V columns stored straight into a paged KV cache.
@@ -455,9 +457,12 @@ int maxfp8_moe_create_indices(
  * kernels: max/kernels/src/shmem/ep_comm.mojo:4409-4500, 4505-4624).
  * in [max_rows, 2 * inter]: out[m, k] = silu(in[m, k]) * in[m, inter + k] for the
  * rows m < row_offsets[num_offsets - 1] (read on the device; the other rows are not written).
- * quantize == 0: out has in_dtype.  quantize != 0: out is e4m3fn with one f32 scale per 128
+ * quantize == 0: out has in_dtype.  quantize == 1: out is e4m3fn with one f32 scale per 128
  * outputs, out_scales[k / 128, m] (row stride scales_ld), scale = max(amax, 1e-4) / 448 and
- * out = clamp(value / scale) -- this op's own recipe.  inter % 128 == 0 (quantize) or % 8.
+ * out = clamp(value / scale) -- this op's own recipe.  inter % 128 == 0.
+ * quantize == 2: like 0, with silu(in[m, k]) rounded to in_dtype before the product -- the arithmetic of
+ * the dense gated MLP, where silu and the multiplication are two operations on bf16 tensors
+ * (max/python/max/nn/linear.py:1072); out_scales is not used.
  */
 int maxfp8_fused_silu(
     void* out, void* out_scales, const void* in, const uint32_t* row_offsets,

@@ -49,7 +49,7 @@ EXPORTS = (
     "maxfp8_copy_bytes",
     "maxfp8_decode_weight_read_probe",
     "maxfp8_mfma_issue_probe",
-    "maxfp8_tail_cut_given_up",
+    "maxfp8_handovers_given_up",
 )
 
 _lib = None
@@ -125,8 +125,8 @@ def lib() -> ctypes.CDLL:
     L.maxfp8_copy_bytes.argtypes = [vp, vp, i64, vp]
     L.maxfp8_decode_weight_read_probe.restype = ci
     L.maxfp8_decode_weight_read_probe.argtypes = [vp, i64, i64, i64, i64, vp]
-    L.maxfp8_tail_cut_given_up.restype = ctypes.c_longlong
-    L.maxfp8_tail_cut_given_up.argtypes = []
+    L.maxfp8_handovers_given_up.restype = ctypes.c_longlong
+    L.maxfp8_handovers_given_up.argtypes = []
     L.maxfp8_mfma_issue_probe.restype = ci
     L.maxfp8_mfma_issue_probe.argtypes = [ci, ci, ci, i64, vp, vp, vp, vp, vp, vp, vp]
     _lib = L

@@ -37,7 +37,7 @@ int rmsnorm_quantize_dispatch(void*, void*, const void*, const void*, int64_t, i
 int quantize_static_dispatch(void*, const void*, int64_t, int64_t, int64_t, int64_t, int, float, hipStream_t);
 int quantize_tensor_dispatch(void*, void*, const void*, int64_t, int64_t, int64_t, int64_t, int, int, float, hipStream_t);
 int moe_create_indices_dispatch(uint32_t*, uint32_t*, uint32_t*, int32_t*, uint32_t*, const int32_t*, int64_t, int64_t, hipStream_t);
-int fused_silu_dispatch(void*, float*, const void*, const uint32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool,
+int fused_silu_dispatch(void*, float*, const void*, const uint32_t*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int,
                         hipStream_t);
 int cast_f32_to_e4m3fn_dispatch(void*, const float*, int64_t, hipStream_t);
 int cast_e4m3fn_to_f32_dispatch(float*, const void*, int64_t, hipStream_t);
@@ -63,6 +63,7 @@ int gemm_persist_probe(const GemmArgs&, bool, int, hipStream_t);
 int gemm_w4_probe(const GemmArgs&, bool, int, int, hipStream_t);
 bool gemm_w4_ok(const GemmArgs&, bool);
 int gemm_w4_gave_up(unsigned int*);
+int gemm_streamk_gave_up(unsigned int*);
 
 // v rounded to bf16 / f16 and widened back: how an op parameter of the input's dtype arrives
 static float round_to_dtype(float v, int dtype) {
@@ -340,13 +341,15 @@ int maxfp8_fused_silu(void* out, void* out_scales, const void* in, const uint32_
   if (max_rows == 0 || inter == 0) return MAXFP8_OK;
   if (inter % 128 != 0)
     MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused_silu: the output width %lld must be a multiple of 128", (long long)inter);
-  if (in_row_stride < 2 * inter || out_row_stride < inter || (quantize && scales_ld < max_rows))
+  if (quantize < 0 || quantize > 2) MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused_silu: quantize = %d is not 0, 1 or 2", quantize);
+  const bool quant = quantize == 1;
+  if (in_row_stride < 2 * inter || out_row_stride < inter || (quant && scales_ld < max_rows))
     MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "fused_silu: strides smaller than the extents");
-  if (!out || !in || !row_offsets || (quantize && !out_scales)) MAXFP8_FAIL(MAXFP8_ERR_NULL, "fused_silu: null pointer");
-  if (!is_aligned(in, 16) || in_row_stride % 8 != 0 || !is_aligned(out, 16) || out_row_stride % (quantize ? 8 : 8) != 0)
+  if (!out || !in || !row_offsets || (quant && !out_scales)) MAXFP8_FAIL(MAXFP8_ERR_NULL, "fused_silu: null pointer");
+  if (!is_aligned(in, 16) || in_row_stride % 8 != 0 || !is_aligned(out, 16) || out_row_stride % 8 != 0)
     MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "fused_silu: rows must be 16-byte aligned");
   return fused_silu_dispatch(out, (float*)out_scales, in, row_offsets, num_offsets, max_rows, inter, in_row_stride,
-                             out_row_stride, scales_ld, quantize != 0, (hipStream_t)stream);
+                             out_row_stride, scales_ld, quantize, (hipStream_t)stream);
 }
 
 size_t maxfp8_matmul_workspace_bytes(int64_t M, int64_t N, int64_t K) {
@@ -764,10 +767,11 @@ int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t
   return gemm_skinny_read_probe(b, M, N, K, ldb, (hipStream_t)stream);
 }
 
-long long maxfp8_tail_cut_given_up(void) {
-  unsigned int count = 0;
-  const int rc = gemm_w4_gave_up(&count);
-  return rc == MAXFP8_OK ? (long long)count : (long long)rc;
+long long maxfp8_handovers_given_up(void) {
+  unsigned int pieces = 0, shares = 0;
+  int rc = gemm_w4_gave_up(&pieces);
+  if (rc == MAXFP8_OK) rc = gemm_streamk_gave_up(&shares);
+  return rc == MAXFP8_OK ? (long long)pieces + (long long)shares : (long long)rc;
 }
 
 int maxfp8_mfma_issue_probe(int kernel, int blockscale, int level, int64_t slabs, const void* a, const void* b, const float* a_scales,

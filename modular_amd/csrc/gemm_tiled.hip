@@ -644,6 +644,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4) ? 2
 // up (its predecessor never ran: a hung GPU) poisons its tile with NaN instead of hanging too.
 constexpr int kStreamkSlots = 64, kStreamkMaxBlocks = 512;
 static __device__ unsigned int g_streamk_flags[kStreamkSlots * kStreamkMaxBlocks];
+static __device__ unsigned int g_streamk_gave_up;   // hand-overs a block stopped waiting for (their tiles hold NaN)
 
 // PROBE (measurement aid, results meaningless): 1 the same loop with every copy reading tile (0, 0) and slabs 0..7 over
 // and over, so that the operands stay in L2, one job of K / 128 slabs per block; 2 the same without copies, waits and
@@ -846,6 +847,7 @@ __device__ __forceinline__ void persist_body(const GemmArgs& p, uint8_t* smem) {
           __builtin_amdgcn_s_sleep(16);
         }
         asm volatile("" ::: "memory");
+        if (!there && tid == 0) atomicAdd(&g_streamk_gave_up, 1u);
         // (the slot's address is formed here, out of sight of the optimiser: hoisted out of the job loop, the 32
         // fragment offsets would sit in scalar registers for the whole kernel)
         uint32_t base = (uint32_t)l * PARTIAL_BYTES + (uint32_t)wave * (PARTIAL_BYTES / NWAVES);
@@ -1751,6 +1753,16 @@ static int launch_streamk(const GemmArgs& p_in, hipStream_t stream, const char* 
   p.streamk_seq = n;
   p.streamk_slot = (int)(n % kStreamkSlots);
   return launch_with_lds(gemm_streamk_kernel<256, 256, 2, 4, BLOCKSCALE>, attr_done, lds, 512, p, dim3((unsigned)streamk_blocks()), stream, name);
+}
+
+// Hand-overs of the work-split kernel that a block stopped waiting for, on the current device since the library was
+// loaded (0 unless a GPU stopped in the middle of a launch, or more launches of this kind were in flight at once than
+// there are sets of flags).  Waits for the device's work to finish.
+int gemm_streamk_gave_up(unsigned int* count) {
+  hipError_t e = hipDeviceSynchronize();
+  if (e == hipSuccess) e = hipMemcpyFromSymbol(count, HIP_SYMBOL(g_streamk_gave_up), sizeof(unsigned int));
+  if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "stream-K: cannot read the count of abandoned hand-overs: %s", hipGetErrorString(e));
+  return MAXFP8_OK;
 }
 
 // Sums the split-K partial results in split order (deterministic), applies the row / tensor

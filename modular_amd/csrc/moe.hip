@@ -225,18 +225,29 @@ __device__ __forceinline__ void exact_div8(const float (&a)[8], const float (&b)
 
 // gate / (1 + exp(-gate)) * up, every step rounded to f32 (ep_comm.mojo:4494-4497), for eight outputs.
 // (1 + exp(-gate) = inf, gate < -88: outside the fast division's range, and gate / inf = -0 is what the IEEE division gives)
+// ROUND_ACT: the activation is rounded to bf16 before the product, as where silu and the multiplication are two bf16
+// operations (the dense gated MLP, max/python/max/nn/linear.py:1072: ops.silu(gate) * up).
+template <bool ROUND_ACT>
 __device__ __forceinline__ void silu_mul8(const float (&gate)[8], const float (&up)[8], float (&f)[8]) {
   float d[8], sig[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) d[j] = 1.0f + expf(-gate[j]);
   exact_div8<false>(gate, d, sig);
+  if constexpr (ROUND_ACT) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t w = pack_bf16x2(sig[2 * j], sig[2 * j + 1]);
+      sig[2 * j] = __uint_as_float(w << 16);
+      sig[2 * j + 1] = __uint_as_float(w & 0xffff0000u);
+    }
+  }
 #pragma unroll
   for (int j = 0; j < 8; ++j) f[j] = sig[j] * up[j];
 }
 
 // 16 lanes own 128 consecutive outputs of one row (8 each): one 16-byte load of gate and of up
 // per lane; QUANT: amax over the 16 lanes by DPP, 8-byte packed fp8 store, lane 0 writes the scale.
-template <bool QUANT>
+template <bool QUANT, bool ROUND_ACT = false>
 __global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__ out, float* __restrict__ scales,
                                                               const uint16_t* __restrict__ in,
                                                               const uint32_t* __restrict__ row_offsets, int num_offsets,
@@ -264,7 +275,7 @@ __global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__
       up[2 * j] = __uint_as_float(uw[j] << 16);
       up[2 * j + 1] = __uint_as_float(uw[j] & 0xffff0000u);
     }
-    silu_mul8(gate, up, f);
+    silu_mul8<ROUND_ACT>(gate, up, f);
     if constexpr (!QUANT) {
       uint32_t w[4];
 #pragma unroll
@@ -296,13 +307,17 @@ __global__ __launch_bounds__(256) void fused_silu_bf16_kernel(void* __restrict__
 
 int fused_silu_dispatch(void* out, float* scales, const void* in, const uint32_t* row_offsets, int64_t num_offsets,
                         int64_t max_rows, int64_t inter, int64_t in_stride, int64_t out_stride, int64_t scales_ld,
-                        bool quant, hipStream_t stream) {
+                        int mode, hipStream_t stream) {
+  const bool quant = mode == 1;
   // the number of rows in use is only known on the device: the grid is sized for max_rows and
   // walks the items in strides
   const int64_t items = max_rows * (inter / 128);
   const unsigned blocks = (unsigned)(ceil_div(items, 16) < 8192 ? ceil_div(items, 16) : 8192);
   if (quant)
     hipLaunchKernelGGL(fused_silu_bf16_kernel<true>, dim3(blocks), dim3(256), 0, stream, out, scales, (const uint16_t*)in,
+                       row_offsets, (int)num_offsets, max_rows, (int)inter, in_stride, out_stride, scales_ld);
+  else if (mode == 2)
+    hipLaunchKernelGGL((fused_silu_bf16_kernel<false, true>), dim3(blocks), dim3(256), 0, stream, out, scales, (const uint16_t*)in,
                        row_offsets, (int)num_offsets, max_rows, (int)inter, in_stride, out_stride, scales_ld);
   else
     hipLaunchKernelGGL(fused_silu_bf16_kernel<false>, dim3(blocks), dim3(256), 0, stream, out, scales, (const uint16_t*)in,

@@ -81,8 +81,9 @@ class MLP(torch.nn.Module):
     weights when the quantisation allows it (`QuantConfig.can_use_fused_mlp`, linear.py:1029-1035);
     here the two weights ARE one buffer (`gate_up_weight`, with `gate_proj.weight` / `up_proj.weight`
     views of its halves), so nothing is concatenated per call.  With SiLU and no bias the activation
-    and the product with `up` are one kernel (`fused_silu`) whose bf16 result `down_proj` quantises
-    like any other input: the reference's arithmetic, five launches for the whole block.
+    and the product with `up` are one kernel (`fused_silu` with the activation rounded to bf16 before
+    the product, as the reference's two bf16 operations `ops.silu(gate) * up` round it, linear.py:1072)
+    whose bf16 result `down_proj` quantises like any other input: five launches for the whole block.
 
     `fuse_activation_quant=True` (dynamic block scaling only) also folds the quantisation for
     `down_proj` into that kernel (`fused_silu_quantized`: four launches, no bf16 intermediate).
@@ -188,7 +189,7 @@ class MLP(torch.nn.Module):
             return y.reshape(*lead, self.hidden_dim)
         if self._silu_kernel():
             both = quantized_matmul(x2, self.gate_up_weight, self.gate_up_weight_scale, None, cfg)
-            hidden = fused_silu(both, self._all_rows(x2.shape[0], x2.device))
+            hidden = fused_silu(both, self._all_rows(x2.shape[0], x2.device), round_activation=True)
             return self.down_proj(hidden).reshape(*lead, self.hidden_dim)
         act = self._ACTIVATIONS[self.activation_function]
         if self._one_matmul and self.gate_proj.bias is None:

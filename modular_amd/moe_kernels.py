@@ -46,15 +46,20 @@ def _check_silu_input(input: torch.Tensor, row_offsets: torch.Tensor) -> None:
     _require_gpu(input, row_offsets)
 
 
-def fused_silu(input: torch.Tensor, row_offsets: torch.Tensor) -> torch.Tensor:
-    """silu(input[:, :I]) * input[:, I:] for the rows below row_offsets[-1]; [max_rows, I]."""
+def fused_silu(input: torch.Tensor, row_offsets: torch.Tensor, *, round_activation: bool = False) -> torch.Tensor:
+    """silu(input[:, :I]) * input[:, I:] for the rows below row_offsets[-1]; [max_rows, I].
+
+    round_activation=True (not a parameter of the reference's kernel): silu's result is rounded to the input's dtype
+    before the product, which is what the reference's dense MLP computes with its two separate bf16 operations
+    (ops.silu(gate) * up, max/python/max/nn/linear.py:1072); the MoE kernel rounds once, after the product."""
     _check_silu_input(input, row_offsets)
     input = input.contiguous()
     rows, two_i = input.shape
     inter = two_i // 2
     out = torch.empty((rows, inter), dtype=input.dtype, device=input.device)
     st = _lib.lib().maxfp8_fused_silu(out.data_ptr(), None, input.data_ptr(), row_offsets.data_ptr(), row_offsets.shape[0],
-                                      rows, inter, two_i, inter, 0, _DT[input.dtype], 0, _stream(input))
+                                      rows, inter, two_i, inter, 0, _DT[input.dtype], 2 if round_activation else 0,
+                                      _stream(input))
     _lib.check(st)
     return out
 

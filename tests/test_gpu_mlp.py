@@ -82,30 +82,39 @@ def test_block_scaled_mlp_stage_by_stage(dev, M, hidden, ffl):
 @pytest.mark.parametrize("M,hidden,ffl", [(48, 512, 1024), (257, 1024, 3584)])
 def test_block_scaled_mlp_default_route_quantises_like_a_linear(dev, M, hidden, ffl):
     """Without the opt-in the activations that reach the second matmul are what the reference's block hands it:
-    silu(gate) * up rounded to bf16, quantised by down_proj's own rule (upper bound 1200, multiplication by the
-    guarded reciprocal).  The fp8 bytes and scales are those of the oracle's quantiser on that bf16 tensor."""
+    silu(gate) rounded to bf16, times up, rounded to bf16 (two bf16 operations, linear.py:1072), quantised by
+    down_proj's own rule (upper bound 1200, multiplication by the guarded reciprocal).  The fp8 bytes and scales are
+    those of the oracle's quantiser on that bf16 tensor."""
     mlp, parts = make_block_mlp(hidden, ffl, dev)
     assert not mlp._fused() and mlp._silu_kernel()
     x = synth.activations(M, hidden, seed=8).to(dev)
     y = mlp(x)
     both = mx.quantized_matmul(x, mlp.gate_up_weight, mlp.gate_up_weight_scale, None, BLK)
     rows = torch.tensor([0, M], dtype=torch.int64).to(torch.uint32).to(dev)
-    hidden_act = mx.fused_silu(both, rows)
+    hidden_act = mx.fused_silu(both, rows, round_activation=True)
     assert torch.equal(y, mlp.down_proj(hidden_act)), "the block is its stages"
-    # the stage in front of the second quantiser against the oracle: equal but for the last bit of exp
-    want_h = oracle.fused_silu(bf16_bits(both), M, quantize=False, threads=NT)
-    assert (bf16_bits(hidden_act) != want_h).mean() <= 5e-3
+    # the stage in front of the second quantiser against float64 arithmetic with the two roundings: equal but for
+    # activations within the last bit of exp of a bf16 rounding boundary, and those one bf16 step apart
+    g64, u64 = both[:, :ffl].double().cpu(), both[:, ffl:].double().cpu()
+    act = (g64 / (1.0 + torch.exp(-g64))).to(torch.float32).to(torch.bfloat16)
+    want_h = (act.double() * u64).to(torch.float32).to(torch.bfloat16)
+    got_bits, want_bits = bf16_bits(hidden_act).astype(np.int32), bf16_bits(want_h).astype(np.int32)
+    assert (got_bits != want_bits).mean() <= 5e-3 and np.abs(got_bits - want_bits).max() <= 1
+    # (the MoE kernel's single rounding is another tensor: the flag is not a no-op)
+    once = mx.fused_silu(both, rows)
+    assert np.array_equal(bf16_bits(once), oracle.fused_silu(bf16_bits(both), M, quantize=False, threads=NT)) or \
+        (bf16_bits(once) != oracle.fused_silu(bf16_bits(both), M, quantize=False, threads=NT)).mean() <= 5e-3
+    assert not torch.equal(once, hidden_act)
     # what down_proj quantises: bit-exact with the oracle's quantize_dynamic_scaled_fp8 on the same bf16 input
     hq, hs = mx.quantize_dynamic_scaled_float8(hidden_act, BLK.input_scale, BLK.weight_scale, scales_type=torch.float32)
     want_q, want_s = oracle.quantize_dynamic_scaled_fp8(bf16_bits(hidden_act), 128, threads=NT)
     assert np.array_equal(fp8_bytes(hq), want_q) and np.array_equal(f32_np(hs)[:, :M], want_s)
-    # ... and the three-Linear route with torch's bf16 silu and product between them: the same block up to one
-    # rounding of silu(gate) * up instead of two, which moves about one fp8 code in a hundred by a step in front of
-    # the second matmul -- fp8 quantisation noise, a per cent of the result's norm
+    # ... and the three-Linear route with torch's bf16 silu and product between them: the same roundings, so the same
+    # block element by element (where torch's exp and the kernel's differ in their last bit, a rare activation lands
+    # on the other side of a bf16 boundary and moves an fp8 code in front of the second matmul)
     want = mlp.down_proj(torch.nn.functional.silu(mlp.gate_proj(x)) * mlp.up_proj(x))
     torch.cuda.synchronize()
-    diff = (y.double() - want.double()).norm() / want.double().norm()
-    assert float(diff) < 0.03, f"default route against the three linears: relative difference {float(diff):.3f}"
+    assert_rel(f32_np(y), f32_np(want), 2e-2, "default route against the three linears")
     # calling twice reuses the [0, rows] operand: no host tensor is built per call
     assert len(mlp._row_offsets) == 1 and mlp(x) is not None and len(mlp._row_offsets) == 1
 
@@ -145,9 +154,8 @@ def test_per_token_mlp_runs_gate_and_up_as_one_matmul(dev):
     y = mlp(x)
     want = mlp.down_proj(torch.nn.functional.silu(mlp.gate_proj(x)) * mlp.up_proj(x))
     torch.cuda.synchronize()
-    # (one rounding of silu(gate) * up instead of torch's two: a few fp8 codes differ in front of down_proj)
-    diff = (y.double() - want.double()).norm() / want.double().norm()
-    assert float(diff) < 0.03, f"per-token MLP against its three linears: relative difference {float(diff):.3f}"
+    # (the same two roundings as torch's silu and product: element by element)
+    assert_rel(f32_np(y), f32_np(want), 2e-2, "per-token MLP against its three linears")
 
 
 def test_mlp_argument_checks(dev):

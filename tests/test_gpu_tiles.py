@@ -403,7 +403,7 @@ def test_tail_cut_repeated_launches_with_fresh_data(dev, tune):
         want = run()
         torch.cuda.synchronize()
         _one_bf16_step_apart(got, want)
-    assert L.maxfp8_tail_cut_given_up() == 0
+    assert L.maxfp8_handovers_given_up() == 0
 
 
 def test_tail_cut_recorded_into_a_graph(dev, tune):
@@ -445,7 +445,7 @@ def test_tail_cut_recorded_into_a_graph(dev, tune):
         run(eager, torch.cuda.current_stream())
         torch.cuda.synchronize()
         assert torch.equal(got.view(torch.int16), eager.view(torch.int16)), f"replay {seed}"
-    assert L.maxfp8_tail_cut_given_up() == 0
+    assert L.maxfp8_handovers_given_up() == 0
 
 
 # ---- the persistent kernel with its work split along K ("stream-K") --------------------------------------------
@@ -576,3 +576,4 @@ def test_stream_k_repeated_launches_with_fresh_data(dev, tune):
         want = mx.dynamic_scaled_matmul(a, b, sa, sb, BLK.input_scale, BLK.weight_scale, out_type=torch.bfloat16, algo="tiled")
         torch.cuda.synchronize()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"launch {seed}"
+    assert L.maxfp8_handovers_given_up() == 0   # (no block ever stopped waiting for its predecessor)
