@@ -384,6 +384,7 @@ def read_ceiling(wl, steps):
 
 
 MFMA_CEILING_KERNELS = {0: ("eight waves, 256 x 256 tiles (gemm_persist_kernel)", 256),
+                        4: ("four waves, 128 x 256 tiles (gemm_w4_kernel)", 128),
                         5: ("four waves, 160 x 256 tiles (gemm_w4_kernel)", 160),
                         6: ("four waves, 192 x 256 tiles (gemm_w4_kernel)", 192)}
 

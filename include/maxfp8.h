@@ -500,7 +500,7 @@ int maxfp8_decode_weight_read_probe(const void* b, int64_t M, int64_t N, int64_t
 
 /*
  * Measurement aid with no counterpart in the reference: the main loop of a dense block- or row-scaled matmul kernel
- * (kernel 0: eight waves, 256 x 256 tiles; kernel 5 / 6: four waves, 160 x 256 / 192 x 256 tiles) run for `slabs` K slabs of 128 bytes
+ * (kernel 0: eight waves, 256 x 256 tiles; kernel 4 / 5 / 6: four waves, 128 x 256 / 160 x 256 / 192 x 256 tiles) run for `slabs` K slabs of 128 bytes
  * by one block on every compute unit, all blocks on the same tile:
  *   level 2: the MFMA loop alone (block scaling: with its promotions), fragments read from what one copy left in LDS;
  *   level 1: the whole loop -- LDS-DMA copies, waits, barriers -- with operands that stay in L2 (slabs 0..7 of tile

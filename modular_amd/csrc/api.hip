@@ -138,7 +138,7 @@ static const Tuning* read_tuning(unsigned generation) {
   t->grouped_overlap = num("MAXFP8_GROUPED_OVERLAP", 1) != 0;
   t->grouped_persist = num("MAXFP8_GROUPED_PERSIST", 1) != 0;
   const int w4 = num("MAXFP8_W4", -1);
-  t->w4 = (w4 == 0 || w4 == 5 || w4 == 6) ? w4 : -1;
+  t->w4 = (w4 == 0 || w4 == 4 || w4 == 5 || w4 == 6) ? w4 : -1;
   const int w4_split = num("MAXFP8_W4_SPLIT", -1);
   t->w4_split = (w4_split == 0 || w4_split == 1) ? w4_split : -1;
   t->skinny_alds = num("MAXFP8_SKINNY_ALDS", 1) != 0;
@@ -778,8 +778,8 @@ int maxfp8_mfma_issue_probe(int kernel, int blockscale, int level, int64_t slabs
                             const float* b_scales, void* c, uint64_t* clocks, void* stream) {
   if (!a || !b || !c || !a_scales || !b_scales) MAXFP8_FAIL(MAXFP8_ERR_NULL, "issue probe: null pointer");
   if (clocks && !is_aligned(clocks, 8)) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "issue probe: clocks must be 8-byte aligned");
-  if ((kernel != 0 && kernel != 5 && kernel != 6) || (level != 1 && level != 2) || slabs < 8 || slabs > (1 << 22) || slabs % 2 != 0)
-    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "issue probe: kernel 0 / 5 / 6, level 1 / 2, an even number of slabs in [8, 2^22]");
+  if ((kernel != 0 && kernel != 4 && kernel != 5 && kernel != 6) || (level != 1 && level != 2) || slabs < 8 || slabs > (1 << 22) || slabs % 2 != 0)
+    MAXFP8_FAIL(MAXFP8_ERR_SHAPE, "issue probe: kernel 0 / 4 / 5 / 6, level 1 / 2, an even number of slabs in [8, 2^22]");
   if (!is_aligned(a, 16) || !is_aligned(b, 16) || !is_aligned(c, 16)) MAXFP8_FAIL(MAXFP8_ERR_ALIGN, "issue probe: 16-byte aligned buffers");
   GemmArgs p;
   memset(&p, 0, sizeof(p));

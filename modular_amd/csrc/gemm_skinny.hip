@@ -347,7 +347,8 @@ static int launch_skinny_r(const GemmArgs& p, int64_t batch, hipStream_t stream)
   auto kern = gemm_skinny_kernel<NTW, MT, BLOCKSCALE, RING_KB, NWAVES, ALDS>;
   static PerDeviceFlag attr;
   bool& attr_done = attr.here();
-  constexpr int smem_max = Cfg::SMEM + (ALDS ? NWAVES * kSkinnyALdsBytes : 0);
+  constexpr int smem_all = Cfg::SMEM + (ALDS ? NWAVES * kSkinnyALdsBytes : 0);
+  constexpr int smem_max = smem_all < 160 * 1024 ? smem_all : 160 * 1024;  // (what a launch asks for was checked against the CU's LDS)
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem_max);
     if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "gemm_skinny: cannot reserve %d bytes of LDS: %s", smem_max, hipGetErrorString(e));

@@ -1978,11 +1978,11 @@ static float persistent_cost(int64_t tiles, int slots, float t) {
   return (float)full * t + (rest ? t * (0.75f + 0.3f * (float)rest / (float)slots) : 0.f);
 }
 
-// Per-slab and per-tile times (microseconds, chip full, operands from HBM) of the four-wave kernel's two tile heights:
-// index 0: 160 x 256, 1: 192 x 256.  Against the eight-wave persistent kernel's 1.63 / 1.40 per slab of a 256 x 256 tile
+// Per-slab and per-tile times (microseconds, chip full, operands from HBM) of the four-wave kernel's three tile heights:
+// index 0: 128 x 256, 1: 160 x 256, 2: 192 x 256.  Against the eight-wave persistent kernel's 1.63 / 1.40 per slab of a 256 x 256 tile
 // that is 6 ... 9 % less per flop with block scaling and level with row scaling; what decides between the three is
 // mostly how the tile count divides by the CUs.
-static const float kW4SlabBlock[2] = {1.00f, 1.14f}, kW4SlabRow[2] = {0.88f, 1.00f}, kW4Tile = 5.5f;
+static const float kW4SlabBlock[3] = {0.90f, 1.00f, 1.14f}, kW4SlabRow[3] = {0.93f, 0.88f, 1.00f}, kW4Tile = 5.5f;
 // With the tail cut: whole rounds, then a piece per block and the hand-over: a piece's sums written through to memory,
 // then read and added by the tile's last block, piece after piece (measured on 4096 x 7168 x 16384, 104 tiles in two
 // pieces each behind two whole rounds, and on 2048 x 7168 x 18432, 52 tiles in four pieces behind one).
@@ -2000,8 +2000,8 @@ static int pick_w4(int64_t M, int64_t N, int64_t K, bool blockscale, float other
   const int nslab = (int)(K / 128), slots = compute_units();
   int best = 0;
   float best_cost = forced > 0 ? 3.0e38f : 0.97f * other_cost;  // (a forced height is taken whatever it costs)
-  for (int i = 0; i < 2; ++i) {
-    const int tm = 5 + i;
+  for (int i = 0; i < 3; ++i) {
+    const int tm = 4 + i;
     if (forced > 0 && tm != forced) continue;
     const float t_slab = blockscale ? kW4SlabBlock[i] : kW4SlabRow[i], t = (float)nslab * t_slab + kW4Tile;
     const int64_t tiles = ceil_div(M, 32 * tm) * ceil_div(N, 256);

@@ -676,7 +676,7 @@ W4Split gemm_w4_split(int64_t M, int64_t N, int64_t K, int tm) {
   return W4Split{g, (int)u, (size_t)g * 32 * tm * 256 * 4};
 }
 
-// rows of a tile: 32 * tm (tm = 5 or 6 sixteen-row groups per wave); split: cut the tail (p.workspace holds what
+// rows of a tile: 32 * tm (tm = 4, 5 or 6 sixteen-row groups per wave); split: cut the tail (p.workspace holds what
 // gemm_w4_split asks for)
 int gemm_w4_launch(const GemmArgs& p_in, bool blockscale, int tm, bool split, hipStream_t stream) {
   GemmArgs p = p_in;
@@ -701,6 +701,8 @@ int gemm_w4_launch(const GemmArgs& p_in, bool blockscale, int tm, bool split, hi
                                                             : kW4FlagSets / 2 + (int)(recorded.fetch_add(1, std::memory_order_relaxed) % (kW4FlagSets / 2));
     }
   }
+  if (tm == 4)
+    return blockscale ? launch_w4<4, true, 0>(p, blocks, stream, "gemm_w4_block_128x256") : launch_w4<4, false, 0>(p, blocks, stream, "gemm_w4_row_128x256");
   if (tm == 5)
     return blockscale ? launch_w4<5, true, 0>(p, blocks, stream, "gemm_w4_block_160x256") : launch_w4<5, false, 0>(p, blocks, stream, "gemm_w4_row_160x256");
   return blockscale ? launch_w4<6, true, 0>(p, blocks, stream, "gemm_w4_block_192x256") : launch_w4<6, false, 0>(p, blocks, stream, "gemm_w4_row_192x256");
@@ -719,6 +721,10 @@ int gemm_w4_gave_up(unsigned int* count) {
 int gemm_w4_probe(const GemmArgs& p, bool blockscale, int level, int tm, hipStream_t stream) {
   const unsigned blocks = (unsigned)compute_units();
   const char* name = "gemm_w4_probe";
+  if (tm == 4) {
+    if (level == 1) return blockscale ? launch_w4<4, true, 1>(p, blocks, stream, name) : launch_w4<4, false, 1>(p, blocks, stream, name);
+    return blockscale ? launch_w4<4, true, 2>(p, blocks, stream, name) : launch_w4<4, false, 2>(p, blocks, stream, name);
+  }
   if (tm == 5) {
     if (level == 1) return blockscale ? launch_w4<5, true, 1>(p, blocks, stream, name) : launch_w4<5, false, 1>(p, blocks, stream, name);
     return blockscale ? launch_w4<5, true, 2>(p, blocks, stream, name) : launch_w4<5, false, 2>(p, blocks, stream, name);

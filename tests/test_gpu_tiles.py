@@ -201,10 +201,10 @@ def test_two_region_launch(dev, tune, M, K, N, kind):
 PERSIST_SHAPES = [(512, 512, 256), (4096, 8192, 256), (2560, 7680, 384), (8192, 8192, 128), (1024, 4096, 144), (256, 256, 1024)]
 
 
-# The four-wave kernel (MAXFP8_W4=5 / 6: 160 x 256 / 192 x 256 tiles, one wave per SIMD; it takes the shapes whose K is an
+# The four-wave kernel (MAXFP8_W4=4 / 5 / 6: 128 x 256 / 160 x 256 / 192 x 256 tiles, one wave per SIMD; it takes the shapes whose K is an
 # even number of slabs and leaves the others to the eight-wave kernel) makes the same sums in the same order and is held
 # to the same bits.
-FORMS = {"eight waves": "0", "four waves, 160 rows": "5", "four waves, 192 rows": "6"}
+FORMS = {"eight waves": "0", "four waves, 128 rows": "4", "four waves, 160 rows": "5", "four waves, 192 rows": "6"}
 
 
 @pytest.mark.parametrize("M,N,K", PERSIST_SHAPES)
@@ -243,7 +243,7 @@ def test_persistent_kernel_exact(dev, tune, M, N, K, form):
 
 @pytest.mark.parametrize("M,N,K", [(4096, 2112, 7168), (320, 264, 512), (1000, 8, 1024), (161, 1544, 768)])
 @pytest.mark.parametrize("kind", ["block", "row"])
-@pytest.mark.parametrize("rows", ["5", "6"])
+@pytest.mark.parametrize("rows", ["4", "5", "6"])
 def test_four_wave_kernel_ragged_edges(dev, tune, M, N, K, kind, rows):
     # a last row tile past M and a last column tile past N (DeepSeek-V3's fused q_a + kv_a projection: N = 1536 + 576 = 2112 =
     # 8 tiles and a quarter): bit-equal to the per-tile kernel, and nothing written outside the result.  Through the C ABI,
@@ -341,7 +341,7 @@ def _one_bf16_step_apart(got, want):
 
 @pytest.mark.parametrize("M,N,K", TAIL_CUT_SHAPES)
 @pytest.mark.parametrize("kind", ["block", "row"])
-@pytest.mark.parametrize("rows", ["5", "6"])
+@pytest.mark.parametrize("rows", ["4", "5", "6"])
 def test_tail_cut_against_the_uncut_kernel(dev, tune, M, N, K, kind, rows):
     if kind == "row" and K > 4096:
         pytest.skip("one long-K case is enough")
