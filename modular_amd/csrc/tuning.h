@@ -7,7 +7,8 @@
 //   MAXFP8_SPLITK=n            force the K split of the tiled matmul
 //   MAXFP8_ONE_REGION=1        never cut a matmul into two regions
 //   MAXFP8_PERSIST=0           per-tile kernels instead of the persistent one
-//   MAXFP8_W4=0 / 5 / 6        whole-tile matmuls: the four-wave kernel never / in 160 x 256 / in 192 x 256 tiles
+//   MAXFP8_W4=0 / 4 / 5 / 6    whole-tile matmuls: the four-wave kernel never / in 128 x 256 / 160 x 256 / 192 x 256 tiles
+//   MAXFP8_W4_SPLIT=0 / 1      its last round of tiles cut into pieces along K: never / wherever a shape has a cut
 //                              (default: where the cost model says it pays)
 //   MAXFP8_STREAMK=0 / 2       never / always split the work of whole-tile matmuls evenly over the blocks
 //                              (default 1: where the cost model says it pays)
