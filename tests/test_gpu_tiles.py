@@ -406,6 +406,42 @@ def test_tail_cut_repeated_launches_with_fresh_data(dev, tune):
     assert L.maxfp8_handovers_given_up() == 0
 
 
+def test_tail_cut_on_two_streams_at_once(dev, tune):
+    """Launches that overlap in time each bring a workspace of their own and draw a set of flags of their own: two
+    streams issue the same matmul on different activations, back to back, sixteen times each without waiting for one
+    another; every result equals what the same launch gives alone."""
+    M, N, K = 2040, 6144, 2048
+    tune(MAXFP8_W4="5", MAXFP8_W4_SPLIT="1")
+    if "tail cut" not in _lib.matmul_describe(M, N, K, True, True):
+        pytest.skip("no cut at this shape on this chip")
+    L = _lib.lib()
+    need = L.maxfp8_matmul_workspace_bytes(M, N, K)
+    _, bd, sad, sbd = _tail_cut_operands(M, N, K, "block", False, dev)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    acts = [[synth.random_fp8((M, K), 300 + 16 * s_ + i).to(dev) for i in range(16)] for s_ in range(2)]
+    outs = [[torch.empty((M, N), dtype=torch.bfloat16, device=dev) for _ in range(16)] for _ in range(2)]
+    spaces = [torch.empty((need,), dtype=torch.uint8, device=dev) for _ in range(2)]
+
+    def launch(a, out, ws, stream):
+        st = L.maxfp8_matmul_dynamic_scaled_fp8(out.data_ptr(), a.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), M, N, K,
+                                                K, K, N, _lib.GRAN_BLOCK, _lib.GRAN_BLOCK, 1, 128, 128, sad.shape[1], K // 128,
+                                                _lib.BF16, _lib.F32, _lib.ALGO_TILED, ws.data_ptr(), need, stream.cuda_stream)
+        assert st == 0, _lib.last_error()
+
+    torch.cuda.synchronize()
+    for i in range(16):
+        for s_ in range(2):
+            launch(acts[s_][i], outs[s_][i], spaces[s_], streams[s_])
+    torch.cuda.synchronize()
+    alone = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    for s_ in range(2):
+        for i in range(16):
+            launch(acts[s_][i], alone, spaces[0], torch.cuda.current_stream())
+            torch.cuda.synchronize()
+            assert torch.equal(outs[s_][i].view(torch.int16), alone.view(torch.int16)), f"stream {s_}, launch {i}"
+    assert L.maxfp8_handovers_given_up() == 0
+
+
 def test_tail_cut_recorded_into_a_graph(dev, tune):
     # A recorded launch replays with the arguments of the recording -- the set of flags among them.  The flags are
     # lowered by the launch that raised them, so a replay finds them as the recording did; recorded launches draw
