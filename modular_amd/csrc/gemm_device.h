@@ -44,8 +44,8 @@ __device__ __forceinline__ void buffer_store_b128_guarded(const v4u_t v, const _
 }
 
 // tile number -> (row tile, column tile): groups of GROUP_M row tiles share weight columns, walked column-major
+template <int GROUP_M = 4>
 __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  constexpr int GROUP_M = 4;
   const int per_group = GROUP_M * tiles_n;
   const int group = pid / per_group;
   const int first_m = group * GROUP_M;

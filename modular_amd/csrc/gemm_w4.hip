@@ -109,6 +109,11 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // a product is folded in LAG MFMAs after its own (2: 4 ... 6 % slower, the FMAs then wait for the matrix pipe; 4: the same)
   constexpr int LAG = 3;
   static_assert(TN == 8 && TM >= 3 && TM <= 8, "wave tile");
+  // Row tiles that share weight columns in the tile order: the 32 blocks of an XCD work on a patch of kGroupM row tiles
+  // x 32 / kGroupM column tiles at a time, and what the XCD's L2 fetches for it is the patch's rows of both operands --
+  // least for a square patch: 8 x 4 for 128-row tiles (q_b M = 1024: 47 -> 43 us against 4 x 8; o_proj M = 1024: 112 ->
+  // 109), 4 x 8 for the taller ones (2 x 16 and 8 x 4 measured slower there).
+  constexpr int kGroupM = TM == 4 ? 8 : 4;
   static_assert(PER_B + NSTORE < 64, "the count must fit the vmcnt field");
   static_assert(IB % 2 == 0, "the weight copies go out in two halves");
 
@@ -270,7 +275,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
 
   // ---- prologue: slabs 0 and 1 of the first tile
   int tm, tn;
-  tile_coords(job.tile, tiles_m, tiles_n, tm, tn);
+  tile_coords<kGroupM>(job.tile, tiles_m, tiles_n, tm, tn);
   if constexpr (PROBE != 0) tm = tn = 0;
   TileAt cur_at = tile_at(tm, tn);
   {
@@ -344,7 +349,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     const bool has_next = k + 1 < njobs;
     const Job next_job = has_next ? job_of(k + 1, nullptr) : job;
     int tm2 = tm, tn2 = tn;
-    if (has_next) tile_coords(next_job.tile, tiles_m, tiles_n, tm2, tn2);
+    if (has_next) tile_coords<kGroupM>(next_job.tile, tiles_m, tiles_n, tm2, tn2);
     const TileAt next_at = tile_at(tm2, tn2);
     // the first slab of the next job (of nothing behind the block's last one: offsets past 2^31 read as zeros)
     const SlabAt next0 = slab_at(next_at, next_job.s0, has_next ? 0u : 0x80000000u);
