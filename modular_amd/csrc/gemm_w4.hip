@@ -113,7 +113,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // x 32 / kGroupM column tiles at a time, and what the XCD's L2 fetches for it is the patch's rows of both operands --
   // least for a square patch: 8 x 4 for 128-row tiles (q_b M = 1024: 47 -> 43 us against 4 x 8; o_proj M = 1024: 112 ->
   // 109), 4 x 8 for the taller ones (3, 6 and 8 row tiles measured within a per cent of 4 on the long-K shapes, 8 a seventh
-  slower on kv_b M = 4096).
+  // slower on kv_b M = 4096).
   constexpr int kGroupM = TM == 4 ? 8 : 4;
   static_assert(PER_B + NSTORE < 64, "the count must fit the vmcnt field");
   static_assert(IB % 2 == 0, "the weight copies go out in two halves");
