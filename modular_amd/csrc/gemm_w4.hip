@@ -38,10 +38,10 @@
 //
 // The last round.  Tiles are dealt out in whole rounds of the blocks; what is left for a last round is often a fraction
 // of a round, and its tiles take as long as any.  Where the caller brings a workspace, the tiles beyond the last whole
-// round are cut along K into two to four pieces, a block per piece (see the job list in w4_body): the pieces' f32 sums go
-// through the workspace and the block that holds a tile's last slabs adds them up, in slab order, and stores the tile.
-// These sums are added in another order than the uncut kernel's: equal where every sum is exact, a bf16 step apart at
-// most elsewhere; the same bits from launch to launch.
+// round are cut along K into two to four pieces, a block per piece (see the job list in w4_body): the blocks of a tile
+// share its rows out between them, exchange the f32 sums of each other's rows through the workspace, and each adds up,
+// converts and stores its own rows.  These sums are added in another order than the uncut kernel's: equal where every
+// sum is exact, a bf16 step apart at most elsewhere; the same bits from launch to launch.
 #include <stdlib.h>
 
 #include <atomic>
@@ -87,11 +87,12 @@ __device__ __forceinline__ int lane_here() {
 constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) { return (vmcnt & 15) | ((vmcnt >> 4) << 14) | (7 << 4) | (lgkmcnt << 8); }
 
 // Flags of the tail pieces: a set per launch in flight (handed out round-robin: the first half to ordinary launches,
-// the second to launches recorded into a graph, which replay with the set of the recording), a word per block.  A
-// flag is raised by the block that wrote a piece and put back to zero by the one block that takes the piece, so a
-// launch leaves its set as it found it.  And the count of pieces a block gave up waiting for.
-constexpr int kW4FlagSets = 64, kW4MaxBlocks = 512;
-static __device__ unsigned int g_w4_flags[kW4FlagSets * kW4MaxBlocks];
+// the second to launches recorded into a graph, which replay with the set of the recording), and in a set a word per
+// block and reader (a tile has at most kW4MaxPieces pieces).  A flag is raised by the block that wrote its sums and put
+// back to zero by the one block it is meant for, so a launch leaves its set as it found it.  And the count of pieces a
+// block gave up waiting for.
+constexpr int kW4FlagSets = 64, kW4MaxBlocks = 512, kW4MaxPieces = 4;
+static __device__ unsigned int g_w4_flags[kW4FlagSets * kW4MaxBlocks * kW4MaxPieces];
 static __device__ unsigned int g_w4_gave_up;
 
 // PROBE (measurement aid, results meaningless): 0 the matmul; 1 the same loop with every copy reading tile (0, 0) and
@@ -135,13 +136,16 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // blocks of an XCD walk the same slabs of neighbouring tiles in step, as they do in the whole rounds -- they find each
   // other's operands in their L2.
   //
-  // A job: slabs [s0, s1) of a tile.  WHOLE: all of them, the tile is stored.  PART: the sum goes to this block's slot of
-  // the workspace and a flag follows.  LAST (the piece with the tile's last slab): waits for the tile's other pieces,
-  // adds them in the order of their slabs and stores the tile.
+  // A job: slabs [s0, s1) of a tile.  WHOLE: all of them, the tile is stored.  PIECE: one of the P pieces of a tail tile.
+  // The P blocks of a tile share its rows out between them (16-row group mt of every wave belongs to piece mt P / TM):
+  // a block writes the sums of the other blocks' rows to its slot of the workspace, raises a flag for each of them, then
+  // waits for theirs, adds their sums of its own rows to its own (own first, then the others in the order of their
+  // slabs: the same order on every launch) and stores those rows of the tile.  Nobody waits before it has published, so
+  // nobody waits for a block that waits; each block moves (P - 1) / P of a tile each way and converts 1 / P of it.
   //
   // (Jobs are worked out from the block's number every time one begins, behind a value the optimiser cannot see through:
   // kept in scalar registers across the slab loop, the block's bookkeeping pushed the loop's own values out.)
-  enum { WHOLE = 0, PART = 1, LAST = 2 };
+  enum { WHOLE = 0, PIECE = 1 };
   struct Job { int tile, s0, s1, kind; };
   struct Plan { int main_total, run_begin, nb, my, n_main, tail_c, tail_u; };
   auto plan_of = [&]() {
@@ -164,7 +168,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       const int T = total - pl.main_total, P = (nslab + pl.tail_u - 1) / pl.tail_u;
       if (pl.tail_c < T * P) {
         const int q = pl.tail_c / T, s0 = q * pl.tail_u, s1 = min(s0 + pl.tail_u, nslab);
-        tail = Job{pl.main_total + (pl.tail_c - q * T), s0, s1, s1 == nslab ? (s0 == 0 ? WHOLE : LAST) : PART};
+        tail = Job{pl.main_total + (pl.tail_c - q * T), s0, s1, P > 1 ? PIECE : WHOLE};
         n_tail = 1;
       }
     }
@@ -478,73 +482,71 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         out[1] = wall_clock64() - probe_r0;
       }
     }
-    if (job.kind == PART) {
-      // ---- the sum of this piece goes to the block's slot; the flag follows once every wave's stores have completed
+    // the 16-row groups of a wave that this block converts and stores: all of them, or its share of a tail tile
+    int mt_lo = 0, mt_hi = TM;
+    if (job.kind == PIECE) {
       const Plan pl = plan_of();
-      const int tail_c = pl.tail_c;
+      const int tail_c = pl.tail_c, T = total - pl.main_total, P = (nslab + pl.tail_u - 1) / pl.tail_u;
+      const int q = tail_c / T, t = tail_c - q * T;
+      mt_lo = q * TM / P;
+      mt_hi = (q + 1) * TM / P;
       const __amdgpu_buffer_rsrc_t w_rsrc = t2_rsrc(p.workspace, t2_clamp_u32((int64_t)gridDim.x * SLOT_BYTES));
-      unsigned int* const flags = g_w4_flags + (size_t)p.streamk_slot * kW4MaxBlocks;
-      const uint32_t base = (uint32_t)tail_c * SLOT_BYTES + (uint32_t)wave * (SLOT_BYTES / 4);
+      // (a flag per block and reader: the reader puts it down again)
+      unsigned int* const flags = g_w4_flags + (size_t)p.streamk_slot * (kW4MaxBlocks * kW4MaxPieces);
       const int lane_p = lane_here();
+      // ---- the other blocks' rows go to this block's slot; the flags follow once every wave's stores have completed
+      {
+        const uint32_t base = (uint32_t)tail_c * SLOT_BYTES + (uint32_t)wave * (SLOT_BYTES / 4);
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i) {
+          if (i >= mt_lo && i < mt_hi) continue;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const v4f a4 = acc[i][j];
-          const v4u_t v = {__float_as_uint(a4[0]), __float_as_uint(a4[1]), __float_as_uint(a4[2]), __float_as_uint(a4[3])};
-          buffer_store_b128_guarded<kDeviceScope>(v, w_rsrc, (uint32_t)lane_p * 16u, base + (uint32_t)(i * TN + j) * 1024u);
+          for (int j = 0; j < TN; ++j) {
+            const v4f a4 = acc[i][j];
+            const v4u_t v = {__float_as_uint(a4[0]), __float_as_uint(a4[1]), __float_as_uint(a4[2]), __float_as_uint(a4[3])};
+            buffer_store_b128_guarded<kDeviceScope>(v, w_rsrc, (uint32_t)lane_p * 16u, base + (uint32_t)(i * TN + j) * 1024u);
+          }
         }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-      if (wave == 0 && lane_p == 0) __hip_atomic_store(flags + tail_c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      stored = false;  // (nothing of this wave is in flight any more)
-      job = next_job;
-      tm = tm2;
-      tn = tn2;
-      cur_at = next_at;
-      continue;
-    }
-    if (job.kind == LAST) {
-      // ---- the tile's other pieces, in the order of their slabs
-      const Plan pl = plan_of();
-      const int tail_c = pl.tail_c;
-      const __amdgpu_buffer_rsrc_t w_rsrc = t2_rsrc(p.workspace, t2_clamp_u32((int64_t)gridDim.x * SLOT_BYTES));
-      unsigned int* const flags = g_w4_flags + (size_t)p.streamk_slot * kW4MaxBlocks;
-      // (the piece before slab q u of tile t is the work of block (q - 1) T + t ...)
-      const int T = total - pl.main_total;
-      const int lane_l = lane_here();
-      for (int c = job.tile - pl.main_total; c < tail_c; c += T) {
-        // (in practice long written: the other blocks computed their pieces first.  Every lane reads the same word; a
-        // block that gives up -- its partner never ran: a hung GPU -- poisons its tile with NaN and counts the event)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        if (wave == 0 && lane_p < P && lane_p != q)
+          __hip_atomic_store(flags + tail_c * kW4MaxPieces + lane_p, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      // ---- the other blocks' sums of this block's rows
+      for (int r = 0; r < P; ++r) {
+        if (r == q) continue;
+        const int c = t + r * T;
+        // (in practice written by the time this block has published its own: the pieces are equally long.  Every lane
+        // reads the same word; a block that gives up -- its partner never ran: a hung GPU -- poisons its rows with NaN
+        // and counts the event)
         bool there = false;
         for (int spin = 0; spin < (1 << 22); ++spin) {
           // (one value for the wave, so that the loop's exit is the same for every lane)
-          const unsigned int seen = __builtin_amdgcn_readfirstlane(__hip_atomic_load(flags + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+          const unsigned int seen = __builtin_amdgcn_readfirstlane(
+              __hip_atomic_load(flags + c * kW4MaxPieces + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
           if (seen != 0u) { there = true; break; }
           __builtin_amdgcn_s_sleep(16);
         }
         asm volatile("" ::: "memory");
         // (every wave has seen the flag: down it goes, for the next launch that uses this set)
         __builtin_amdgcn_s_barrier();
-        if (wave == 0 && lane_l == 0) {
-          if (there) __hip_atomic_store(flags + c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (wave == 0 && lane_p == 0) {
+          if (there) __hip_atomic_store(flags + c * kW4MaxPieces + q, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           else atomicAdd(&g_w4_gave_up, 1u);
         }
         const uint32_t base = (uint32_t)c * SLOT_BYTES + (uint32_t)wave * (SLOT_BYTES / 4);
-
-        // (a row of fragments at a time: all the loads in flight at once would want as many registers again as the sums)
         const uint32_t poison = there ? 0u : 0x7fc00000u;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
+          if (i < mt_lo || i >= mt_hi) continue;
           v4u_t v[TN];
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            v[j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (uint32_t)lane_l * 16u, base + (uint32_t)(i * TN + j) * 1024u, kDeviceScope);
+            v[j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (uint32_t)lane_p * 16u, base + (uint32_t)(i * TN + j) * 1024u, kDeviceScope);
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             acc[i][j] += v4f{__uint_as_float(v[j].x | poison), __uint_as_float(v[j].y | poison), __uint_as_float(v[j].z | poison),
                              __uint_as_float(v[j].w | poison)};
-          if (i & 1) asm volatile("" ::: "memory");
         }
       }
     }
@@ -579,6 +581,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     for (int h = 0; h < TN / 4; ++h) c_lane_h[h] = tn * BN + wn * WN + h * 64 + cc * 8 < p.N ? c_lane : 0x80000000u;
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) {
+      if (mt < mt_lo || mt >= mt_hi) continue;   // (a piece of a tail tile: the other rows are another block's)
       float a_s = 1.f;
       if constexpr (!BLOCKSCALE) a_s = a_s_all[mt];
 #pragma unroll
