@@ -570,6 +570,12 @@ def kernels_launched(kind, M, K, N):
         if os.environ.get("MAXFP8_GROUPED_PERSIST", "1") == "0":
             return "gemm_grouped_kernel", ("gemm_grouped_large_kernel (full 256-row tiles of experts with >= 1024 rows) + "
                                            "gemm_grouped_kernel (the rest), side by side on two streams")
+        if os.environ.get("MAXFP8_GROUPED_W4", "1") != "0":
+            return "gemm_w4_grouped_kernel", ("gemm_w4_grouped_kernel (four waves, 192 x 256 tiles: every slot's full 192 rows, a rest of more "
+                                              "than 32 rows behind them, and slots of 129-191 rows) on the caller's stream + "
+                                              "gemm_grouped_persist_kernel (the other rows: 128 x 256 tiles, weight-streaming rings for at most "
+                                              "32 rows) on a second stream, side by side; the blocks of the first launch past its share "
+                                              "of the chip, which they work out from the group sizes, exit at once")
         return "gemm_grouped_persist_kernel", ("one persistent launch, a block per CU: 256 x 256 tiles of every full 256 rows, "
                                                "256 x 128 / 128 x 256 tiles of the rests, weight-streaming rings for rests of at "
                                                "most 32 rows; the CUs are shared out between the matrix-bound and the streaming tiles")

@@ -144,6 +144,12 @@ static const Tuning* read_tuning(unsigned generation) {
   t->skinny_alds = num("MAXFP8_SKINNY_ALDS", 1) != 0;
   const char* sb = getenv("MAXFP8_GROUPED_SHARE");
   t->grouped_share = sb ? (float)atof(sb) : 0.5f;
+  t->grouped_w4 = num("MAXFP8_GROUPED_W4", 1) != 0;
+  t->grouped_w4_rows = num("MAXFP8_GROUPED_W4_ROWS", 2048);
+  const char* sw = getenv("MAXFP8_GROUPED_W4_SHARE");
+  t->grouped_w4_share = sw ? (float)atof(sw) : 0.6f;
+  t->grouped_w4_hot_rest = num("MAXFP8_GROUPED_W4_HOT_REST", 32);
+  t->grouped_w4_cold_rows = num("MAXFP8_GROUPED_W4_COLD_ROWS", 128);
   t->skinny = num("MAXFP8_SKINNY", 0);
   t->generation = generation;
   return t;

@@ -45,6 +45,8 @@ struct GemmArgs {
   int num_active;
   int small_rows;            // a tile with at most this many rows left for it uses the small tile shape (0: none does)
   int big_rows, big_bm;      // slots with at least big_rows rows give their full big_bm-row tiles to the large-tile launch (0: none)
+  int heads_elsewhere;       // the persistent launch: the rows of w4_grouped_head_rows are the four-wave launch's, it has no L tiles
+  int w4_hot_rest, w4_cold_rows;  // ... see w4_grouped_head_rows
   // The large-tile launch as a fixed set of blocks that share the chip with the other launch (0: one block per tile):
   int big_tile_rows;         // upper bound of the number of big_bm-row tiles over all slots
   float share_bias;          // scales the other launch's estimated work when the blocks decide how many of them stay
@@ -68,6 +70,16 @@ struct GemmArgs {
 };
 
 #if defined(__HIPCC__)
+// Rows of a slot that go to the grouped form of the four-wave kernel (192 x 256 tiles) when it runs beside the persistent
+// launch: the slot's full 192-row tiles; what is left behind them when that is more than hot_rest rows (one more tile,
+// stored up to the slot's end); a slot without a full tile whole when it has more than cold_rows rows.  The persistent
+// launch keeps the other rows.
+__device__ __forceinline__ int w4_grouped_head_rows(int rows, int hot_rest, int cold_rows) {
+  const int full = rows / 192 * 192;
+  if (full == 0) return rows > cold_rows ? rows : 0;
+  return rows - full > hot_rest ? rows : full;
+}
+
 // Element idx of a row / tensor scale vector of the given dtype, widened to f32 (exact): how the reference's
 // epilogue reads its scales (max/kernels/src/linalg/fp8_quantization.mojo:1218-1240: load, cast, multiply in f32).
 __device__ __forceinline__ float scale_at(const float* base, int64_t idx, int dtype) {

@@ -1435,8 +1435,8 @@ __global__ __launch_bounds__(512, 1) void gemm_grouped_persist_kernel(GemmArgs p
     int c[4] = {0, 0, 0, 0};
     if (tid < na) {
       const int rows = grouped_slot_count(p, tid);
-      const int head = grouped_head_rows(p, rows), rest = rows - head;
-      c[0] = head / 256;
+      const int head = p.heads_elsewhere ? w4_grouped_head_rows(rows, p.w4_hot_rest, p.w4_cold_rows) : grouped_head_rows(p, rows), rest = rows - head;
+      c[0] = p.heads_elsewhere ? 0 : head / 256;
       if (rest > 256) c[1] = (rest + 255) / 256;        // (slots below big_rows keep all their rows here)
       else if (rest > 128) c[1] = 1;
       else if (rest > p.small_rows) c[2] = 1;
@@ -1557,7 +1557,7 @@ __global__ __launch_bounds__(512, 1) void gemm_grouped_persist_kernel(GemmArgs p
     const int slot = lo, tile = rt - tb[lo];
     int64_t slot_begin, slot_end;
     grouped_slot_rows(p, slot, slot_begin, slot_end);
-    const int head = grouped_head_rows(p, (int)(slot_end - slot_begin));
+    const int head = p.heads_elsewhere ? w4_grouped_head_rows((int)(slot_end - slot_begin), p.w4_hot_rest, p.w4_cold_rows) : grouped_head_rows(p, (int)(slot_end - slot_begin));
     const int64_t row_begin = kind == 0 ? slot_begin + (int64_t)tile * 256 : slot_begin + head + (int64_t)tile * 256;
     const int64_t row_end = kind == 0 ? row_begin + 256 : slot_end;
     const int bn = kind == 1 ? 128 : (kind == 3 ? S_COLS : 256);
@@ -1696,6 +1696,8 @@ static bool persist_ok(const GemmArgs& p, bool blockscale, dim3 grid) {
 
 // The four-wave kernel (gemm_w4.hip): 0 (no), or the sixteen-row groups per wave -- 5: tiles of 160 x 256, 6: 192 x 256.
 bool gemm_w4_ok(const GemmArgs& p, bool blockscale);
+bool gemm_w4_grouped_ok(const GemmArgs& p);
+int gemm_w4_grouped_launch(const GemmArgs& p, hipStream_t stream);
 int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, bool split, hipStream_t stream);
 W4Split gemm_w4_split(int64_t M, int64_t N, int64_t K, int tm);
 
@@ -2271,9 +2273,37 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int6
   // One persistent launch that shares the chip out between its four kinds of tiles (the tuning switch
   // `grouped_persist` = 0 goes back to the two launches below).
   if (tuning().grouped_persist && !big && p.num_active <= kGroupedMaxSlots) {
+    p.share_bias = tuning().grouped_share * 2.0f;
+    // Block scaling, a slot of more than 128 rows possible, and enough rows for it to matter: every slot's full 192-row
+    // tiles, and a rest of more than 128 rows, go to the four-wave kernel (a quarter faster per row than the L tiles
+    // below on the matrix pipe, twice as fast as the M2 tiles), which is issued first on the caller's stream; the
+    // persistent launch takes the rests of at most 128 rows down the second stream.  How the
+    // CUs are shared is decided on the device, where the group sizes are (see gemm_w4.hip).
+    if (blockscale && tuning().grouped_w4 && tune != 4 && max_tokens > tuning().grouped_w4_cold_rows && T >= tuning().grouped_w4_rows && gemm_w4_grouped_ok(p)) {
+      SideStream* side = side_stream();
+      if (side) {
+        std::unique_lock<std::mutex> side_lock(side->mu);  // one fork / join at a time per device
+        p.big_rows = 0;
+        p.big_bm = 192;
+        p.small_rows = 32;
+        p.w4_hot_rest = tuning().grouped_w4_hot_rest;
+        p.w4_cold_rows = tuning().grouped_w4_cold_rows;
+        if (hipEventRecord(side->fork, stream) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+          MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "grouped matmul: cannot order the second stream behind the caller's: %s", hipGetErrorString(hipGetLastError()));
+        GemmArgs ph = p;
+        ph.share_bias = tuning().grouped_w4_share < 0.f ? tuning().grouped_w4_share : p.share_bias * tuning().grouped_w4_share;
+        int rc = gemm_w4_grouped_launch(ph, stream);
+        if (rc == MAXFP8_OK) {
+          p.heads_elsewhere = 1;
+          rc = launch_grouped_persist<true>(p, side->stream, "gemm_grouped_persist_block");
+        }
+        if ((hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(stream, side->join, 0) != hipSuccess) && rc == MAXFP8_OK)
+          MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "grouped matmul: cannot join the second stream: %s", hipGetErrorString(hipGetLastError()));
+        return rc;
+      }
+    }
     // (every slot's full 256-row tiles are L tiles here: one kernel, no second launch to fill)
     p.big_rows = tune != 4 ? 256 : 0;
-    p.share_bias = tuning().grouped_share * 2.0f;
     return blockscale ? launch_grouped_persist<true>(p, stream, "gemm_grouped_persist_block")
                       : launch_grouped_persist<false>(p, stream, "gemm_grouped_persist_row");
   }

@@ -98,7 +98,19 @@ static __device__ unsigned int g_w4_gave_up;
 // PROBE (measurement aid, results meaningless): 0 the matmul; 1 the same loop with every copy reading tile (0, 0) and
 // slabs 0..7 over and over, so that its operands stay in L2; 2 the same without copies, waits and barriers -- the
 // MFMA loop on what the prologue left in LDS.
-template <int TM, int TN, bool BLOCKSCALE, int PROBE>
+//
+// GROUPED (the MoE matmul, block scaling; BM = 192): the tiles are those of w4_grouped_head_rows of every slot -- its full
+// BM-row tiles and one more for a rest of more than 128 rows, stored up to the slot's end --
+// numbered through all slots as if they were the row tiles of one matrix: row tile v lies in the slot
+// found by bisection in a prefix table that every block builds in LDS from the device-resident offsets, and its weights
+// are that slot's expert's.  The other rows are another launch's, sent down a second stream at the same time: this
+// launch is issued first with a block per CU, every block adds up what both launches have to do (tiles x the cost
+// model's time per tile), and the blocks past this launch's share of the chip exit at once and leave their CUs to the
+// other one.
+constexpr int kW4GroupedSlots = 256;  // slots (active experts) the tables hold, one per thread
+constexpr int kW4GroupedTableBytes = (4 * kW4GroupedSlots + 16) * 4;
+
+template <int TM, int TN, bool BLOCKSCALE, int PROBE, bool GROUPED = false>
 __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   constexpr int WM = TM * 16, WN = TN * 16, BM = 2 * WM, BN = 2 * WN;
   constexpr int IA = BM / 32, IB = BN / 32;                  // copy instructions per wave and slab (8 rows each)
@@ -119,14 +131,82 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   static_assert(PER_B + NSTORE < 64, "the count must fit the vmcnt field");
   static_assert(IB % 2 == 0, "the weight copies go out in two halves");
 
+  static_assert(!GROUPED || (BLOCKSCALE && PROBE == 0), "the grouped form is built for block scaling");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int lm = lane & 15, lq = lane >> 4;
   const int nslab = p.K / 128;                               // whole slabs, an even number of them (the host's rule)
 
+  // ---- grouped: the tables (behind the side buffers).  hdr[0] = row tiles of all slots, hdr[1] = the blocks that stay;
+  // tab_tiles[z] = row tiles in the slots before z, tab_begin[z] = slot z's first row, tab_expert[z] = its expert.
+  int* const hdr = reinterpret_cast<int*>(smem + SIDE_BASE + 4 * SIDE_BYTES);
+  int* const tab_tiles = hdr + 8;                      // (kW4GroupedSlots + 1 entries: the last is the total)
+  int* const tab_begin = tab_tiles + kW4GroupedSlots + 8;
+  int* const tab_expert = tab_begin + kW4GroupedSlots;
+  int* const tab_end = tab_expert + kW4GroupedSlots;
+  if constexpr (GROUPED) {
+    static_assert(BM == 192, "w4_grouped_head_rows");
+    const int na = p.num_active;
+    if (tid < 8) hdr[tid] = 0;
+    __syncthreads();
+    int c = 0, begin = 0, end = 0, e = -1;
+    if (tid < na) {
+      // (rows held inside [0, M): a stale routing tensor must not turn into accesses outside the operands)
+      const int64_t M = p.M;
+      int64_t b64 = p.offsets[tid], e64 = p.offsets[tid + 1];
+      if (b64 > M) b64 = M;
+      if (e64 > M) e64 = M;
+      if (e64 < b64) e64 = b64;
+      const int rows = (int)(e64 - b64);
+      const int head = w4_grouped_head_rows(rows, p.w4_hot_rest, p.w4_cold_rows), rest = rows - head;
+      c = (head + BM - 1) / BM;
+      begin = (int)b64;
+      end = (int)e64;
+      e = p.expert_ids[tid];
+      // the other launch's tiles, for the shares: a rest of more than small_rows, of anything
+      if (rest > p.small_rows) atomicAdd(&hdr[3], 1);
+      else if (rest > 0) atomicAdd(&hdr[4], 1);
+    }
+    int incl = c;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    __shared__ int s_wave_sum[4];
+    if (lane == 63) s_wave_sum[wave] = incl;
+    __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += s_wave_sum[w];
+    tab_tiles[tid] = before + incl - c;
+    if (tid == 255) tab_tiles[256] = before + incl;
+    tab_begin[tid] = begin;
+    tab_expert[tid] = e;
+    tab_end[tid] = end;
+    if (tid == 255) {
+      const int R = before + incl;
+      const float ns = (float)nslab;
+      const int ncol = (p.N + BN - 1) / BN;
+      const float w_here = (float)(R * ncol) * (ns * 1.15f + 3.0f);
+      const float w_there = (float)(hdr[2] * ((p.N + 127) / 128) + hdr[3] * ((p.N + 255) / 256)) * (ns * 0.92f + 9.0f) +
+                            (float)(hdr[4] * ((p.N + 511) / 512)) * (ns * 2.6f + 6.0f) * p.share_bias;
+      const int G = (int)gridDim.x & ~7;
+      int keep = (int)((float)G * w_here / (w_here + w_there + 1e-9f) + 4.0f) & ~7;
+      if (p.share_bias < 0.f) keep = (int)(-p.share_bias) & ~7;
+      if (keep < 8) keep = 8;
+      if (keep > G) keep = G;
+      if (keep > R * ncol) keep = (R * ncol + 7) & ~7;
+      hdr[0] = R;
+      hdr[1] = R > 0 ? keep : 0;
+    }
+    __syncthreads();
+    if ((int)blockIdx.x >= hdr[1]) return;
+  }
+  auto grouped_hdr = [&](int i) { return __builtin_amdgcn_readfirstlane(hdr[i]); };
+
   // ---- this block's tiles: every nb-th tile of its XCD's contiguous run (blocks are dealt to the XCDs round-robin)
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN, total = tiles_m * tiles_n;
+  const int tiles_m = GROUPED ? grouped_hdr(0) : (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN, total = tiles_m * tiles_n;
   const int bs_rows = (p.N + 127) / 128;  // rows of the weight scales: a wave whose columns all lie past N reads the last one
   // The tail (p.tail_units = u > 0; the host then launches a multiple of 8 blocks and no more than there are tiles): the
   // T tiles beyond the last whole round of the blocks are not dealt out whole.  Each is cut along K into pieces of u slabs
@@ -149,9 +229,9 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   struct Job { int tile, s0, s1, kind; };
   struct Plan { int main_total, run_begin, nb, my, n_main, tail_c, tail_u; };
   auto plan_of = [&]() {
-    const int bid = opaque_uniform((int)blockIdx.x), G = (int)gridDim.x;
+    const int bid = opaque_uniform((int)blockIdx.x), G = GROUPED ? grouped_hdr(1) : (int)gridDim.x;
     const int xcd = bid & 7, my = bid >> 3;
-    const int tail_u = PROBE ? 0 : p.tail_units;
+    const int tail_u = PROBE || GROUPED ? 0 : p.tail_units;
     const int main_total = tail_u > 0 ? (total / G) * G : total;
     const int run_begin = xcd * (main_total >> 3) + (xcd < (main_total & 7) ? xcd : (main_total & 7));
     const int run_len = (main_total >> 3) + (xcd < (main_total & 7) ? 1 : 0);
@@ -183,7 +263,8 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // ---- global -> LDS copy plan (LDS-DMA, 16 bytes per lane, 8 rows x 128 bytes per instruction; lane (r, p) fetches
   // the chunk p ^ f(row) of its row, so the bytes land swizzled for conflict-free fragment reads)
   const __amdgpu_buffer_rsrc_t a_rsrc = t2_rsrc(p.a, t2_clamp_u32((int64_t)(p.M - 1) * p.lda + p.K));
-  const __amdgpu_buffer_rsrc_t b_rsrc = t2_rsrc(p.b, t2_clamp_u32((int64_t)(p.N - 1) * p.ldb + p.K));
+  const uint32_t b_range = t2_clamp_u32((int64_t)(p.N - 1) * p.ldb + p.K);
+  const __amdgpu_buffer_rsrc_t b_rsrc = t2_rsrc(p.b, b_range);
   const int cr = lane >> 3, cp = lane & 7;
   const int cchunk = cp ^ cr;
   const int cchunk_b = cp ^ (((wave & 1) << 2) | (cr & 3));
@@ -201,20 +282,33 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     if (mt_w >= TM) s_voff = 0x80000000u;
     s_slab_step = (uint32_t)p.a_scales_ld * 4u;
   }
-  struct TileAt { uint32_t a, b, s; };  // byte offsets of a tile's activation rows, weight rows and activation scales
-  auto tile_at = [&](int tm, int tn) {
-    if constexpr (PROBE != 0) return TileAt{0u, 0u, 0u};
-    return TileAt{(uint32_t)(tm * BM) * (uint32_t)p.lda, (uint32_t)(tn * BN) * (uint32_t)p.ldb, (uint32_t)(tm * BM) * 4u};
+  // byte offsets of a tile's activation rows, weight rows and activation scales; its first row; grouped: its expert's
+  // weights and the element of the weight scales where the expert's begin
+  struct TileAt { uint32_t a, b, s; int row0, row_end; const uint8_t* bp; uint32_t bs0; };
+  // (grouped: tm = the row tile's number among its slot's, slot = that slot)
+  auto tile_at = [&](int tm, int tn, int slot) {
+    if constexpr (PROBE != 0) return TileAt{0u, 0u, 0u, 0, 0, p.b, 0u};
+    if constexpr (GROUPED) {
+      const int lo = slot;
+      const int row0 = __builtin_amdgcn_readfirstlane(tab_begin[lo]) + tm * BM;
+      const int e = __builtin_amdgcn_readfirstlane(tab_expert[lo]), row_end = __builtin_amdgcn_readfirstlane(tab_end[lo]);
+      // (no expert: the weight copies read out of range, i.e. zeros, and the tile is stored as zeros)
+      const uint32_t none = e < 0 ? 0x80000000u : 0u;
+      const int ee = e < 0 ? 0 : e;
+      return TileAt{(uint32_t)row0 * (uint32_t)p.lda, ((uint32_t)(tn * BN) * (uint32_t)p.ldb) | none, (uint32_t)row0 * 4u, row0, row_end,
+                    p.b + (int64_t)ee * p.b_expert_stride, (uint32_t)((int64_t)ee * p.bs_expert_stride)};
+    }
+    return TileAt{(uint32_t)(tm * BM) * (uint32_t)p.lda, (uint32_t)(tn * BN) * (uint32_t)p.ldb, (uint32_t)(tm * BM) * 4u, tm * BM, p.M, p.b, 0u};
   };
   // copy number idx (0 .. PER_A - 1) of a slab's activation rows and scales into activation stage `stage`
   // Where a slab's copies read: the scalar offsets of its first activation, weight and scale copy.  A slab of nothing
   // (behind the block's last tile) gets offsets past 2^31: the scalar offset takes part in the descriptor's range
   // check, so such copies write zeros.  (K is a whole number of slabs: no lane ever reads past a row's end.)
-  struct SlabAt { uint32_t a, b, s; };
+  struct SlabAt { uint32_t a, b, s; const uint8_t* bp; };
   auto slab_at = [&](const TileAt& at, int slab, uint32_t dead) {
     if constexpr (PROBE != 0) slab &= 7;
     const uint32_t koff = (uint32_t)slab * 128u;
-    return SlabAt{(at.a + koff) | dead, (at.b + koff) | dead, (at.s + (uint32_t)slab * s_slab_step) | dead};
+    return SlabAt{(at.a + koff) | dead, (at.b + koff) | dead, (at.s + (uint32_t)slab * s_slab_step) | dead, at.bp};
   };
   // copy number idx (0 .. PER_A - 1) of a slab's activation rows and scales into activation stage `stage`
   auto dma_a = [&](const SlabAt& at, int stage, int idx) {
@@ -228,7 +322,9 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // copy number idx (0 .. PER_B - 1) of a slab's weight rows into weight stage `stage`
   auto dma_b = [&](const SlabAt& at, int stage, int idx) {
     uint8_t* sb = smem + B_BASE + stage * B_STAGE;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(sb + (idx * 4 + wave) * 1024), 16, b_voff, at.b + idx * b_istep, 0, 0);
+    // (grouped: the descriptor of the expert whose rows this slab's copies read)
+    const __amdgpu_buffer_rsrc_t rsrc = GROUPED ? t2_rsrc(at.bp, b_range) : b_rsrc;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(sb + (idx * 4 + wave) * 1024), 16, b_voff, at.b + idx * b_istep, 0, 0);
   };
 
   // ---- fragment read plan.  Activation fragment mt: rows mt * 16 + lm of the wave's rows.  Weight fragments come in
@@ -278,11 +374,35 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   const __amdgpu_buffer_rsrc_t c_rsrc = t2_rsrc(p.c, t2_clamp_u32(((int64_t)(p.M - 1) * p.ldc + p.N) * 2));
   const uint32_t c_row_bytes = (uint32_t)p.ldc * 2u;
 
+  // Where tile number t lies.  Grouped: the tiles are numbered slot by slot, in a slot column by column, in a column
+  // row tile by row tile -- the blocks of an XCD, which take neighbouring numbers, work on all row tiles of a few weight
+  // columns of one expert at a time (each weight tile comes from memory once), and an XCD's run of the numbers is a run
+  // of slots: the weights of an expert are read by one XCD or two.
+  auto locate = [&](int t, int& tm, int& tn, int& slot) {
+    slot = 0;
+    if constexpr (GROUPED) {
+      // the last z with tab_tiles[z] * tiles_n <= t (slots without tiles repeat their successor's value and are skipped
+      // by taking the last)
+      const int v = t / tiles_n;
+      int lo = 0, hi = p.num_active;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (__builtin_amdgcn_readfirstlane(tab_tiles[mid]) <= v) lo = mid; else hi = mid;
+      }
+      const int first = __builtin_amdgcn_readfirstlane(tab_tiles[lo]), c = __builtin_amdgcn_readfirstlane(tab_tiles[lo + 1]) - first;
+      const int rem = t - first * tiles_n;
+      tn = rem / c;
+      tm = rem - tn * c;
+      slot = lo;
+    } else {
+      tile_coords<kGroupM>(t, tiles_m, tiles_n, tm, tn);
+    }
+  };
   // ---- prologue: slabs 0 and 1 of the first tile
-  int tm, tn;
-  tile_coords<kGroupM>(job.tile, tiles_m, tiles_n, tm, tn);
+  int tm, tn, slot;
+  locate(job.tile, tm, tn, slot);
   if constexpr (PROBE != 0) tm = tn = 0;
-  TileAt cur_at = tile_at(tm, tn);
+  TileAt cur_at = tile_at(tm, tn, slot);
   {
     const SlabAt s0 = slab_at(cur_at, job.s0, 0u), s1 = slab_at(cur_at, job.s0 + 1, 0u), s2 = slab_at(cur_at, job.s0 + 2, 0u);
 #pragma unroll
@@ -311,7 +431,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     return blk < bs_rows ? blk : bs_rows - 1;
   };
   // The weight-block scale of a slab is element bs_cur of the weight scales: that of the slab to come is loaded a slab ahead.
-  uint32_t bs_cur = (uint32_t)(bs_block(tn) * p.b_scales_ld + job.s0);
+  uint32_t bs_cur = cur_at.bs0 + (uint32_t)(bs_block(tn) * p.b_scales_ld + job.s0);
   float bs_nxt = 1.f;
   if constexpr (BLOCKSCALE) bs_nxt = scalar_load_f32(p.b_scales + bs_cur);
 
@@ -354,11 +474,12 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     const bool has_next = k + 1 < njobs;
     const Job next_job = has_next ? job_of(k + 1, nullptr) : job;
     int tm2 = tm, tn2 = tn;
-    if (has_next) tile_coords<kGroupM>(next_job.tile, tiles_m, tiles_n, tm2, tn2);
-    const TileAt next_at = tile_at(tm2, tn2);
+    int slot2 = slot;
+    if (has_next) locate(next_job.tile, tm2, tn2, slot2);
+    const TileAt next_at = tile_at(tm2, tn2, slot2);
     // the first slab of the next job (of nothing behind the block's last one: offsets past 2^31 read as zeros)
     const SlabAt next0 = slab_at(next_at, next_job.s0, has_next ? 0u : 0x80000000u);
-    const uint32_t next_bs0 = (uint32_t)(bs_block(tn2) * p.b_scales_ld + next_job.s0);
+    const uint32_t next_bs0 = next_at.bs0 + (uint32_t)(bs_block(tn2) * p.b_scales_ld + next_job.s0);
     const int job_end = job.s1;
 
     v4f acc[TM][TN];
@@ -443,6 +564,9 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
           constexpr int d = ((i - 1) * NCOPY + NSLOT - 1) / NSLOT;
           if constexpr (d < NCOPY && d * NSLOT / NCOPY == i - 1) {
             if constexpr (d < PER_A) dma_a(my, PAR, d);
+            // (grouped: the expert of the weight copies changes with their offset, but at the slab's end, behind these copies:
+            // they read through cur.bp, and the old value need not be kept beside the new one)
+            else if constexpr (GROUPED) dma_b(SlabAt{my.a, my.b, my.s, cur.bp}, bst, d - PER_A);
             else dma_b(my, bst, d - PER_A);
           }
         }
@@ -462,6 +586,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt) af[PAR ^ 1][mt] = in_agprs(af[PAR ^ 1][mt]);
       bst = bst1;
+      if constexpr (GROUPED) cur.bp = slab + 4 == job_end ? next0.bp : cur.bp;
     };
 
     constexpr std::integral_constant<int, 0> EVEN{};
@@ -484,7 +609,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     }
     // the 16-row groups of a wave that this block converts and stores: all of them, or its share of a tail tile
     int mt_lo = 0, mt_hi = TM;
-    if (job.kind == PIECE) {
+    if (!GROUPED && job.kind == PIECE) {
       const Plan pl = plan_of();
       const int tail_c = pl.tail_c, T = total - pl.main_total, P = (nslab + pl.tail_u - 1) / pl.tail_u;
       const int q = tail_c / T, t = tail_c - q * T;
@@ -568,7 +693,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    const uint32_t c_tile = ((uint32_t)(tm * BM + wm * WM) * (uint32_t)p.ldc + (uint32_t)(tn * BN + wn * WN)) * 2u;
+    const uint32_t c_tile = ((uint32_t)(cur_at.row0 + wm * WM) * (uint32_t)p.ldc + (uint32_t)(tn * BN + wn * WN)) * 2u;
     // (the lane's offsets are formed here, out of sight of the optimiser: hoisted out of the tile loop they would sit in
     // vector registers all through the slab loop, which has none to spare)
     const int lane_e = lane_here();
@@ -611,12 +736,16 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       }
     };
     // ... and stored (non-temporal: C is not read again here, and its lines should not push the operands out of L2)
+    // (grouped: C ends, for this tile, where the tile's slot ends -- the rows of a slot's last tile that lie past it are
+    // the next slot's, and are not stored)
+    const __amdgpu_buffer_rsrc_t c_rsrc_tile =
+        GROUPED ? t2_rsrc(p.c, t2_clamp_u32(((int64_t)(cur_at.row_end - 1) * p.ldc + p.N) * 2)) : c_rsrc;
     auto store_step = [&](const v4u_t (&v)[2], int mt, int h) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-        buffer_store_b128_guarded<2>(v[i], c_rsrc, c_lane_h[h], c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes + (uint32_t)h * 128u);
+        buffer_store_b128_guarded<2>(v[i], c_rsrc_tile, c_lane_h[h], c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes + (uint32_t)h * 128u);
     };
-    if (job.kind == WHOLE) {
+    if (GROUPED || job.kind == WHOLE) {
       // The steps overlap: a step's two reads go out together, the next step is converted and written behind them (the
       // LDS executes a wave's operations in order, so those writes cannot overtake the reads), and only then are the
       // reads waited for and stored -- one LDS round trip per step, hidden behind the next step's conversions, instead of
@@ -647,6 +776,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     job = next_job;
     tm = tm2;
     tn = tn2;
+    slot = slot2;
     cur_at = next_at;
   }
   // the last copies (of nothing: every lane out of range) still write zeros into the stages: they must have landed
@@ -658,6 +788,12 @@ template <int TM, int TN, bool BLOCKSCALE, int PROBE>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_w4_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   w4_body<TM, TN, BLOCKSCALE, PROBE>(p, smem);
+}
+
+template <int TM, int TN, bool BLOCKSCALE>
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_w4_grouped_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  w4_body<TM, TN, BLOCKSCALE, 0, true>(p, smem);
 }
 
 template <int TM, int TN, bool BLOCKSCALE>
@@ -745,6 +881,39 @@ int gemm_w4_launch(const GemmArgs& p_in, bool blockscale, int tm, bool split, hi
   if (tm == 5)
     return blockscale ? launch_w4<5, true, 0>(p, blocks, stream, "gemm_w4_block_160x256") : launch_w4<5, false, 0>(p, blocks, stream, "gemm_w4_row_160x256");
   return blockscale ? launch_w4<6, true, 0>(p, blocks, stream, "gemm_w4_block_192x256") : launch_w4<6, false, 0>(p, blocks, stream, "gemm_w4_row_192x256");
+}
+
+// The grouped form takes: block scaling (the caller's business), bf16 C with 16-byte aligned rows, N a multiple of 8, K a
+// whole and even number of slabs, at most kW4GroupedSlots slots, no row index on C, operands whose byte offsets fit 31
+// bits (per expert, for the weights).
+bool gemm_w4_grouped_ok(const GemmArgs& p) {
+  if (p.M < 192 || p.N <= 0 || p.N % 8 != 0 || p.K < 512 || p.K % 256 != 0) return false;
+  if (p.num_active <= 0 || p.num_active > kW4GroupedSlots || p.c_row_index != nullptr) return false;
+  if (p.c_dtype != MAXFP8_BF16 || !p.c_vec8_ok) return false;
+  const int64_t lim = 0x7ff00000ll, nslab = p.K / 128;
+  const int64_t rows = (int64_t)p.M + 192;
+  if (rows * p.lda >= lim || (ceil_div(p.N, 256) * 256) * p.ldb >= lim) return false;
+  if ((nslab * p.a_scales_ld + rows) * 4 >= lim || rows * p.ldc * 2 >= lim) return false;
+  if ((int64_t)p.num_active * p.bs_expert_stride + (ceil_div(p.N, 128) + 1) * p.b_scales_ld >= lim / 4) return false;
+  return true;
+}
+
+// The full 192-row tiles of the slots with at least 192 rows (p.big_rows == p.big_bm == 192); the other launch takes the
+// rest.  A block per CU: the blocks past this launch's share of the chip exit at once.
+int gemm_w4_grouped_launch(const GemmArgs& p, hipStream_t stream) {
+  static PerDeviceFlag attr_done;
+  constexpr int lds = w4_lds_bytes<6, 8, true>() + kW4GroupedTableBytes;
+  static_assert(lds <= 160 * 1024, "one block's LDS");
+  const char* name = "gemm_w4_grouped_block_192x256";
+  auto kern = gemm_w4_grouped_kernel<6, 8, true>;
+  bool& done = attr_done.here();
+  if (!done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, lds, hipGetErrorString(e));
+    done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)((compute_units() / 8) * 8)), dim3(256), lds, stream, p);
+  return launch_status(name);
 }
 
 // Pieces of a cut tail that a block stopped waiting for, on the current device since the library was loaded (0 unless

@@ -34,6 +34,15 @@ struct Tuning {
   bool grouped_persist = true;
   bool grouped_overlap = true;
   float grouped_share = 0.5f;
+  // The grouped matmul's full 192-row tiles on the four-wave kernel, beside the persistent launch of the rest (block
+  // scaling; MAXFP8_GROUPED_W4 = 0: one persistent launch); the least number of rows for it (MAXFP8_GROUPED_W4_ROWS);
+  // a factor on the other launch's estimated work when the blocks decide their shares (MAXFP8_GROUPED_W4_SHARE; a negative
+  // value is the number of blocks that stay, outright: -160 keeps 160); which rows go to the four-wave launch beside the
+  // full 192-row tiles (MAXFP8_GROUPED_W4_HOT_REST, MAXFP8_GROUPED_W4_COLD_ROWS: see w4_grouped_head_rows).
+  bool grouped_w4 = true;
+  int grouped_w4_rows = 2048;
+  float grouped_w4_share = 0.6f;
+  int grouped_w4_hot_rest = 32, grouped_w4_cold_rows = 128;
   int skinny = 0;
   bool skinny_alds = true;
   unsigned generation = 0;  // counts the reloads: part of the key of every cache that depends on the switches

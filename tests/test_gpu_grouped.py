@@ -192,6 +192,77 @@ def test_random_groupings_are_exact(dev, tune, launches):
         assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, N {N}, K {K}, {out}"
 
 
+def test_four_wave_launch_beside_the_persistent_one_is_exact(dev, tune):
+    """Block scaling with K an even number (at least four) of slabs: the slots' full 192-row tiles, and a rest of more
+    than 32 rows behind them (more than 128 rows for a slot without a full tile), go to the grouped form of the
+    four-wave kernel, the other rows to the persistent launch on a second stream.  A seeded sweep of groupings around
+    those bounds (191 / 192 / 193, 224 / 225, 320 / 321, 128 / 129 rows, empty slots, skipped experts, rows past the
+    last slot, ragged N) on integer data: every row that belongs to a slot equals the scalar kernel's bit for bit, with
+    the rule's bounds at their defaults and moved (every rest to the four-wave launch; none)."""
+    rng = np.random.default_rng(5)
+    for it in range(30):
+        hot, cold = [("32", "128"), ("0", "32"), ("128", "128")][it % 3]
+        tune(MAXFP8_GROUPED_W4_ROWS="0", MAXFP8_GROUPED_W4_HOT_REST=hot, MAXFP8_GROUPED_W4_COLD_ROWS=cold)
+        E = int(rng.integers(1, 24))
+        active = int(rng.integers(1, E + 1))
+        if it % 3 == 0:
+            counts = rng.choice([0, 5, 128, 129, 191, 192, 193, 224, 225, 320, 321, 383, 384, 385, 1000], active)
+        elif it % 3 == 1:
+            counts = rng.choice([0, 1, 32, 33, 129, 192, 300, 1023, 1024, 1300, 2600], active)
+        else:
+            counts = (rng.zipf(1.3, active) * 97 % 3000).astype(np.int64)
+        ids = rng.permutation(E)[:active].astype(np.int32)
+        ids[rng.random(active) < 0.1] = -1
+        extra = int(rng.integers(0, 9)) if it % 4 == 0 else 0
+        N = 8 * int(rng.integers(8, 160)) if it % 2 else 128 * int(rng.integers(1, 12))
+        K = 256 * int(rng.integers(2, 7))
+        if counts.sum() == 0:
+            counts[0] = 200
+        live = int(counts.sum())
+        T = live + extra
+        a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (T, K)).astype(np.float32)))
+        b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (E, N, K)).astype(np.float32)))
+        sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (K // 128, -(-T // 4) * 4))).astype(np.float32))
+        sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (E, -(-N // 128), K // 128))).astype(np.float32))
+        off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32)
+        idt = torch.tensor(list(ids) + [-1] * (E - active), dtype=torch.int32)
+        got = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=torch.bfloat16, fill=None)
+        want = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=torch.bfloat16, algo="naive")
+        assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, ids {ids.tolist()}, N {N}, K {K}"
+
+
+def test_four_wave_launch_has_the_bits_of_the_one_launch_form(dev, tune):
+    """Random (inexact) data on a skewed routing of 64 experts: both forms add a row's products up in the same order,
+    so the two launches side by side give the bits of the one persistent launch -- also with a share of the chip forced
+    on the four-wave launch that is too small and too large, and on twelve launches in a row (each block works its
+    share out again, and the second stream is joined every time)."""
+    off, ids, counts, stats = synth.moe_routing(1024, 64, 8, seed=3, zipf_a=1.1)
+    T, N, K = int(counts.sum()), 1024, 1024
+    a, b = synth.random_fp8((T, K), 11).to(dev), synth.random_fp8((64, N, K), 12).to(dev)
+    sa = synth.random_scales((K // 128, T), 13).to(dev)
+    sb = synth.random_scales((64, N // 128, K // 128), 14).to(dev)
+    off, ids = off.to(dev), ids.to(dev)
+    assert int(counts.max()) >= 192 and int((counts % 192 <= 32).sum()) > 0
+
+    def launch():
+        return mx.grouped_dynamic_scaled_fp8_matmul(a, b, sa, sb, off, ids, stats, BLK.input_scale, BLK.weight_scale,
+                                                    out_type=torch.bfloat16)
+
+    tune(MAXFP8_GROUPED_W4="0")
+    want = launch()
+    torch.cuda.synchronize()
+    for share in (None, "-8", "-256"):
+        tune(MAXFP8_GROUPED_W4=None, MAXFP8_GROUPED_W4_SHARE=share)
+        outs = [launch() for _ in range(12)]
+        torch.cuda.synchronize()
+        for i, got in enumerate(outs):
+            assert torch.equal(got, want), f"share {share}, launch {i}"
+    r = int(torch.argmax(counts))
+    row = int(counts[:r].sum())
+    cpu = oracle.matmul_blockwise(fp8_bytes(a[row:row + 1]), fp8_bytes(b[r]), f32_np(sa[:, row:row + 1]), f32_np(sb[r]), threads=NT)
+    assert_rel(f32_np(want[row:row + 1]), cpu, TOL, "a row of the largest slot against the CPU oracle", natural_scale=True)
+
+
 @pytest.mark.parametrize("counts,N", [([1024] * 8, 2048), ([8] * 100, 1024), ([200] * 40, 512), ([100] * 30 + [1300] * 3, 768)])
 def test_launches_of_one_kind_of_tile_many_times(dev, counts, N):
     """A grouping whose tiles are all of one kind (256-row tiles only; streaming tiles only; one mid-size kind) leaves
