@@ -108,9 +108,14 @@ static __device__ unsigned int g_w4_gave_up;
 // model's time per tile), and the blocks past this launch's share of the chip exit at once and leave their CUs to the
 // other one.
 constexpr int kW4GroupedSlots = 256;  // slots (active experts) the tables hold, one per thread
-constexpr int kW4GroupedTableBytes = (4 * kW4GroupedSlots + 16) * 4;
+constexpr int kW4GroupedTableBytes = (16 + 4 * kW4GroupedSlots + 8) * 4 + 4 * 96 * 4;  // (and the index entries of a tile's 96 rows, per wave)
 
-template <int TM, int TN, bool BLOCKSCALE, int PROBE, bool GROUPED = false>
+//
+// GROUPED == 2: with a row index on C (row m of the result goes to row p.c_row_index[m]).  The index entries of a tile's
+// rows are copied into LDS by two more copy instructions per wave, issued behind the stores of the tile before (in front
+// of the first tile: in the prologue) -- not loaded into registers in the epilogue, where waiting for such a load would
+// mean waiting for every weight copy in flight, in-order completion being what the copy waits rely on.
+template <int TM, int TN, bool BLOCKSCALE, int PROBE, int GROUPED = 0>
 __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   constexpr int WM = TM * 16, WN = TN * 16, BM = 2 * WM, BN = 2 * WN;
   constexpr int IA = BM / 32, IB = BN / 32;                  // copy instructions per wave and slab (8 rows each)
@@ -141,14 +146,16 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // ---- grouped: the tables (behind the side buffers).  hdr[0] = row tiles of all slots, hdr[1] = the blocks that stay;
   // tab_tiles[z] = row tiles in the slots before z, tab_begin[z] = slot z's first row, tab_expert[z] = its expert.
   int* const hdr = reinterpret_cast<int*>(smem + SIDE_BASE + 4 * SIDE_BYTES);
-  int* const tab_tiles = hdr + 8;                      // (kW4GroupedSlots + 1 entries: the last is the total)
+  int* const tab_tiles = hdr + 16;                     // (kW4GroupedSlots + 1 entries: the last is the total)
   int* const tab_begin = tab_tiles + kW4GroupedSlots + 8;
   int* const tab_expert = tab_begin + kW4GroupedSlots;
   int* const tab_end = tab_expert + kW4GroupedSlots;
+  constexpr bool SCATTER = GROUPED == 2;
+  uint32_t* const idx_lds = reinterpret_cast<uint32_t*>(tab_end + kW4GroupedSlots) + wave * 96;  // this wave's rows' entries
   if constexpr (GROUPED) {
     static_assert(BM == 192, "w4_grouped_head_rows");
     const int na = p.num_active;
-    if (tid < 8) hdr[tid] = 0;
+    if (tid < 16) hdr[tid] = 0;
     __syncthreads();
     int c = 0, begin = 0, end = 0, e = -1;
     if (tid < na) {
@@ -174,7 +181,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       const int up = __shfl_up(incl, o, 64);
       if (lane >= o) incl += up;
     }
-    __shared__ int s_wave_sum[4];
+    int* const s_wave_sum = hdr + 8;  // (no static LDS in this kernel: it would push the stages past the block's 160 KB)
     if (lane == 63) s_wave_sum[wave] = incl;
     __syncthreads();
     int before = 0;
@@ -398,11 +405,27 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       tile_coords<kGroupM>(t, tiles_m, tiles_n, tm, tn);
     }
   };
+  // the index entries of the 96 rows of this wave in the tile that begins at row0: lane l copies entry l, and lanes 0 .. 31
+  // entry 64 + l (entries past the end of the index read as zero: such rows are not stored).  Two vector memory
+  // operations for every lane's count, whether or not the lane takes part in the second.
+  auto dma_idx = [&](int row0) {
+    if constexpr (SCATTER) {
+      static_assert(!SCATTER || WM == 96, "two copies of 64 and 32 entries");
+      const __amdgpu_buffer_rsrc_t i_rsrc = t2_rsrc(p.c_row_index, t2_clamp_u32((int64_t)p.M * 4));
+      const int l = lane_here();
+      const uint32_t at = (uint32_t)(row0 + wm * WM) * 4u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(i_rsrc, (lds_ptr_t)idx_lds, 4, (uint32_t)l * 4u, at, 0, 0);
+      // (under the execution mask: a lane whose offset is merely out of range would still write a zero, into the next
+      // wave's entries)
+      if (l < 32) __builtin_amdgcn_raw_ptr_buffer_load_lds(i_rsrc, (lds_ptr_t)(idx_lds + 64), 4, (uint32_t)l * 4u, at + 256u, 0, 0);
+    }
+  };
   // ---- prologue: slabs 0 and 1 of the first tile
   int tm, tn, slot;
   locate(job.tile, tm, tn, slot);
   if constexpr (PROBE != 0) tm = tn = 0;
   TileAt cur_at = tile_at(tm, tn, slot);
+  dma_idx(cur_at.row0);
   {
     const SlabAt s0 = slab_at(cur_at, job.s0, 0u), s1 = slab_at(cur_at, job.s0 + 1, 0u), s2 = slab_at(cur_at, job.s0 + 2, 0u);
 #pragma unroll
@@ -728,11 +751,18 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     };
     // ... read back as 8 rows x one whole 128-byte line per instruction (a wave reads back only what it wrote itself, and
     // its LDS operations execute in order) ...
-    auto read_back = [&](v4u_t (&v)[2]) {
+    // (with a row index: dst[i] = the byte offset in C of the row that receives row mt * 16 + i * 8 + rr of the wave's part,
+    // past every range for a row behind the slot's end)
+    auto read_back = [&](v4u_t (&v)[2], uint32_t (&dst)[2], int mt) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int r = i * 8 + rr;
         v[i] = *reinterpret_cast<const v4u_t*>(wbuf + r * 128 + ((cc ^ (r & 7)) * 16));
+        dst[i] = 0u;
+        if constexpr (SCATTER) {
+          const int row = mt * 16 + r;
+          dst[i] = cur_at.row0 + wm * WM + row < cur_at.row_end ? idx_lds[row] * c_row_bytes + (uint32_t)cc * 16u : 0x80000000u;
+        }
       }
     };
     // ... and stored (non-temporal: C is not read again here, and its lines should not push the operands out of L2)
@@ -740,10 +770,14 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     // the next slot's, and are not stored)
     const __amdgpu_buffer_rsrc_t c_rsrc_tile =
         GROUPED ? t2_rsrc(p.c, t2_clamp_u32(((int64_t)(cur_at.row_end - 1) * p.ldc + p.N) * 2)) : c_rsrc;
-    auto store_step = [&](const v4u_t (&v)[2], int mt, int h) {
+    auto store_step = [&](const v4u_t (&v)[2], const uint32_t (&dst)[2], int mt, int h) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        buffer_store_b128_guarded<2>(v[i], c_rsrc_tile, c_lane_h[h], c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes + (uint32_t)h * 128u);
+      for (int i = 0; i < 2; ++i) {
+        if constexpr (SCATTER)
+          buffer_store_b128_guarded<2>(v[i], c_rsrc, dst[i] | (c_lane_h[h] & 0x80000000u), (uint32_t)(tn * BN + wn * WN) * 2u + (uint32_t)h * 128u);
+        else
+          buffer_store_b128_guarded<2>(v[i], c_rsrc_tile, c_lane_h[h], c_tile + (uint32_t)(mt * 16 + i * 8) * c_row_bytes + (uint32_t)h * 128u);
+      }
     };
     if (GROUPED || job.kind == WHOLE) {
       // The steps overlap: a step's two reads go out together, the next step is converted and written behind them (the
@@ -755,10 +789,13 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       static_for<NSTEP>([&](auto S) {
         constexpr int st = decltype(S)::value, mt = st / (TN / 4), h = st % (TN / 4);
         v4u_t v[2];
-        read_back(v);
+        uint32_t dst[2];
+        read_back(v, dst, mt);
         if constexpr (st + 1 < NSTEP) stage((st + 1) / (TN / 4), (st + 1) % (TN / 4));
-        store_step(v, mt, h);
+        store_step(v, dst, mt, h);
       });
+      // (the next tile's index entries, behind this tile's stores)
+      if (has_next) dma_idx(next_at.row0);
     } else {
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt) {
@@ -767,8 +804,9 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         for (int h = 0; h < TN / 4; ++h) {
           stage(mt, h);
           v4u_t v[2];
-          read_back(v);
-          store_step(v, mt, h);
+          uint32_t dst[2];
+          read_back(v, dst, mt);
+          store_step(v, dst, mt, h);
         }
       }
     }
@@ -790,10 +828,10 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
   w4_body<TM, TN, BLOCKSCALE, PROBE>(p, smem);
 }
 
-template <int TM, int TN, bool BLOCKSCALE>
+template <int TM, int TN, bool BLOCKSCALE, bool SCATTER>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_w4_grouped_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  w4_body<TM, TN, BLOCKSCALE, 0, true>(p, smem);
+  w4_body<TM, TN, BLOCKSCALE, 0, SCATTER ? 2 : 1>(p, smem);
 }
 
 template <int TM, int TN, bool BLOCKSCALE>
@@ -884,11 +922,11 @@ int gemm_w4_launch(const GemmArgs& p_in, bool blockscale, int tm, bool split, hi
 }
 
 // The grouped form takes: block scaling (the caller's business), bf16 C with 16-byte aligned rows, N a multiple of 8, K a
-// whole and even number of slabs, at most kW4GroupedSlots slots, no row index on C, operands whose byte offsets fit 31
-// bits (per expert, for the weights).
+// whole and even number of slabs, at most kW4GroupedSlots slots, operands whose byte offsets fit 31 bits (per expert, for
+// the weights).
 bool gemm_w4_grouped_ok(const GemmArgs& p) {
   if (p.M < 192 || p.N <= 0 || p.N % 8 != 0 || p.K < 512 || p.K % 256 != 0) return false;
-  if (p.num_active <= 0 || p.num_active > kW4GroupedSlots || p.c_row_index != nullptr) return false;
+  if (p.num_active <= 0 || p.num_active > kW4GroupedSlots) return false;
   if (p.c_dtype != MAXFP8_BF16 || !p.c_vec8_ok) return false;
   const int64_t lim = 0x7ff00000ll, nslab = p.K / 128;
   const int64_t rows = (int64_t)p.M + 192;
@@ -901,12 +939,13 @@ bool gemm_w4_grouped_ok(const GemmArgs& p) {
 // The full 192-row tiles of the slots with at least 192 rows (p.big_rows == p.big_bm == 192); the other launch takes the
 // rest.  A block per CU: the blocks past this launch's share of the chip exit at once.
 int gemm_w4_grouped_launch(const GemmArgs& p, hipStream_t stream) {
-  static PerDeviceFlag attr_done;
+  static PerDeviceFlag attr_done_plain, attr_done_scatter;
   constexpr int lds = w4_lds_bytes<6, 8, true>() + kW4GroupedTableBytes;
-  static_assert(lds <= 160 * 1024, "one block's LDS");
-  const char* name = "gemm_w4_grouped_block_192x256";
-  auto kern = gemm_w4_grouped_kernel<6, 8, true>;
-  bool& done = attr_done.here();
+  static_assert(lds + 64 <= 160 * 1024, "one block's LDS");
+  const bool scatter = p.c_row_index != nullptr;
+  const char* name = scatter ? "gemm_w4_grouped_block_192x256 (row index)" : "gemm_w4_grouped_block_192x256";
+  auto kern = scatter ? gemm_w4_grouped_kernel<6, 8, true, true> : gemm_w4_grouped_kernel<6, 8, true, false>;
+  bool& done = scatter ? attr_done_scatter.here() : attr_done_plain.here();
   if (!done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, lds, hipGetErrorString(e));

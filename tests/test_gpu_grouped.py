@@ -231,6 +231,48 @@ def test_four_wave_launch_beside_the_persistent_one_is_exact(dev, tune):
         assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, ids {ids.tolist()}, N {N}, K {K}"
 
 
+def test_four_wave_launch_with_a_row_index(dev, tune):
+    """The row index on C (row m of the result is stored at row index[m]: the MoE layer's restore of the token order) on
+    the two launches side by side: the four-wave kernel copies the index entries of a tile's rows into LDS and stores
+    each row through them.  Integer data, groupings around the bounds of the rule that shares the rows out, ragged N,
+    skipped experts: equal to the one-launch form's result, and to the result without an index permuted afterwards."""
+    rng = np.random.default_rng(9)
+    for it in range(12):
+        E = int(rng.integers(1, 20))
+        active = int(rng.integers(1, E + 1))
+        counts = rng.choice([0, 5, 33, 129, 191, 192, 193, 225, 385, 1000, 1300], active)
+        ids = rng.permutation(E)[:active].astype(np.int32)
+        ids[rng.random(active) < 0.1] = -1
+        if counts.sum() == 0:
+            counts[0] = 200
+        T = int(counts.sum())
+        N = 8 * int(rng.integers(8, 160)) if it % 2 else 128 * int(rng.integers(1, 12))
+        K = 256 * int(rng.integers(2, 6))
+        a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (T, K)).astype(np.float32))).to(dev)
+        b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (E, N, K)).astype(np.float32))).to(dev)
+        sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (K // 128, -(-T // 4) * 4))).astype(np.float32)).to(dev)
+        sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (E, -(-N // 128), K // 128))).astype(np.float32)).to(dev)
+        off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32).to(dev)
+        idt = torch.tensor(list(ids) + [-1] * (E - active), dtype=torch.int32).to(dev)
+        perm = torch.from_numpy(rng.permutation(T).astype(np.int64)).to(dev)
+        stats = torch.tensor([int(counts.max()), active], dtype=torch.int64).to(torch.uint32)
+
+        def go(index):
+            return mx.grouped_dynamic_scaled_fp8_matmul(a, b, sa, sb, off, idt, stats, BLK.input_scale, BLK.weight_scale,
+                                                        out_type=torch.bfloat16, out_row_index=index)
+
+        tune(MAXFP8_GROUPED_W4=None, MAXFP8_GROUPED_W4_ROWS="0")
+        got, plain = go(perm.to(torch.uint32)), go(None)
+        tune(MAXFP8_GROUPED_W4="0")
+        want = go(perm.to(torch.uint32))
+        torch.cuda.synchronize()
+        what = f"case {it}: counts {counts.tolist()}, ids {ids.tolist()}, N {N}, K {K}"
+        assert torch.equal(got, want), what + ": differs from the one-launch form"
+        back = torch.empty_like(plain)
+        back[perm] = plain
+        assert torch.equal(got, back), what + ": differs from the plain result permuted"
+
+
 def test_four_wave_launch_has_the_bits_of_the_one_launch_form(dev, tune):
     """Random (inexact) data on a skewed routing of 64 experts: both forms add a row's products up in the same order,
     so the two launches side by side give the bits of the one persistent launch -- also with a share of the chip forced
