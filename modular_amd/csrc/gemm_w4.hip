@@ -204,6 +204,11 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       if (keep < 8) keep = 8;
       if (keep > G) keep = G;
       if (keep > R * ncol) keep = (R * ncol + 7) & ~7;
+      // (the tiles are dealt out in whole rounds of the blocks that stay: no more blocks than that number of rounds needs)
+      if (p.share_bias >= 0.f && R > 0) {
+        const int rounds = (R * ncol + keep - 1) / keep;
+        keep = (((R * ncol + rounds - 1) / rounds) + 7) & ~7;
+      }
       hdr[0] = R;
       hdr[1] = R > 0 ? keep : 0;
     }
