@@ -1997,11 +1997,27 @@ static bool w4_shape(int64_t M, int64_t N, int64_t K) { return M > 0 && N > 0 &&
 
 // Which four-wave tile height, if any, beats `other_cost` (microseconds, what the plan made of the eight-wave shapes
 // costs) by at least 3 %, and whether with its tail cut (*split; the workspace has to hold the pieces).
-static int pick_w4(int64_t M, int64_t N, int64_t K, bool blockscale, float other_cost, size_t workspace_bytes, bool* split) {
+//
+// other_splits: the other plan is a K split (two launches, the shares' sums through memory).  Then the matmul is at most
+// half a round of tiles, and the one candidate is the four-wave kernel with EVERY tile cut into pieces, the pieces
+// exchanging their sums inside the one launch: measured ahead where the pieces fill three quarters of the chip and are at
+// least 16 slabs long (512 x 7168 x 16384: 67 against 84 us; 1024 x 2112 x 7168: 30 against 35; 384 x 6144 x 8192: 35
+// against 42; 768 x 2048 x 8192, 16 slabs: 27 against 32), behind with shorter pieces (8 slabs: 25 against 22) and with
+// fewer blocks (128 x 4096 x 14336, 16 tiles in 64 pieces: 38 against 27; 512 x 2048 x 28672, 128 pieces: 64 against 51).
+static int pick_w4(int64_t M, int64_t N, int64_t K, bool blockscale, float other_cost, bool other_splits, size_t workspace_bytes, bool* split) {
   const int forced = tuning().w4, cut = tuning().w4_split;
   *split = false;
   if (forced == 0 || !tuning().persist || !w4_shape(M, N, K)) return 0;
   const int nslab = (int)(K / 128), slots = compute_units();
+  if (other_splits) {
+    const int tm = forced > 0 ? forced : 4;
+    const W4Split sp = gemm_w4_split(M, N, K, tm);
+    if (cut == 0 || sp.unit <= 0 || sp.bytes > workspace_bytes) return 0;
+    if (ceil_div(M, 32 * tm) * ceil_div(N, 256) * 2 > slots) return 0;  // (not the case meant here)
+    if (forced <= 0 && cut != 1 && (sp.unit < 16 || (int64_t)sp.blocks * 4 < (int64_t)slots * 3)) return 0;
+    *split = true;
+    return tm;
+  }
   int best = 0;
   float best_cost = forced > 0 ? 3.0e38f : 0.97f * other_cost;  // (a forced height is taken whatever it costs)
   for (int i = 0; i < 3; ++i) {
@@ -2042,8 +2058,13 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
   if (kv_on && plan.variant != 1) plan.variant = 3;  // the fused QKV kernels exist in the 256 x 256 and 128 x 128 shapes
   const TileShape& t = kShapes[plan.variant - 1];
   const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+  // (wants_split: the shape calls for a K split, whether or not this workspace holds its partial sums -- what the
+  // four-wave kernel's choice below goes by, so that a caller who brings exactly that kernel's bytes gets the same plan
+  // as one who brings more)
+  bool wants_split = false;
   if (has_workspace && batch == 1 && !kv_on) {
     const int sp = pick_splits(tiles, t.slots, nslab);
+    wants_split = sp > 1;
     if (sp > 1 && (size_t)sp * M * N * 4 <= workspace_bytes) plan.splits = sp;
   }
   if (free_choice && batch == 1 && !kv_on && plan.splits == 1 && !tuning().one_region)
@@ -2064,11 +2085,12 @@ static TiledPlan make_plan(int64_t M, int64_t N, int64_t K, bool blockscale, boo
   }
   // the four-wave kernel against whatever the eight-wave shapes make of the matmul (one launch; a forced tile shape other
   // than 256 x 256, a K split, a batch or the fused QKV epilogue keep it out)
-  if (batch == 1 && !kv_on && plan.splits == 1 && !plan.streamk && (free_choice || plan.variant == 1)) {
+  if (batch == 1 && !kv_on && !plan.streamk && (free_choice || plan.variant == 1)) {
     float other = plan.two.axis ? plan.two.cost : region_cost(M, N, nslab, t, blockscale);
     if (!plan.two.axis && persist_shape(M, N, plan.variant))
       other = persistent_cost(tiles, t.slots, (float)nslab * (blockscale ? t.t_slab_block : t.t_slab_row) + tile_overhead(M, N, plan.variant - 1, 1));
-    plan.w4 = pick_w4(M, N, K, blockscale, other, has_workspace ? workspace_bytes : 0, &plan.w4_split);
+    plan.w4 = pick_w4(M, N, K, blockscale, other, wants_split, has_workspace ? workspace_bytes : 0, &plan.w4_split);
+    if (plan.w4) plan.splits = 1;
   }
   return plan;
 }
@@ -2120,9 +2142,12 @@ int gemm_tiled_describe(int64_t M, int64_t N, int64_t K, bool blockscale, bool h
   auto count = [](int64_t m, int64_t n, const TileShape& t) { return (long long)(ceil_div(m, t.bm) * ceil_div(n, t.bn)); };
   // (what a bf16 result with 16-byte aligned rows gets)
   auto how = [](int64_t m, int64_t n, int variant) { return persist_shape(m, n, variant) ? " persistent" : (variant == 4 ? " three-stage" : ""); };
-  if (plan.w4 && plan.w4_split)
-    return snprintf(buf, len, "%dx256 x%lld persistent, four waves, tail cut in pieces of %d slabs", 32 * plan.w4,
-                    (long long)(ceil_div(M, 32 * plan.w4) * ceil_div(N, 256)), gemm_w4_split(M, N, K, plan.w4).unit);
+  if (plan.w4 && plan.w4_split) {
+    const long long n_tiles = (long long)(ceil_div(M, 32 * plan.w4) * ceil_div(N, 256));
+    const W4Split sp = gemm_w4_split(M, N, K, plan.w4);
+    return snprintf(buf, len, "%dx256 x%lld persistent, four waves, %s cut in pieces of %d slabs", 32 * plan.w4, n_tiles,
+                    n_tiles * 2 <= compute_units() ? "every tile" : "tail", sp.unit);
+  }
   if (plan.w4)
     return snprintf(buf, len, "%dx256 x%lld persistent, four waves", 32 * plan.w4, (long long)(ceil_div(M, 32 * plan.w4) * ceil_div(N, 256)));
   if (plan.two.axis && !plan.streamk) {

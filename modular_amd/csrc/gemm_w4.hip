@@ -885,7 +885,20 @@ W4Split gemm_w4_split(int64_t M, int64_t N, int64_t K, int tm) {
   const int64_t tiles = ceil_div(M, 32 * tm) * ceil_div(N, 256), nslab = K / 128;
   int g = (compute_units() / 8) * 8;
   if (g > kW4MaxBlocks) g = kW4MaxBlocks;
-  if (g < 8 || K % 512 != 0 || tiles <= g || tiles % g == 0) return none;
+  if (g < 8 || K % 512 != 0) return none;
+  if (tiles * 2 <= g) {
+    // fewer tiles than half the blocks: every tile is cut, into as many pieces (four at most, of four slabs at least)
+    // as there are blocks for
+    int64_t pieces = g / tiles;
+    if (pieces > kW4MaxPieces) pieces = kW4MaxPieces;
+    if (pieces > nslab / 4) pieces = nslab / 4;
+    if (pieces < 2) return none;
+    const int64_t u = ceil_div(ceil_div(nslab, pieces), 4) * 4;
+    if (u >= nslab) return none;
+    const int64_t blocks = ceil_div(tiles * ceil_div(nslab, u), 8) * 8;
+    return W4Split{(int)blocks, (int)u, (size_t)blocks * 32 * tm * 256 * 4};
+  }
+  if (tiles <= g || tiles % g == 0) return none;
   int64_t pieces = g / (tiles % g);
   if (pieces > 4) pieces = 4;
   if (pieces < 2) return none;

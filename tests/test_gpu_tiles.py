@@ -367,6 +367,53 @@ def test_tail_cut_against_the_uncut_kernel(dev, tune, M, N, K, kind, rows):
             _one_bf16_step_apart(got, want)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 1792, 4096), (384, 2304, 2048), (1024, 2112, 7168), (130, 520, 1024), (256, 7168, 8192)])
+@pytest.mark.parametrize("kind", ["block", "row"])
+@pytest.mark.parametrize("rows", ["4", "5", "6"])
+def test_every_tile_cut_against_the_uncut_kernel(dev, tune, M, N, K, kind, rows):
+    """At most half a round of tiles: where the other plan is a K split (two launches, the shares' sums through memory)
+    the four-wave kernel can cut EVERY tile into two to four pieces, one block each, which exchange their sums inside the
+    one launch.  Forced here wherever the shape allows it (the planner takes it where the pieces fill three quarters of
+    the chip with at least 16 slabs each), against the same kernel uncut: equal on exact data, a bf16 step apart at most
+    elsewhere, the same bits on two launches."""
+    if kind == "row" and K > 4096:
+        pytest.skip("one long-K case is enough")
+    cfg = BLK if kind == "block" else ROW
+    tune(MAXFP8_W4=rows, MAXFP8_W4_SPLIT="1")
+    cut_text = _lib.matmul_describe(M, N, K, kind == "block", True)
+    if "every tile cut" not in cut_text:
+        pytest.skip(f"no such cut at this tile height: {cut_text}")
+    assert "cut" not in _lib.matmul_describe(M, N, K, kind == "block", False)   # no workspace, no pieces
+    for exact in (True, False):
+        ops = _tail_cut_operands(M, N, K, kind, exact, dev)
+        run = lambda: mx.dynamic_scaled_matmul(*ops, cfg.input_scale, cfg.weight_scale, out_type=torch.bfloat16, algo="tiled")
+        tune(MAXFP8_W4=rows, MAXFP8_W4_SPLIT="1", MAXFP8_SPLITK=None)
+        got, again = run(), run()
+        tune(MAXFP8_W4=rows, MAXFP8_W4_SPLIT="0", MAXFP8_SPLITK="1")
+        uncut = _lib.matmul_describe(M, N, K, kind == "block", True)
+        assert "four waves" in uncut and "cut" not in uncut, uncut
+        want = run()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), again.view(torch.int16)), "two launches, two results"
+        if exact:
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        else:
+            _one_bf16_step_apart(got, want)
+    assert _lib.lib().maxfp8_handovers_given_up() == 0
+
+
+def test_planner_cuts_every_tile_where_it_measured_ahead(dev, tune):
+    """The planner's own choice on a shape of the kind (DeepSeek-V3 fused q_a + kv_a at M = 1024): the cut form, and its
+    result against the CPU oracle on sampled rows."""
+    M, N, K = 1024, 2112, 7168
+    assert "every tile cut" in _lib.matmul_describe(M, N, K, True, True)
+    a, b, sa, sb = make_block(M, N, K, seed=5)
+    c = mm(a, b, sa, sb, BLK, dev, out=torch.bfloat16)
+    rows = [0, 127, 128, 500, 1023]
+    ref = oracle_block(a.view(torch.uint8)[rows].view(a.dtype), b, sa[:, rows].contiguous(), sb)
+    assert_rel(f32_np(c[rows]), ref, TOL, f"every tile cut {M}x{N}x{K}")
+
+
 def test_tail_cut_against_the_oracle(dev, tune):
     tune(MAXFP8_W4="5", MAXFP8_W4_SPLIT="1")
     for (M, N, K) in [(2040, 6144, 1024), (2200, 7168, 512)]:

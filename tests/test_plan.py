@@ -23,8 +23,13 @@ def test_single_shapes_and_k_split():
     # 25 to 32 rows: the tiles only where K is long and N narrow
     assert "K split" in _lib.matmul_describe(32, 8192, 28672) and _lib.matmul_describe(24, 8192, 28672) == "skinny"
     assert _lib.matmul_describe(32, 8192, 8192) == "skinny" and _lib.matmul_describe(32, 10240, 16384) == "skinny"
-    with_ws, without = _lib.matmul_describe(256, 7168, 16384), _lib.matmul_describe(256, 7168, 16384, True, False)
+    with_ws, without = _lib.matmul_describe(256, 4096, 14336), _lib.matmul_describe(256, 4096, 14336, True, False)
     assert "K split" in with_ws and "K split" not in without
+    # where the pieces of a K split would fill three quarters of the chip with at least 16 slabs each, the four-wave kernel
+    # cuts every tile and its blocks exchange their sums inside the one launch
+    assert _lib.matmul_describe(256, 7168, 16384) == "128x256 x56 persistent, four waves, every tile cut in pieces of 32 slabs"
+    assert "K split" in _lib.matmul_describe(1536, 1024, 4096) and "K split" in _lib.matmul_describe(512, 2048, 28672)
+    assert _lib.lib().maxfp8_matmul_workspace_bytes(256, 7168, 16384) >= 224 * 128 * 256 * 4
     assert _lib.matmul_describe(0, 10, 10) == "nothing to do"
 
 
