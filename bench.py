@@ -354,6 +354,76 @@ def moe_layer_ms(steps, fuse):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def moe_routings(steps):
+    """The grouped block-scaled matmul (DeepSeek-V3's two MoE shapes, 256 experts, top-8) over several routings -- the
+    skew of the experts' popularity and the number of tokens -- in both of its forms: the four-wave launch beside the
+    persistent one (the default) and one persistent launch (MAXFP8_GROUPED_W4=0), interleaved in one process.  Yields one
+    record per (shape, routing): microseconds per matmul from a pair of HIP events around `steps` launches, after 0.3 s
+    of the same launches."""
+    import torch
+    import modular_amd as mx
+    from modular_amd import _lib, synth
+
+    dev = torch.device("cuda:0")
+    cfg = mx.blockwise_fp8_config()
+    E = 256
+
+    def form(two_launches):
+        if two_launches:
+            os.environ.pop("MAXFP8_GROUPED_W4", None)
+        else:
+            os.environ["MAXFP8_GROUPED_W4"] = "0"
+        _lib.tuning_reload()
+
+    def timed(fn):
+        t_end = time.perf_counter() + 0.3
+        while time.perf_counter() < t_end:
+            fn()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps * 1e3
+
+    before = os.environ.get("MAXFP8_GROUPED_W4")
+    try:
+        for proj, N, K in (("gate_up", 4096, 7168), ("down", 7168, 2048)):
+            w = synth.random_fp8((E, N, K), 1, device=dev)
+            ws = synth.random_scales((E, N // 128, K // 128), 2, device=dev, lo=0.001, hi=0.01)
+            for tokens, zipf in ((4096, 1.1), (4096, 0.0), (4096, 0.5), (4096, 2.0), (1024, 1.1), (512, 1.1), (16384, 1.1), (8192, 0.0)):
+                off, ids, counts, stats = synth.moe_routing(tokens, E, 8, seed=0, zipf_a=zipf, device=dev)
+                T = int(counts.sum())
+                a = synth.random_fp8((T, K), 3, device=dev)
+                sa = synth.random_scales((K // 128, T), 4, device=dev, lo=0.01, hi=0.1)
+
+                def fn():
+                    return mx.grouped_dynamic_scaled_fp8_matmul(a, w, sa, ws, off, ids, stats, cfg.input_scale, cfg.weight_scale)
+
+                us = {}
+                for rep in range(2):  # (interleaved: one launch, two launches, and again; the second pair is reported)
+                    for two in (False, True):
+                        form(two)
+                        us[two] = timed(fn)
+                c = counts.tolist()
+                yield {"projection": proj, "N": N, "K": K, "tokens": tokens, "zipf": zipf, "rows": T, "active_experts": sum(x > 0 for x in c),
+                       "largest_expert": max(c), "experts_with_192_rows_or_more": sum(x >= 192 for x in c),
+                       "one_launch_us": round(us[False], 1), "two_launches_us": round(us[True], 1),
+                       "two_over_one": round(us[True] / us[False], 3)}
+                del a, sa
+                torch.cuda.empty_cache()
+            del w, ws
+            torch.cuda.empty_cache()
+    finally:
+        if before is None:
+            os.environ.pop("MAXFP8_GROUPED_W4", None)
+        else:
+            os.environ["MAXFP8_GROUPED_W4"] = before
+        _lib.tuning_reload()
+
+
 def read_ceiling(wl, steps):
     """Average time of the decode matmul's read-only probe (the same grid, LDS ring and DMA instructions streaming
     the same weight copies, nothing else) over `steps` back-to-back launches, in milliseconds."""
@@ -673,6 +743,10 @@ def main():
                     help="the expert matmuls of the FP8 MoE layer on configs[4]'s routing (grouping, gathered quantise, grouped "
                          "gate_up, silu * up, quantise, grouped down): milliseconds per call, one JSON line for each way of the "
                          "activation quantisation (two kernels, one kernel)")
+    ap.add_argument("--moe-routings", action="store_true",
+                    help="the grouped block-scaled matmul of DeepSeek-V3's two MoE shapes over several routings (skew, number of "
+                         "tokens), as the four-wave launch beside the persistent one and as one persistent launch: one JSON line "
+                         "per shape and routing")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="the dense kernels' main loops on operands that stay on the chip (LDS-resident: MFMA loop alone and "
                          "with promotions; L2-resident: with copies and barriers), one JSON line each: the issue ceiling the "
@@ -733,6 +807,10 @@ def main():
                               "fuse_activation_quant": fuse, "ms_per_call": round(ms, 4), "steps": args.steps,
                               "timing": "host clock around the calls, no host synchronisation inside a call"}), flush=True)
             torch.cuda.empty_cache()
+        return
+    if args.moe_routings:
+        for rec in moe_routings(min(args.steps, 30)):
+            print(json.dumps(rec), flush=True)
         return
     if args.mfma_ceiling:
         for rec in mfma_ceiling():
