@@ -229,6 +229,19 @@ def test_four_wave_launch_beside_the_persistent_one_is_exact(dev, tune):
         got = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=torch.bfloat16, fill=None)
         want = run(a, b, sa, sb, off, idt, int(counts.max()), active, dev, out=torch.bfloat16, algo="naive")
         assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, ids {ids.tolist()}, N {N}, K {K}"
+    # a slot of more than 24 row tiles (its tiles are walked in groups of 12 row tiles) between small ones
+    tune(MAXFP8_GROUPED_W4_ROWS="0", MAXFP8_GROUPED_W4_HOT_REST=None, MAXFP8_GROUPED_W4_COLD_ROWS=None)
+    counts, N, K = np.array([40, 5003, 200, 7]), 776, 512
+    T = int(counts.sum())
+    a = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (T, K)).astype(np.float32)))
+    b = fp8_from_bytes(oracle.e4m3fn_encode(rng.integers(-4, 5, (4, N, K)).astype(np.float32)))
+    sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (K // 128, -(-T // 4) * 4))).astype(np.float32))
+    sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, (4, -(-N // 128), K // 128))).astype(np.float32))
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)).to(torch.uint32)
+    idt = torch.tensor([2, 0, 3, 1], dtype=torch.int32)
+    got = run(a, b, sa, sb, off, idt, 5003, 4, dev, out=torch.bfloat16)
+    want = run(a, b, sa, sb, off, idt, 5003, 4, dev, out=torch.bfloat16, algo="naive")
+    assert torch.equal(got, want), "a slot of 27 row tiles"
 
 
 def test_four_wave_launch_with_a_row_index(dev, tune):
