@@ -1696,8 +1696,8 @@ static bool persist_ok(const GemmArgs& p, bool blockscale, dim3 grid) {
 
 // The four-wave kernel (gemm_w4.hip): 0 (no), or the sixteen-row groups per wave -- 5: tiles of 160 x 256, 6: 192 x 256.
 bool gemm_w4_ok(const GemmArgs& p, bool blockscale);
-bool gemm_w4_grouped_ok(const GemmArgs& p);
-int gemm_w4_grouped_launch(const GemmArgs& p, hipStream_t stream);
+bool gemm_w4_grouped_ok(const GemmArgs& p, bool blockscale);
+int gemm_w4_grouped_launch(const GemmArgs& p, bool blockscale, hipStream_t stream);
 int gemm_w4_launch(const GemmArgs& p, bool blockscale, int tm, bool split, hipStream_t stream);
 W4Split gemm_w4_split(int64_t M, int64_t N, int64_t K, int tm);
 
@@ -2299,12 +2299,12 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int6
   // `grouped_persist` = 0 goes back to the two launches below).
   if (tuning().grouped_persist && !big && p.num_active <= kGroupedMaxSlots) {
     p.share_bias = tuning().grouped_share * 2.0f;
-    // Block scaling, a slot of more than 128 rows possible, and enough rows for it to matter: every slot's full 192-row
+    // A slot of more than 128 rows possible, and enough rows for it to matter: every slot's full 192-row
     // tiles, and a rest of more than 128 rows, go to the four-wave kernel (a quarter faster per row than the L tiles
     // below on the matrix pipe, twice as fast as the M2 tiles), which is issued first on the caller's stream; the
     // persistent launch takes the rests of at most 128 rows down the second stream.  How the
     // CUs are shared is decided on the device, where the group sizes are (see gemm_w4.hip).
-    if (blockscale && tuning().grouped_w4 && tune != 4 && max_tokens > tuning().grouped_w4_cold_rows && T >= tuning().grouped_w4_rows && gemm_w4_grouped_ok(p)) {
+    if (tuning().grouped_w4 && tune != 4 && max_tokens > tuning().grouped_w4_cold_rows && T >= tuning().grouped_w4_rows && gemm_w4_grouped_ok(p, blockscale)) {
       SideStream* side = side_stream();
       if (side) {
         std::unique_lock<std::mutex> side_lock(side->mu);  // one fork / join at a time per device
@@ -2317,10 +2317,11 @@ int gemm_grouped_dispatch(const GemmArgs& p_in, bool blockscale, int64_t T, int6
           MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "grouped matmul: cannot order the second stream behind the caller's: %s", hipGetErrorString(hipGetLastError()));
         GemmArgs ph = p;
         ph.share_bias = tuning().grouped_w4_share < 0.f ? tuning().grouped_w4_share : p.share_bias * tuning().grouped_w4_share;
-        int rc = gemm_w4_grouped_launch(ph, stream);
+        int rc = gemm_w4_grouped_launch(ph, blockscale, stream);
         if (rc == MAXFP8_OK) {
           p.heads_elsewhere = 1;
-          rc = launch_grouped_persist<true>(p, side->stream, "gemm_grouped_persist_block");
+          rc = blockscale ? launch_grouped_persist<true>(p, side->stream, "gemm_grouped_persist_block")
+                          : launch_grouped_persist<false>(p, side->stream, "gemm_grouped_persist_row");
         }
         if ((hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(stream, side->join, 0) != hipSuccess) && rc == MAXFP8_OK)
           MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "grouped matmul: cannot join the second stream: %s", hipGetErrorString(hipGetLastError()));

@@ -99,7 +99,7 @@ static __device__ unsigned int g_w4_gave_up;
 // slabs 0..7 over and over, so that its operands stay in L2; 2 the same without copies, waits and barriers -- the
 // MFMA loop on what the prologue left in LDS.
 //
-// GROUPED (the MoE matmul, block scaling; BM = 192): the tiles are those of w4_grouped_head_rows of every slot -- its full
+// GROUPED (the MoE matmul; BM = 192): the tiles are those of w4_grouped_head_rows of every slot -- its full
 // BM-row tiles and one more for a rest of more than 128 rows, stored up to the slot's end --
 // numbered through all slots as if they were the row tiles of one matrix: row tile v lies in the slot
 // found by bisection in a prefix table that every block builds in LDS from the device-resident offsets, and its weights
@@ -136,7 +136,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   static_assert(PER_B + NSTORE < 64, "the count must fit the vmcnt field");
   static_assert(IB % 2 == 0, "the weight copies go out in two halves");
 
-  static_assert(!GROUPED || (BLOCKSCALE && PROBE == 0), "the grouped form is built for block scaling");
+  static_assert(!GROUPED || PROBE == 0, "the probe runs the dense form");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -719,10 +719,11 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       for (int q = 0; q < TN / 2; ++q)
 #pragma unroll
         for (int i = 0; i < 8; ++i)
-          b_s[q][i] = scale_at(p.b_scales, (int64_t)min(tn * BN + wn * WN + q * 32 + lq * 8 + i, p.N - 1) * p.b_scale_stride, p.scales_dtype);
+          b_s[q][i] = scale_at(p.b_scales, (int64_t)cur_at.bs0 + (int64_t)min(tn * BN + wn * WN + q * 32 + lq * 8 + i, p.N - 1) * p.b_scale_stride,
+                               p.scales_dtype);  // (grouped: bs0 = where the expert's scales begin)
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt) {
-        int64_t m = (int64_t)tm * BM + wm * WM + mt * 16 + lm;
+        int64_t m = (int64_t)cur_at.row0 + wm * WM + mt * 16 + lm;
         if (m >= p.M) m = p.M - 1;
         a_s_all[mt] = scale_at(p.a_scales, m * p.a_scale_stride, p.scales_dtype);
       }
@@ -842,6 +843,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
 
 template <int TM, int TN, bool BLOCKSCALE, bool SCATTER>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_w4_grouped_kernel(GemmArgs p) {
+  static_assert(BLOCKSCALE || !SCATTER, "the row index on C is the block-scaled MoE layer's");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   w4_body<TM, TN, BLOCKSCALE, 0, SCATTER ? 2 : 1>(p, smem);
 }
@@ -946,31 +948,36 @@ int gemm_w4_launch(const GemmArgs& p_in, bool blockscale, int tm, bool split, hi
   return blockscale ? launch_w4<6, true, 0>(p, blocks, stream, "gemm_w4_block_192x256") : launch_w4<6, false, 0>(p, blocks, stream, "gemm_w4_row_192x256");
 }
 
-// The grouped form takes: block scaling (the caller's business), bf16 C with 16-byte aligned rows, N a multiple of 8, K a
-// whole and even number of slabs, at most kW4GroupedSlots slots, operands whose byte offsets fit 31 bits (per expert, for
-// the weights).
-bool gemm_w4_grouped_ok(const GemmArgs& p) {
+// The grouped form takes: bf16 C with 16-byte aligned rows, N a multiple of 8, K a whole and even number of slabs, at most
+// kW4GroupedSlots slots, operands whose byte offsets fit 31 bits (per expert, for the weights); row scaling: f32 scales,
+// no row index on C.
+bool gemm_w4_grouped_ok(const GemmArgs& p, bool blockscale) {
+  if (!blockscale && (p.c_row_index != nullptr || p.scales_dtype != MAXFP8_F32)) return false;
   if (p.M < 192 || p.N <= 0 || p.N % 8 != 0 || p.K < 512 || p.K % 256 != 0) return false;
   if (p.num_active <= 0 || p.num_active > kW4GroupedSlots) return false;
   if (p.c_dtype != MAXFP8_BF16 || !p.c_vec8_ok) return false;
   const int64_t lim = 0x7ff00000ll, nslab = p.K / 128;
   const int64_t rows = (int64_t)p.M + 192;
   if (rows * p.lda >= lim || (ceil_div(p.N, 256) * 256) * p.ldb >= lim) return false;
-  if ((nslab * p.a_scales_ld + rows) * 4 >= lim || rows * p.ldc * 2 >= lim) return false;
-  if ((int64_t)p.num_active * p.bs_expert_stride + (ceil_div(p.N, 128) + 1) * p.b_scales_ld >= lim / 4) return false;
+  if (rows * p.ldc * 2 >= lim) return false;
+  if (blockscale && (nslab * p.a_scales_ld + rows) * 4 >= lim) return false;
+  // (the element of the weight scales where an expert's begin rides in 32 bits: fine for expert numbers below 2^16 with
+  // fewer than 2^15 scales per expert)
+  if (p.bs_expert_stride >= (1 << 15)) return false;
   return true;
 }
 
 // The full 192-row tiles of the slots with at least 192 rows (p.big_rows == p.big_bm == 192); the other launch takes the
 // rest.  A block per CU: the blocks past this launch's share of the chip exit at once.
-int gemm_w4_grouped_launch(const GemmArgs& p, hipStream_t stream) {
-  static PerDeviceFlag attr_done_plain, attr_done_scatter;
-  constexpr int lds = w4_lds_bytes<6, 8, true>() + kW4GroupedTableBytes;
+int gemm_w4_grouped_launch(const GemmArgs& p, bool blockscale, hipStream_t stream) {
+  static PerDeviceFlag attr_done_plain, attr_done_scatter, attr_done_row;
+  constexpr int lds = w4_lds_bytes<6, 8, true>() + kW4GroupedTableBytes;  // (the row-scaled kernel takes the same, for simplicity)
   static_assert(lds + 64 <= 160 * 1024, "one block's LDS");
   const bool scatter = p.c_row_index != nullptr;
-  const char* name = scatter ? "gemm_w4_grouped_block_192x256 (row index)" : "gemm_w4_grouped_block_192x256";
-  auto kern = scatter ? gemm_w4_grouped_kernel<6, 8, true, true> : gemm_w4_grouped_kernel<6, 8, true, false>;
-  bool& done = scatter ? attr_done_scatter.here() : attr_done_plain.here();
+  const char* name = !blockscale ? "gemm_w4_grouped_row_192x256" : (scatter ? "gemm_w4_grouped_block_192x256 (row index)" : "gemm_w4_grouped_block_192x256");
+  auto kern = !blockscale ? gemm_w4_grouped_kernel<6, 8, false, false>
+                          : (scatter ? gemm_w4_grouped_kernel<6, 8, true, true> : gemm_w4_grouped_kernel<6, 8, true, false>);
+  bool& done = !blockscale ? attr_done_row.here() : (scatter ? attr_done_scatter.here() : attr_done_plain.here());
   if (!done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) MAXFP8_FAIL(MAXFP8_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, lds, hipGetErrorString(e));

@@ -131,3 +131,31 @@ def test_block_and_row_scaled_launches_in_flight_together(dev):
     for i, (gb, gr) in enumerate(zip(got_b, got_r)):
         assert torch.equal(gb[:live], want_b[:live]), f"block-scaled launch {i}"
         assert torch.equal(gr[:live], want_r[:live]), f"row-scaled launch {i}"
+
+
+def test_four_wave_launch_beside_the_persistent_one(dev, tune):
+    """Row scaling on the two launches side by side (the slots' full 192-row tiles and the rests behind them on the grouped
+    form of the four-wave kernel, the other rows on the persistent launch): the bits of the one persistent launch
+    (MAXFP8_GROUPED_W4=0) on a sweep of groupings around the bounds of the rule that shares the rows out, with a skipped
+    expert, rows past the last slot and a ragged N; one of them against the oracle."""
+    rng = np.random.default_rng(21)
+    for it in range(10):
+        E = int(rng.integers(2, 14))
+        active = int(rng.integers(1, E + 1))
+        counts = rng.choice([0, 5, 33, 128, 129, 191, 192, 193, 225, 385, 700, 1300], active)
+        ids = rng.permutation(E)[:active].astype(np.int32)
+        if active > 1 and it % 3 == 0:
+            ids[int(rng.integers(0, active))] = -1
+        if counts.sum() == 0:
+            counts[0] = 200
+        N = 8 * int(rng.integers(8, 120)) if it % 2 else 128 * int(rng.integers(1, 9))
+        K = 256 * int(rng.integers(2, 6))
+        args = make(list(counts), list(ids), E, N, K, seed=it, extra_rows=int(it % 4 == 0) * 5)
+        tune(MAXFP8_GROUPED_W4=None, MAXFP8_GROUPED_W4_ROWS="0")
+        got = run(*args, int(counts.max()), active, dev, out=torch.bfloat16)
+        tune(MAXFP8_GROUPED_W4="0")
+        want = run(*args, int(counts.max()), active, dev, out=torch.bfloat16)
+        live = int(counts.sum())
+        assert torch.equal(got[:live], want[:live]), f"case {it}: counts {counts.tolist()}, ids {ids.tolist()}, N {N}, K {K}"
+        if it == 1:
+            assert_rel(f32_np(got)[:live], ref(*args, active)[:live], TOL, "grouped rowwise, two launches")
