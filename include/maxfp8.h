@@ -381,6 +381,7 @@ int maxfp8_grouped_matmul_dynamic_scaled_fp8_scatter(
  *   a [T, K], b [num_experts, N, K] e4m3fn contiguous; a_scales [T, 1], b_scales [num_experts, N, 1] f32;
  *   expert_start_indices, expert_ids, max_num_tokens_per_expert, num_active_experts as in
  *   maxfp8_grouped_matmul_dynamic_scaled_fp8.  Needs K % 16 == 0 and 16-byte aligned a, b.
+ * Launches as that entry point does (a large matmul: two launches side by side, joined on `stream`).
  */
 int maxfp8_grouped_matmul_rowwise_dynamic_scaled_fp8(
     void* c, const void* a, const void* b, const void* a_scales, const void* b_scales,
