@@ -143,8 +143,10 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   const int lm = lane & 15, lq = lane >> 4;
   const int nslab = p.K / 128;                               // whole slabs, an even number of them (the host's rule)
 
-  // ---- grouped: the tables (behind the side buffers).  hdr[0] = row tiles of all slots, hdr[1] = the blocks that stay;
-  // tab_tiles[z] = row tiles in the slots before z, tab_begin[z] = slot z's first row, tab_expert[z] = its expert.
+  // ---- grouped: the tables (behind the side buffers).  hdr[0] = row tiles of all slots, hdr[1] = the blocks that stay,
+  // hdr[3] / hdr[4] = the other launch's row tiles (rests of more than small_rows rows / of fewer), hdr[8..11] = the
+  // waves' sums of the scan; tab_tiles[z] = row tiles in the slots before z, tab_begin[z] / tab_end[z] = slot z's rows,
+  // tab_expert[z] = its expert; then, per wave, the index entries of a tile's rows (GROUPED == 2).
   int* const hdr = reinterpret_cast<int*>(smem + SIDE_BASE + 4 * SIDE_BYTES);
   int* const tab_tiles = hdr + 16;                     // (kW4GroupedSlots + 1 entries: the last is the total)
   int* const tab_begin = tab_tiles + kW4GroupedSlots + 8;
@@ -195,12 +197,16 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
       const int R = before + incl;
       const float ns = (float)nslab;
       const int ncol = (p.N + BN - 1) / BN;
+      // (microseconds of one CU: this launch's tiles; the other launch's 128 x 256 tiles and its weight-streaming tiles of
+      // 512 columns, as its own blocks price them)
+      // (row scaling: the same figure although its tiles are a seventh faster -- priced at 1.0 the launch kept fewer
+      // blocks and the pair took 805 instead of 750 microseconds on the 7168 x 2048 shape)
       const float w_here = (float)(R * ncol) * (ns * 1.15f + 3.0f);
-      const float w_there = (float)(hdr[2] * ((p.N + 127) / 128) + hdr[3] * ((p.N + 255) / 256)) * (ns * 0.92f + 9.0f) +
+      const float w_there = (float)(hdr[3] * ((p.N + 255) / 256)) * (ns * 0.92f + 9.0f) +
                             (float)(hdr[4] * ((p.N + 511) / 512)) * (ns * 2.6f + 6.0f) * p.share_bias;
       const int G = (int)gridDim.x & ~7;
       int keep = (int)((float)G * w_here / (w_here + w_there + 1e-9f) + 4.0f) & ~7;
-      if (p.share_bias < 0.f) keep = (int)(-p.share_bias) & ~7;
+      if (p.share_bias < 0.f) keep = (int)(-p.share_bias) & ~7;  // (tuning runs: the number itself)
       if (keep < 8) keep = 8;
       if (keep > G) keep = G;
       if (keep > R * ncol) keep = (R * ncol + 7) & ~7;
