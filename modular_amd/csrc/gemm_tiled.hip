@@ -2014,7 +2014,13 @@ static int pick_w4(int64_t M, int64_t N, int64_t K, bool blockscale, float other
     const W4Split sp = gemm_w4_split(M, N, K, tm);
     if (cut == 0 || sp.unit <= 0 || sp.bytes > workspace_bytes) return 0;
     if (ceil_div(M, 32 * tm) * ceil_div(N, 256) * 2 > slots) return 0;  // (not the case meant here)
-    if (forced <= 0 && cut != 1 && (sp.unit < 16 || (int64_t)sp.blocks * 4 < (int64_t)slots * 3)) return 0;
+    // (more than four pieces only where they are long: 128 x 8192 x 28672 in eight pieces of 28 slabs 59 against 64 us,
+    // 512 x 2048 x 28672 46 against 52; in eight of 16 slabs 128 x 8192 x 16384 47 against 41.  And only where the rows
+    // fill three quarters of the 128-row tiles: 48 ... 64 rows on 8192 x 28672 took 56 against 48 ... 51.)
+    const int64_t pieces = ceil_div(nslab, sp.unit), rows_padded = ceil_div(M, 32 * tm) * 32 * tm;
+    if (forced <= 0 && cut != 1 &&
+        (sp.unit < (pieces > 4 ? 24 : 16) || (int64_t)sp.blocks * 4 < (int64_t)slots * 3 || M * 4 < rows_padded * 3))
+      return 0;
     *split = true;
     return tm;
   }

@@ -91,7 +91,7 @@ constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) { return (vmcnt & 15) | ((vmcn
 // block and reader (a tile has at most kW4MaxPieces pieces).  A flag is raised by the block that wrote its sums and put
 // back to zero by the one block it is meant for, so a launch leaves its set as it found it.  And the count of pieces a
 // block gave up waiting for.
-constexpr int kW4FlagSets = 64, kW4MaxBlocks = 512, kW4MaxPieces = 4;
+constexpr int kW4FlagSets = 64, kW4MaxBlocks = 512, kW4MaxPieces = 8;
 static __device__ unsigned int g_w4_flags[kW4FlagSets * kW4MaxBlocks * kW4MaxPieces];
 static __device__ unsigned int g_w4_gave_up;
 
@@ -235,7 +235,7 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
   // other's operands in their L2.
   //
   // A job: slabs [s0, s1) of a tile.  WHOLE: all of them, the tile is stored.  PIECE: one of the P pieces of a tail tile.
-  // The P blocks of a tile share its rows out between them (16-row group mt of every wave belongs to piece mt P / TM):
+  // The P blocks of a tile share its rows out between them (step st of every wave's epilogue -- 16 rows x 64 columns -- belongs to piece st P / (2 TM)):
   // a block writes the sums of the other blocks' rows to its slot of the workspace, raises a flag for each of them, then
   // waits for theirs, adds their sums of its own rows to its own (own first, then the others in the order of their
   // slabs: the same order on every launch) and stores those rows of the tile.  Nobody waits before it has published, so
@@ -648,14 +648,15 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         out[1] = wall_clock64() - probe_r0;
       }
     }
-    // the 16-row groups of a wave that this block converts and stores: all of them, or its share of a tail tile
-    int mt_lo = 0, mt_hi = TM;
+    // the steps of the epilogue (16 rows x 64 columns of a wave's part: step = 2 * group of rows + half of the columns)
+    // that this block converts and stores: all of them, or its share of a tile that is cut
+    int st_lo = 0, st_hi = 2 * TM;
     if (!GROUPED && job.kind == PIECE) {
       const Plan pl = plan_of();
       const int tail_c = pl.tail_c, T = total - pl.main_total, P = (nslab + pl.tail_u - 1) / pl.tail_u;
       const int q = tail_c / T, t = tail_c - q * T;
-      mt_lo = q * TM / P;
-      mt_hi = (q + 1) * TM / P;
+      st_lo = q * (2 * TM) / P;
+      st_hi = (q + 1) * (2 * TM) / P;
       const __amdgpu_buffer_rsrc_t w_rsrc = t2_rsrc(p.workspace, t2_clamp_u32((int64_t)gridDim.x * SLOT_BYTES));
       // (a flag per block and reader: the reader puts it down again)
       unsigned int* const flags = g_w4_flags + (size_t)p.streamk_slot * (kW4MaxBlocks * kW4MaxPieces);
@@ -665,9 +666,9 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         const uint32_t base = (uint32_t)tail_c * SLOT_BYTES + (uint32_t)wave * (SLOT_BYTES / 4);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-          if (i >= mt_lo && i < mt_hi) continue;
 #pragma unroll
           for (int j = 0; j < TN; ++j) {
+            if (2 * i + j / 4 >= st_lo && 2 * i + j / 4 < st_hi) continue;
             const v4f a4 = acc[i][j];
             const v4u_t v = {__float_as_uint(a4[0]), __float_as_uint(a4[1]), __float_as_uint(a4[2]), __float_as_uint(a4[3])};
             buffer_store_b128_guarded<kDeviceScope>(v, w_rsrc, (uint32_t)lane_p * 16u, base + (uint32_t)(i * TN + j) * 1024u);
@@ -703,16 +704,17 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
         const uint32_t base = (uint32_t)c * SLOT_BYTES + (uint32_t)wave * (SLOT_BYTES / 4);
         const uint32_t poison = there ? 0u : 0x7fc00000u;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          if (i < mt_lo || i >= mt_hi) continue;
-          v4u_t v[TN];
+        for (int st = 0; st < 2 * TM; ++st) {
+          if (st < st_lo || st >= st_hi) continue;
+          const int i = st / 2, j0 = (st & 1) * 4;
+          v4u_t v[4];
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            v[j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (uint32_t)lane_p * 16u, base + (uint32_t)(i * TN + j) * 1024u, kDeviceScope);
+          for (int j = 0; j < 4; ++j)
+            v[j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (uint32_t)lane_p * 16u, base + (uint32_t)(i * TN + j0 + j) * 1024u, kDeviceScope);
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] += v4f{__uint_as_float(v[j].x | poison), __uint_as_float(v[j].y | poison), __uint_as_float(v[j].z | poison),
-                             __uint_as_float(v[j].w | poison)};
+          for (int j = 0; j < 4; ++j)
+            acc[i][j0 + j] += v4f{__uint_as_float(v[j].x | poison), __uint_as_float(v[j].y | poison), __uint_as_float(v[j].z | poison),
+                                  __uint_as_float(v[j].w | poison)};
         }
       }
     }
@@ -818,9 +820,9 @@ __device__ __forceinline__ void w4_body(const GemmArgs& p, uint8_t* smem) {
     } else {
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt) {
-        if (mt < mt_lo || mt >= mt_hi) continue;   // (a piece of a tail tile: the other rows are another block's)
 #pragma unroll
         for (int h = 0; h < TN / 4; ++h) {
+          if (2 * mt + h < st_lo || 2 * mt + h >= st_hi) continue;   // (a piece of a cut tile: the other steps are another block's)
           stage(mt, h);
           v4u_t v[2];
           uint32_t dst[2];
@@ -902,8 +904,8 @@ W4Split gemm_w4_split(int64_t M, int64_t N, int64_t K, int tm) {
   if (g > kW4MaxBlocks) g = kW4MaxBlocks;
   if (g < 8 || K % 512 != 0) return none;
   if (tiles * 2 <= g) {
-    // fewer tiles than half the blocks: every tile is cut, into as many pieces (four at most, of four slabs at least)
-    // as there are blocks for
+    // fewer tiles than half the blocks: every tile is cut, into as many pieces (eight at most -- a piece owns at least
+    // one of the 2 tm steps of the epilogue --, of four slabs at least) as there are blocks for
     int64_t pieces = g / tiles;
     if (pieces > kW4MaxPieces) pieces = kW4MaxPieces;
     if (pieces > nslab / 4) pieces = nslab / 4;

@@ -367,12 +367,12 @@ def test_tail_cut_against_the_uncut_kernel(dev, tune, M, N, K, kind, rows):
             _one_bf16_step_apart(got, want)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 1792, 4096), (384, 2304, 2048), (1024, 2112, 7168), (130, 520, 1024), (256, 7168, 8192)])
+@pytest.mark.parametrize("M,N,K", [(256, 1792, 4096), (384, 2304, 2048), (1024, 2112, 7168), (130, 520, 1024), (256, 7168, 8192), (128, 1024, 8192)])
 @pytest.mark.parametrize("kind", ["block", "row"])
 @pytest.mark.parametrize("rows", ["4", "5", "6"])
 def test_every_tile_cut_against_the_uncut_kernel(dev, tune, M, N, K, kind, rows):
     """At most half a round of tiles: where the other plan is a K split (two launches, the shares' sums through memory)
-    the four-wave kernel can cut EVERY tile into two to four pieces, one block each, which exchange their sums inside the
+    the four-wave kernel can cut EVERY tile into two to eight pieces, one block each, which exchange their sums inside the
     one launch.  Forced here wherever the shape allows it (the planner takes it where the pieces fill three quarters of
     the chip with at least 16 slabs each), against the same kernel uncut: equal on exact data, a bf16 step apart at most
     elsewhere, the same bits on two launches."""

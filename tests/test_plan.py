@@ -28,7 +28,10 @@ def test_single_shapes_and_k_split():
     # where the pieces of a K split would fill three quarters of the chip with at least 16 slabs each, the four-wave kernel
     # cuts every tile and its blocks exchange their sums inside the one launch
     assert _lib.matmul_describe(256, 7168, 16384) == "128x256 x56 persistent, four waves, every tile cut in pieces of 32 slabs"
-    assert "K split" in _lib.matmul_describe(1536, 1024, 4096) and "K split" in _lib.matmul_describe(512, 2048, 28672)
+    # (not with pieces of 8 slabs, not with eight pieces of 16, not where the rows fill less than three quarters of the tiles)
+    assert "K split" in _lib.matmul_describe(1536, 1024, 4096) and "K split" in _lib.matmul_describe(128, 8192, 16384)
+    assert "K split" in _lib.matmul_describe(48, 8192, 28672)
+    assert _lib.matmul_describe(512, 2048, 28672) == "128x256 x32 persistent, four waves, every tile cut in pieces of 28 slabs"
     assert _lib.lib().maxfp8_matmul_workspace_bytes(256, 7168, 16384) >= 224 * 128 * 256 * 4
     assert _lib.matmul_describe(0, 10, 10) == "nothing to do"
 
