@@ -343,7 +343,7 @@ int maxfp8_fused_qkv_matmul_ragged_paged_scale(
  *                         => no-op.  max_num_tokens_per_expert is an upper bound
  *                         used only to bound the launch.
  *
- * Enqueued on `stream`; a large matmul (T >= 2048, bf16 c) runs as two launches side by side,
+ * Enqueued on `stream`; a large matmul (T >= 4096, bf16 c) runs as two launches side by side,
  * one of them on a stream the library keeps per device, ordered behind `stream` by an event
  * and joined to it by another before the call returns: work enqueued on `stream` afterwards
  * sees all of c.  Nothing is allocated per call; the call records into a HIP graph.

@@ -145,7 +145,7 @@ static const Tuning* read_tuning(unsigned generation) {
   const char* sb = getenv("MAXFP8_GROUPED_SHARE");
   t->grouped_share = sb ? (float)atof(sb) : 0.5f;
   t->grouped_w4 = num("MAXFP8_GROUPED_W4", 1) != 0;
-  t->grouped_w4_rows = num("MAXFP8_GROUPED_W4_ROWS", 2048);
+  t->grouped_w4_rows = num("MAXFP8_GROUPED_W4_ROWS", 4096);
   const char* sw = getenv("MAXFP8_GROUPED_W4_SHARE");
   t->grouped_w4_share = sw ? (float)atof(sw) : 0.6f;
   t->grouped_w4_hot_rest = num("MAXFP8_GROUPED_W4_HOT_REST", 32);

@@ -40,7 +40,7 @@ struct Tuning {
   // value is the number of blocks that stay, outright: -160 keeps 160); which rows go to the four-wave launch beside the
   // full 192-row tiles (MAXFP8_GROUPED_W4_HOT_REST, MAXFP8_GROUPED_W4_COLD_ROWS: see w4_grouped_head_rows).
   bool grouped_w4 = true;
-  int grouped_w4_rows = 2048;
+  int grouped_w4_rows = 4096;
   float grouped_w4_share = 0.6f;
   int grouped_w4_hot_rest = 32, grouped_w4_cold_rows = 128;
   int skinny = 0;
