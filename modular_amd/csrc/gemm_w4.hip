@@ -99,7 +99,9 @@ static __device__ unsigned int g_w4_gave_up;
 // slabs 0..7 over and over, so that its operands stay in L2; 2 the same without copies, waits and barriers -- the
 // MFMA loop on what the prologue left in LDS.
 //
-// GROUPED (the MoE matmul; BM = 192): the tiles are those of w4_grouped_head_rows of every slot -- its full
+// GROUPED (the MoE matmul -- rows sorted by expert, slot z = rows [offsets[z], offsets[z + 1]) times the weights of expert
+// expert_ids[z], zeros where that is -1: max/kernels/src/linalg/grouped_matmul_sm100_blockwise_fp8.mojo:2938-3105,
+// grouped_matmul.mojo:1440-1713 for row scaling; BM = 192): the tiles are those of w4_grouped_head_rows of every slot -- its full
 // BM-row tiles and one more for a rest of more than 128 rows, stored up to the slot's end --
 // numbered through all slots as if they were the row tiles of one matrix: row tile v lies in the slot
 // found by bisection in a prefix table that every block builds in LDS from the device-resident offsets, and its weights
